@@ -1,0 +1,60 @@
+// Shared device helpers for the gfx950 kernels: bfloat16 storage, wave and block
+// reductions with a fixed order, error reporting of the C entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define TQK_WAVE 64
+#define TQK_PAGE 64
+
+// ---- storage types ----------------------------------------------------------
+// bfloat16 is kept as its 16 bits; every computation is in float.
+struct bf16_t { uint16_t bits; };
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);   // NaN stays NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                                               // round to nearest even
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { bf16_t r; r.bits = float_to_bf16_bits(v); return r; }
+
+// ---- reductions ---------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, TQK_WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, TQK_WAVE));
+    return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.  `scratch`
+// holds one float per wave.  The order of additions is fixed by the block shape.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x & (TQK_WAVE - 1), wave = threadIdx.x / TQK_WAVE;
+    const int n_waves = (blockDim.x + TQK_WAVE - 1) / TQK_WAVE;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < n_waves; ++w) total += scratch[w];
+    return total;
+}
+
+// ---- host side ------------------------------------------------------------------
+enum { TQK_F32 = 0, TQK_BF16 = 1 };
+
+int tqk_fail(const char* fmt, ...);           // records the message, returns -1
+int tqk_check_launch(const char* what);       // 0, or -1 with the HIP error recorded
+
+#define TQK_REQUIRE(cond, ...) do { if (!(cond)) return tqk_fail(__VA_ARGS__); } while (0)

@@ -1,0 +1,198 @@
+// Embedding gather, residual add + RMSNorm, bias + rotation + cache write, SwiGLU.
+// Memory-bound kernels; all arithmetic in float32.
+#include "common.h"
+#include "tq_kernels.h"
+
+// ---- embedding ------------------------------------------------------------------
+// The reference looks rows up with candle's embedding op (src/models/turbo_generic.rs:1958).
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
+                             int hidden, int vocab, float* __restrict__ out) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    float* o = out + (size_t)t * hidden;
+    if (id < 0 || id >= vocab) {
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = 0.f;
+        return;
+    }
+    const T* row = table + (size_t)id * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_float(row[i]);
+}
+
+extern "C" int tqk_embed(const void* table, int table_dtype, const int32_t* ids, int n_tokens,
+                         int hidden, int vocab, float* out, void* stream) {
+    TQK_REQUIRE(table && ids && out, "tqk_embed: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "tqk_embed: bad sizes tokens=%d hidden=%d vocab=%d", n_tokens, hidden, vocab);
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (table_dtype == TQK_F32)
+        embed_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)table, ids, hidden, vocab, out);
+    else if (table_dtype == TQK_BF16)
+        embed_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)table, ids, hidden, vocab, out);
+    else
+        return tqk_fail("tqk_embed: unknown dtype %d", table_dtype);
+    return tqk_check_launch("tqk_embed");
+}
+
+// ---- residual add + RMSNorm -----------------------------------------------------
+// y = x / sqrt(mean(x^2) + eps) * w in float32, cast last, as
+// src/models/turbo_generic.rs:41-51 does (division by the root, weight inside).
+template <typename TA, typename TW>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__ delta,
+                                   const TW* __restrict__ weight, float eps,
+                                   const int32_t* __restrict__ rows, int hidden,
+                                   TA* __restrict__ out, int write_back) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t row = rows ? (size_t)rows[r] : (size_t)r;
+    float* hr = h ? h + row * hidden : nullptr;
+    const TA* dr = delta ? delta + row * hidden : nullptr;
+    TA* o = out + (size_t)r * hidden;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = (hr ? hr[i] : 0.f) + (dr ? to_float(dr[i]) : 0.f);
+        if (write_back) hr[i] = v;
+        ss += v * v;
+    }
+    const float total = block_sum(ss, scratch);
+    const float rms = sqrtf(total / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        // the same thread wrote h[i] above, so with write_back the value is read back exactly
+        float v = write_back ? hr[i] : ((hr ? hr[i] : 0.f) + (dr ? to_float(dr[i]) : 0.f));
+        o[i] = from_float<TA>((v / rms) * to_float(weight[i]));
+    }
+}
+
+extern "C" int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const void* weight,
+                               int weight_dtype, float eps, const int32_t* rows, int n_rows,
+                               int hidden, void* out, int write_back, void* stream) {
+    TQK_REQUIRE(weight && out, "tqk_add_rmsnorm: null pointer");
+    TQK_REQUIRE(h || delta, "tqk_add_rmsnorm: neither h nor delta given");
+    TQK_REQUIRE(!write_back || (h && !rows), "tqk_add_rmsnorm: write_back needs h and no row list");
+    TQK_REQUIRE(n_rows >= 0 && hidden > 0, "tqk_add_rmsnorm: bad sizes rows=%d hidden=%d", n_rows, hidden);
+    if (n_rows == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = hidden >= 2048 ? 512 : 256;
+#define LAUNCH(TA, TW) add_rmsnorm_kernel<TA, TW><<<n_rows, threads, 0, s>>>( \
+        h, (const TA*)delta, (const TW*)weight, eps, rows, hidden, (TA*)out, write_back)
+    if (act_dtype == TQK_F32 && weight_dtype == TQK_F32) LAUNCH(float, float);
+    else if (act_dtype == TQK_F32 && weight_dtype == TQK_BF16) LAUNCH(float, bf16_t);
+    else if (act_dtype == TQK_BF16 && weight_dtype == TQK_F32) LAUNCH(bf16_t, float);
+    else if (act_dtype == TQK_BF16 && weight_dtype == TQK_BF16) LAUNCH(bf16_t, bf16_t);
+    else return tqk_fail("tqk_add_rmsnorm: unknown dtypes act=%d weight=%d", act_dtype, weight_dtype);
+#undef LAUNCH
+    return tqk_check_launch("tqk_add_rmsnorm");
+}
+
+// ---- bias + rotation + cache write ------------------------------------------------
+// Rotation as src/models/turbo_generic.rs:417-427 (halves) and :430-443 (pairs), angle
+// tables as :1654-1670, applied after the bias (:805-813, :832-833); the cache holds
+// rotated keys.  A block handles one head of one token; a thread computes one element
+// and reads the partner it rotates with.
+template <typename TA, typename TB>
+__global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restrict__ bias,
+                                  const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+                                  int rot_dim, int style, int max_positions,
+                                  const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                                  const int32_t* __restrict__ page_table, int table_width,
+                                  TA* __restrict__ keys, TA* __restrict__ values,
+                                  TA* __restrict__ q_out, int n_heads, int n_kv_heads, int head_dim,
+                                  int write_kv) {
+    const int t = blockIdx.x;
+    const int head = blockIdx.y;                       // 0..nh-1 q, then nkv k heads, then nkv v heads
+    const int total = (n_heads + 2 * n_kv_heads) * head_dim;
+    const int pos = tok_pos[t];
+    const int kind = head < n_heads ? 0 : (head < n_heads + n_kv_heads ? 1 : 2);
+    if (kind != 0 && !write_kv) return;
+    const TA* src = qkv + (size_t)t * total + (size_t)head * head_dim;
+    const TB* b = bias ? bias + (size_t)head * head_dim : nullptr;
+
+    TA* dst;
+    if (kind == 0) {
+        dst = q_out + ((size_t)t * n_heads + head) * head_dim;
+    } else {
+        const int kvh = kind == 1 ? head - n_heads : head - n_heads - n_kv_heads;
+        const int page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+        if (page < 0) return;                          // the host never lets this happen
+        TA* base = kind == 1 ? keys : values;
+        dst = base + (((size_t)page * n_kv_heads + kvh) * TQK_PAGE + (pos % TQK_PAGE)) * head_dim;
+    }
+
+    const int half_rot = rot_dim / 2;
+    const bool rotate = style != 0 && kind != 2 && pos < max_positions;
+    for (int i = threadIdx.x; i < head_dim; i += blockDim.x) {
+        float x = to_float(src[i]) + (b ? to_float(b[i]) : 0.f);
+        if (rotate && i < rot_dim) {
+            // `first`: this element is x0 of its pair, else x1; p is the pair's table column
+            int p, partner; bool first;
+            if (style == 1) { first = i < half_rot; p = first ? i : i - half_rot; partner = first ? i + half_rot : i - half_rot; }
+            else { first = (i & 1) == 0; p = i >> 1; partner = i ^ 1; }
+            const float y = to_float(src[partner]) + (b ? to_float(b[partner]) : 0.f);
+            const float c = cos_table[(size_t)pos * half_rot + p];
+            const float s = sin_table[(size_t)pos * half_rot + p];
+            x = first ? x * c - y * s : y * s + x * c;
+        }
+        dst[i] = from_float<TA>(x);
+    }
+}
+
+extern "C" int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, int bias_dtype,
+                              const float* cos_table, const float* sin_table, int rot_dim, int style,
+                              int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
+                              const int32_t* page_table, int table_width, int n_seqs, void* keys, void* values,
+                              int n_pages, void* q_out, int n_tokens, int n_heads, int n_kv_heads,
+                              int head_dim, int write_kv, void* stream) {
+    TQK_REQUIRE(qkv && tok_pos && q_out, "tqk_rope_store: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0, "tqk_rope_store: bad sizes");
+    TQK_REQUIRE(style >= 0 && style <= 2, "tqk_rope_store: unknown rotation style %d", style);
+    if (style != 0) {
+        TQK_REQUIRE(cos_table && sin_table, "tqk_rope_store: rotation without tables");
+        TQK_REQUIRE(rot_dim > 0 && rot_dim % 2 == 0 && rot_dim <= head_dim, "tqk_rope_store: rot_dim %d must be even and <= head_dim %d", rot_dim, head_dim);
+        TQK_REQUIRE(max_positions > 0, "tqk_rope_store: empty angle table");
+    } else {
+        rot_dim = 0;
+    }
+    if (write_kv) {
+        TQK_REQUIRE(keys && values && tok_seq && page_table, "tqk_rope_store: cache write without cache pointers");
+        TQK_REQUIRE(table_width > 0 && n_pages > 0 && n_seqs > 0, "tqk_rope_store: empty page table");
+    }
+    if (n_tokens == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid(n_tokens, n_heads + 2 * n_kv_heads);
+    const int threads = 64;
+#define LAUNCH(TA, TB) rope_store_kernel<TA, TB><<<grid, threads, 0, s>>>( \
+        (const TA*)qkv, (const TB*)bias, cos_table, sin_table, rot_dim, style, max_positions, tok_seq, tok_pos, \
+        page_table, table_width, (TA*)keys, (TA*)values, (TA*)q_out, n_heads, n_kv_heads, head_dim, write_kv)
+    if (act_dtype == TQK_F32 && bias_dtype == TQK_F32) LAUNCH(float, float);
+    else if (act_dtype == TQK_F32 && bias_dtype == TQK_BF16) LAUNCH(float, bf16_t);
+    else if (act_dtype == TQK_BF16 && bias_dtype == TQK_F32) LAUNCH(bf16_t, float);
+    else if (act_dtype == TQK_BF16 && bias_dtype == TQK_BF16) LAUNCH(bf16_t, bf16_t);
+    else return tqk_fail("tqk_rope_store: unknown dtypes act=%d bias=%d", act_dtype, bias_dtype);
+#undef LAUNCH
+    return tqk_check_launch("tqk_rope_store");
+}
+
+// ---- SwiGLU ----------------------------------------------------------------------
+// silu(gate) * up, src/models/turbo_generic.rs:105-111 and :64-66.
+template <typename TA>
+__global__ void swiglu_kernel(const TA* __restrict__ gate_up, TA* __restrict__ out, int inter, size_t total) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t t = i / inter, c = i % inter;
+    const float g = to_float(gate_up[t * 2 * inter + c]);
+    const float u = to_float(gate_up[t * 2 * inter + inter + c]);
+    out[i] = from_float<TA>((g / (1.f + expf(-g))) * u);
+}
+
+extern "C" int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, void* stream) {
+    TQK_REQUIRE(gate_up && out, "tqk_swiglu: null pointer");
+    TQK_REQUIRE(n_tokens >= 0 && inter > 0, "tqk_swiglu: bad sizes");
+    if (n_tokens == 0) return 0;
+    const size_t total = (size_t)n_tokens * inter;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    hipStream_t s = (hipStream_t)stream;
+    if (act_dtype == TQK_F32) swiglu_kernel<float><<<blocks, 256, 0, s>>>((const float*)gate_up, (float*)out, inter, total);
+    else if (act_dtype == TQK_BF16) swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, total);
+    else return tqk_fail("tqk_swiglu: unknown dtype %d", act_dtype);
+    return tqk_check_launch("tqk_swiglu");
+}

@@ -1,0 +1,86 @@
+/* C entry points of the gfx950 kernel library.
+ *
+ * In the manner of the reference's C boundary (tq-kv/include/tq_kv.h:27-84): plain
+ * C types, int32 status (0 ok, -1 error), a message for the last error.  Pointers
+ * are device pointers unless said otherwise; `stream` is a hipStream_t.  Every
+ * entry point checks its sizes on the host and refuses what its kernel does not
+ * handle; none allocates.
+ *
+ * dtype codes: 0 = float32, 1 = bfloat16.
+ */
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* tqk_last_error(void);
+int tqk_abi_version(void);
+
+/* out[t, :] = float(table[ids[t], :]); ids outside [0, vocab) give zeros. */
+int tqk_embed(const void* table, int table_dtype, const int32_t* ids, int n_tokens,
+              int hidden, int vocab, float* out, void* stream);
+
+/* Row r (row index rows[r], or r if rows is NULL):
+ *   v = (h ? h[row] : 0) + (delta ? delta[row] : 0);  if write_back: h[row] = v;
+ *   out[r] = v / sqrt(mean(v^2) + eps) * weight          (all in float32)
+ * delta and out have dtype act_dtype. */
+int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const void* weight,
+                    int weight_dtype, float eps, const int32_t* rows, int n_rows,
+                    int hidden, void* out, int write_back, void* stream);
+
+/* y[M,N] = x[M,K] w[N,K]^T (+ bias[N]); float32 accumulation in a fixed order that
+ * does not depend on M.  Any sizes. */
+int tqk_gemm(const void* x, int x_dtype, const void* w, int w_dtype, const void* bias,
+             int bias_dtype, void* y, int y_dtype, int M, int N, int K, void* stream);
+
+/* Skinny product for few rows: y[M,N] = x[M,K] w[N,K]^T, bfloat16 in, MFMA, float32
+ * accumulation; epilogue 0: store y (y_dtype), 1: w holds gate rows then up rows
+ * (N = 2*inter), y[M,inter] = silu(gate)*up (bfloat16).  K must be a multiple of 32. */
+int tqk_skinny_bf16(const void* x, const void* w, void* y, int y_dtype, int M, int N, int K,
+                    int epilogue, void* stream);
+
+/* For each token t and head: add bias, rotate q and k heads by the angle table row
+ * tok_pos[t] (style 0: none, 1: halves (j, j+rot/2), 2: pairs (2j, 2j+1)), write q to
+ * q_out [tokens, heads, head_dim] and, if write_kv, k and v into the pages of the
+ * token's sequence: keys/values [n_pages, kv_heads, 64, head_dim]. */
+int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, int bias_dtype,
+                   const float* cos_table, const float* sin_table, int rot_dim, int style,
+                   int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
+                   const int32_t* page_table, int table_width, int n_seqs, void* keys, void* values,
+                   int n_pages, void* q_out, int n_tokens, int n_heads, int n_kv_heads,
+                   int head_dim, int write_kv, void* stream);
+
+/* Softmax attention of each token's query over its sequence's cached positions
+ * lo..tok_pos[t], lo = max(0, tok_pos - window + 1) if window > 0 else 0.  One wave
+ * per (token, head); float32 throughout; out [tokens, heads*head_dim]. */
+int tqk_attention(const void* q, const void* keys, const void* values, int act_dtype,
+                  const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* page_table,
+                  int table_width, int n_seqs, int n_pages, int window, float scale, void* out,
+                  int n_tokens, int n_heads, int n_kv_heads, int head_dim, void* stream);
+
+/* out[t, i] = silu(gate_up[t, i]) * gate_up[t, inter + i] */
+int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, void* stream);
+
+/* out[r] = lowest index of the largest value of logits[r, :] */
+int tqk_argmax(const float* logits, int n_rows, int vocab, int32_t* out, void* stream);
+
+/* For every generated token of the row's request, once per occurrence:
+ * l > 0 ? l / penalty : l * penalty.  hist [n_req, hist_cap], hist_len [n_req]. */
+int tqk_repeat_penalty(float* logits, int n_rows, int vocab, const int32_t* row_req,
+                       const int32_t* hist, int hist_cap, const int32_t* hist_len, int n_req,
+                       float penalty, void* stream);
+
+/* hist[row_req[r], hist_len[..]++] = tokens[r] */
+int tqk_append_history(const int32_t* tokens, const int32_t* row_req, int32_t* hist, int hist_cap,
+                       int32_t* hist_len, int n_rows, void* stream);
+
+/* One draw per row from softmax(logits / temperature) cut to top_k (0: off) and top_p
+ * (>= 1: off), by inverse CDF over the kept tokens in order of id with uniforms[r]. */
+int tqk_sample(const float* logits, int n_rows, int vocab, float temperature, int top_k, float top_p,
+               const float* uniforms, int32_t* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,98 @@
+"""What one step knows about its batch, on the host and on the device.
+
+A step runs the tokens it is given as one packed batch: the tokens of sequence 0,
+then of sequence 1, and so on.  For each token the device knows which sequence of
+the step it belongs to and its absolute position; for each sequence its slot, how
+many positions the cache held before the step and how many tokens it brings; for
+each cache group the page table of the step's sequences.  All of it is built on the
+host as one int32 array and uploaded in one copy.
+"""
+import numpy as np
+import torch
+
+
+class _Arrays:
+    pass
+
+
+class HostStaging:
+    """A pinned host buffer that is reused from step to step; the copy of the step
+    before must have finished before it is written again."""
+
+    def __init__(self, device):
+        self.device = device
+        self.buf = None
+        self.event = None
+
+    def upload(self, packed):
+        n = packed.shape[0]
+        if self.event is not None:
+            self.event.synchronize()
+        if self.buf is None or self.buf.shape[0] < n:
+            self.buf = torch.empty(max(4096, 2 * n), dtype=torch.int32, pin_memory=True)
+        self.buf[:n].numpy()[:] = packed
+        dev = torch.empty(n, dtype=torch.int32, device=self.device)
+        dev.copy_(self.buf[:n], non_blocking=True)
+        self.event = torch.cuda.Event()
+        self.event.record()
+        return dev
+
+
+class StepContext:
+    """items: [(slot, start, tokens)] with `start` the sequence's length before the step;
+    want: for each item the indices among its tokens whose logits are wanted."""
+
+    def __init__(self, items, want, cache, device, staging=None):
+        self.n_seqs = len(items)
+        lens = [len(toks) for _, _, toks in items]
+        self.n_tokens = int(sum(lens))
+        host = _Arrays()
+        host.tokens = np.concatenate([np.asarray(toks, dtype=np.int64) for _, _, toks in items]).astype(np.int32)
+        host.seq_slot = np.asarray([slot for slot, _, _ in items], dtype=np.int32)
+        host.seq_start = np.asarray([start for _, start, _ in items], dtype=np.int32)
+        host.seq_new = np.asarray(lens, dtype=np.int32)
+        host.cu = np.zeros(self.n_seqs + 1, dtype=np.int32)
+        np.cumsum(host.seq_new, out=host.cu[1:])
+        host.tok_seq = np.repeat(np.arange(self.n_seqs, dtype=np.int32), host.seq_new)
+        host.tok_pos = (np.arange(self.n_tokens, dtype=np.int32) - np.repeat(host.cu[:-1], host.seq_new)
+                        + np.repeat(host.seq_start, host.seq_new)).astype(np.int32)
+        rows = []
+        for i, w in enumerate(want):
+            for j in w:
+                if not 0 <= j < lens[i]:
+                    raise IndexError("wanted place %d is outside the %d tokens of sequence %d" % (j, lens[i], i))
+                rows.append(int(host.cu[i]) + int(j))
+        host.want_rows = np.asarray(rows, dtype=np.int32)
+        self.host = host
+        self.all_decode = all(n == 1 for n in lens)
+        self.max_new = max(lens)
+        self.max_end = int((host.seq_start + host.seq_new).max())
+        self.groups = list(cache.kv_groups) if cache is not None else []
+        slots = [slot for slot, _, _ in items]
+        self.host_tables = [cache.page_table(g, slots) for g in self.groups]
+
+        names = ["tokens", "tok_seq", "tok_pos", "seq_slot", "seq_start", "seq_new", "cu", "want_rows"]
+        parts = [getattr(host, n) for n in names] + [t.reshape(-1) for t in self.host_tables]
+        offsets, total = [], 0
+        for p in parts:
+            offsets.append(total)
+            total += (p.shape[0] + 3) // 4 * 4
+        packed = np.zeros(max(total, 4), dtype=np.int32)
+        for off, p in zip(offsets, parts):
+            packed[off:off + p.shape[0]] = p
+        if staging is not None:
+            flat = staging.upload(packed)
+        else:
+            flat = torch.from_numpy(packed).to(device)
+        self.flat = flat
+        dev = _Arrays()
+        for name, off, p in zip(names, offsets, parts):
+            setattr(dev, name, flat[off:off + p.shape[0]])
+        self.dev = dev
+        self._tables = {}
+        for g, off, t in zip(self.groups, offsets[len(names):], self.host_tables):
+            self._tables[id(g)] = flat[off:off + t.size].view(t.shape)
+
+    def page_table(self, group):
+        """[sequences of the step, width] int32 page ids of a cache group, on the device."""
+        return self._tables[id(group)]

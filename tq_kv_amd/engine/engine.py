@@ -1,0 +1,70 @@
+"""The engine: a model, its cache, and the one step function everything above uses.
+
+The reference's step is `forward(tokens, index_pos)` for one sequence with the last
+row's logits (src/models/turbo_generic.rs:1950-1987) and its per-request state is one
+position counter (src/engine.rs:117, :322-324).  Here a step takes a batch of
+sequences with unequal numbers of new tokens (whole prompts, or one token each, or
+anything between), runs exactly those tokens against what the cache holds, and
+returns the logits at the wanted places.
+"""
+import torch
+
+from ..cache.store import Cache
+from .context import HostStaging, StepContext
+
+
+class StepError(ValueError):
+    pass
+
+
+class Engine:
+    """model: a loaded Model.  max_tokens: positions live sequences may hold together,
+    each sequence counted up to a multiple of 64.  max_slots: most live sequences."""
+
+    def __init__(self, model, max_tokens, max_slots=256):
+        self.model = model
+        self.max_tokens = int(max_tokens)
+        self.cache = Cache(model.needs, model.cache_of, self.max_tokens, max_slots, model.dtype, model.device)
+        self.staging = HostStaging(model.device) if model.device.type == "cuda" else None
+        self.vocab_size = model.spec.vocab_size
+        self.max_positions = model.spec.max_positions
+
+    # -- sequences --------------------------------------------------------
+    def open(self):
+        """Start a sequence: a slot of the cache with nothing in it."""
+        return self.cache.acquire()
+
+    def close(self, slot):
+        """End a sequence: its slot and pages go back and will be used again."""
+        self.cache.release(slot)
+
+    def length(self, slot):
+        return self.cache.length(slot)
+
+    # -- the step ---------------------------------------------------------
+    def step(self, items):
+        """items: [(slot, tokens, want)].  tokens: the sequence's next tokens (at least one);
+        want: indices among them whose logits are wanted (may be empty).  Returns float32
+        logits [sum of len(want), vocab] in the order of items and of want."""
+        if not items:
+            raise StepError("a step needs at least one sequence")
+        seen = set()
+        for slot, tokens, _ in items:
+            if slot in seen:
+                raise StepError("slot %d appears twice in one step" % slot)
+            seen.add(slot)
+            if len(tokens) == 0:
+                raise StepError("Empty prompt")          # src/engine.rs:347-349
+            lo, hi = min(tokens), max(tokens)
+            if lo < 0 or hi >= self.vocab_size:
+                raise StepError("token id %d is outside the vocabulary of %d" % (lo if lo < 0 else hi, self.vocab_size))
+            if self.cache.length(slot) + len(tokens) > self.max_positions:
+                raise StepError("sequence would reach %d positions, the model has %d"
+                                % (self.cache.length(slot) + len(tokens), self.max_positions))
+        sizes = [(slot, len(tokens)) for slot, tokens, _ in items]
+        self.cache.reserve(sizes)
+        ctx = StepContext([(slot, self.cache.length(slot), tokens) for slot, tokens, _ in items],
+                          [want for _, _, want in items], self.cache, self.model.device, self.staging)
+        logits = self.model.forward(ctx, self.cache)
+        self.cache.commit(sizes)
+        return logits

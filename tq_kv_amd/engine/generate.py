@@ -1,0 +1,106 @@
+"""The generation loop above the step function.
+
+One request in the reference (src/engine.rs:364-438): the prompt whole, a first draw,
+then while fewer than max_tokens tokens have been emitted: stop if the drawn token is
+a stop token (it is not emitted), emit it, feed it, draw the next.  Here many
+requests run as batches that start together: their prompts in one step, then one
+token each per step; a request that ends leaves the batch and gives its slot back at
+once, the others go on unchanged; when a batch is done the next one starts, until
+every request has been served.
+
+The loop only decides; it computes nothing.  It needs of the engine `open()`,
+`close(slot)`, `step(items)`, `max_tokens` and `max_positions`, and of the sampler
+`sample(logits, rows)`, so it can be tested without a GPU.
+"""
+from ..cache.store import PAGE
+from ..sampling.params import GenerationParams
+
+
+class GenerationError(ValueError):
+    pass
+
+
+def _room(prompt_len, max_new):
+    """Cache positions a request may come to hold, counted in whole pages."""
+    longest = prompt_len + max(0, max_new - 1)      # the last emitted token is never fed
+    return (longest + PAGE - 1) // PAGE * PAGE
+
+
+def plan_batches(prompt_lens, max_new, max_tokens, max_batch):
+    """Cut the requests, in order, into batches that fit the cache: at most max_batch
+    requests and at most max_tokens positions (whole pages each).  Returns lists of
+    request indices."""
+    batches, cur, used = [], [], 0
+    for i, n in enumerate(prompt_lens):
+        need = _room(n, max_new)
+        if need > max_tokens:
+            raise GenerationError("request %d needs %d cache positions, the engine has %d" % (i, need, max_tokens))
+        if cur and (len(cur) >= max_batch or used + need > max_tokens):
+            batches.append(cur)
+            cur, used = [], 0
+        cur.append(i)
+        used += need
+    if cur:
+        batches.append(cur)
+    return batches
+
+
+def generate(engine, prompts, params=None, eos_ids=(), on_tokens=None, max_batch=64, make_sampler=None):
+    """prompts: token-id lists.  Returns for each prompt the emitted token ids.
+
+    eos_ids: stop tokens.  on_tokens(pairs): called after every step with the
+    (request index, token) pairs emitted by it.  make_sampler(params, request_ids): the
+    sampler of a batch (default: the device sampler)."""
+    params = params or GenerationParams()
+    eos = set(int(t) for t in eos_ids)
+    prompts = [list(p) for p in prompts]
+    for i, p in enumerate(prompts):
+        if not p:
+            raise GenerationError("Empty prompt" if len(prompts) == 1 else "Empty prompt (request %d)" % i)
+        if len(p) + max(0, params.max_tokens - 1) > engine.max_positions:
+            raise GenerationError("request %d: %d prompt tokens and %d new ones exceed the model's %d positions"
+                                  % (i, len(p), params.max_tokens, engine.max_positions))
+    if make_sampler is None:
+        from ..sampling.sampler import Sampler
+
+        def make_sampler(p, request_ids):
+            return Sampler(p, request_ids, engine.model.device)
+
+    emitted = [[] for _ in prompts]
+    for batch in plan_batches([len(p) for p in prompts], params.max_tokens, engine.max_tokens, max_batch):
+        _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, make_sampler(params, batch))
+    return emitted
+
+
+def _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, sampler):
+    slots = {}
+    try:
+        for r in batch:
+            slots[r] = engine.open()
+        logits = engine.step([(slots[r], prompts[r], [len(prompts[r]) - 1]) for r in batch])
+        live = list(range(len(batch)))                 # indices into `batch`
+        drawn = dict(zip(live, sampler.sample(logits, live)))
+        while live:
+            feed, pairs = [], []
+            for b in live:
+                r = batch[b]
+                tok = drawn[b]
+                if len(emitted[r]) >= params.max_tokens or tok in eos:
+                    engine.close(slots.pop(r))          # stop tokens are not emitted (src/engine.rs:381)
+                    continue
+                emitted[r].append(tok)
+                pairs.append((r, tok))
+                if len(emitted[r]) >= params.max_tokens:
+                    engine.close(slots.pop(r))          # nothing more to draw for it
+                    continue
+                feed.append(b)
+            if on_tokens is not None and pairs:
+                on_tokens(pairs)
+            live = feed
+            if not live:
+                break
+            logits = engine.step([(slots[batch[b]], [drawn[b]], [0]) for b in live])
+            drawn = dict(zip(live, sampler.sample(logits, live)))
+    finally:
+        for slot in slots.values():
+            engine.close(slot)

@@ -1,0 +1,127 @@
+"""A model: parts built from a ModelSpec, weights loaded into them, and the forward
+pass of one step.  It knows nothing of any architecture: embedding, the blocks in
+the order the spec gives, final norm and head on the wanted rows, as the
+reference's forward does for its one sequence (src/models/turbo_generic.rs:1950-1987).
+"""
+import torch
+
+from .. import kernels as K
+from ..config import catalog
+from ..config.base import ConfigError, read_config_json
+from ..config.registry import config_from_dict, spec_for
+from ..parts.linear import linear
+from ..parts.registry import BuildEnv
+from ..parts.spec import TensorSpec
+from ..weights import load_folder, random_tensors, write_model_folder
+
+DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+          torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def run_dtype(name):
+    if name not in DTYPES:
+        raise ValueError("dtype must be bfloat16 or float32, got %r" % (name,))
+    return DTYPES[name]
+
+
+class Model:
+    def __init__(self, spec, dtype="bfloat16", device="cuda", config=None):
+        self.spec = spec
+        self.config = config
+        self.dtype = run_dtype(dtype)
+        self.device = torch.device(device)
+        self.env = BuildEnv(self.device, self.dtype)
+        self.blocks = [self.env.build("block", layer.block) for layer in spec.layers]
+        self.final_norm = self.env.build("norm", spec.final_norm)
+        for i, run in enumerate(spec.order):
+            if not 0 <= run.layer < len(self.blocks):
+                raise ValueError("run %d names layer %d, the model has %d" % (i, run.layer, len(self.blocks)))
+            if run.cache_of is not None and not 0 <= run.cache_of < i:
+                raise ValueError("run %d reads the cache of run %r, which is not an earlier run" % (i, run.cache_of))
+        self.needs = [self.blocks[run.layer].cache_need() for run in spec.order]
+        self.cache_of = [run.cache_of for run in spec.order]
+        self.embedding = None
+        self.head = None
+        self.loaded = False
+
+    # -- tensors ----------------------------------------------------------
+    def tensor_specs(self):
+        """Full tensor name -> TensorSpec of everything the model loads."""
+        s = self.spec
+        out = {s.embedding_name: TensorSpec((s.vocab_size, s.hidden_size))}
+        for layer, block in zip(s.layers, self.blocks):
+            for name, spec in block.tensors().items():
+                out[layer.prefix + name] = spec
+        for name, spec in self.final_norm.tensors().items():
+            out[s.final_norm_prefix + name] = spec
+        if s.head_name is not None:
+            out[s.head_name] = TensorSpec((s.vocab_size, s.hidden_size))
+        return out
+
+    def load(self, tensors):
+        """Give every part its tensors (full names, already on the device)."""
+        s = self.spec
+        self.embedding = tensors[s.embedding_name]
+        for layer, block in zip(s.layers, self.blocks):
+            block.load({name: tensors[layer.prefix + name] for name in block.tensors()})
+        self.final_norm.load({name: tensors[s.final_norm_prefix + name] for name in self.final_norm.tensors()})
+        self.head = self.embedding if s.head_name is None else tensors[s.head_name]
+        self.loaded = True
+        return self
+
+    # -- construction -----------------------------------------------------
+    @classmethod
+    def from_config_dict(cls, raw, dtype="bfloat16", device="cuda"):
+        name, config = config_from_dict(raw)
+        return cls(spec_for(name, config), dtype, device, config=config)
+
+    @classmethod
+    def from_dir(cls, model_dir, dtype="bfloat16", device="cuda"):
+        """A model folder: config.json picks the architecture, *.safetensors hold the weights."""
+        model = cls.from_config_dict(read_config_json(model_dir), dtype, device)
+        return model.load(load_folder(model_dir, model.tensor_specs(), model.dtype, model.device))
+
+    @classmethod
+    def random(cls, shape, seed=0, dtype="bfloat16", device="cuda"):
+        """Random weights made in memory.  shape: a catalog name ("tiny:a", "qwen2.5:7b") or a
+        config.json dictionary.  Weights are drawn on `device`."""
+        raw = shape if isinstance(shape, dict) else catalog.find(shape)
+        if raw is None:
+            raise ConfigError("Model '%s' not found. Available shapes: %s"
+                              % (shape, ", ".join("%s:%s" % e for e in catalog.entries())))
+        model = cls.from_config_dict(raw, dtype, device)
+        store = torch.bfloat16 if model.dtype == torch.bfloat16 else torch.float32
+        return model.load(random_tensors(model.tensor_specs(), seed, store, model.device))
+
+    @staticmethod
+    def write_random_folder(folder, shape, seed=0, store_dtype=torch.bfloat16):
+        """Write config.json and model.safetensors with random weights; returns the folder."""
+        raw = shape if isinstance(shape, dict) else catalog.find(shape)
+        if raw is None:
+            raise ConfigError("Model '%s' not found. Available shapes: %s"
+                              % (shape, ", ".join("%s:%s" % e for e in catalog.entries())))
+        model = Model.from_config_dict(raw, "float32", "cpu")
+        return write_model_folder(folder, raw, model.tensor_specs(), seed, store_dtype)
+
+    # -- one step ---------------------------------------------------------
+    def forward(self, ctx, cache):
+        """Run the step's tokens through every run of the order; logits [wanted rows, vocab]
+        float32 for ctx's wanted rows."""
+        if not self.loaded:
+            raise RuntimeError("the model has no weights yet")
+        s = self.spec
+        h = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.float32, device=self.device)
+        K.embed(self.embedding, ctx.dev.tokens, h)
+        delta = None
+        for i, run in enumerate(s.order):
+            delta = self.blocks[run.layer].forward(h, delta, ctx, cache.entry(i))
+        n_rows = ctx.dev.want_rows.shape[0]
+        if n_rows == 0:
+            return torch.empty((0, s.vocab_size), dtype=torch.float32, device=self.device)
+        x = self.final_norm.gather_add_norm(h, delta, ctx.dev.want_rows)
+        return linear(x, self.head, out_dtype=torch.float32)
+
+    def __repr__(self):
+        s = self.spec
+        return "Model(architecture=%s, layers=%d, runs=%d, hidden=%d, vocab=%d, dtype=%s)" % (
+            s.architecture, len(s.layers), len(s.order), s.hidden_size, s.vocab_size, str(self.dtype).replace("torch.", ""))

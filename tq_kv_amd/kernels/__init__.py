@@ -1,0 +1,222 @@
+"""Python face of the gfx950 kernel library: one function per C entry point.
+
+Every function checks device, dtype, contiguity and shapes on the host before the
+kernel is launched, because a kernel that reads out of bounds can take the whole
+GPU down.  There is no fallback: without the built library, or on tensors that
+are not on the GPU, these functions raise.
+"""
+import ctypes
+
+import torch
+
+from ..csrc import build as _build
+
+_LIB = None
+
+F32, BF16 = 0, 1
+STYLE_NONE, STYLE_HALVES, STYLE_PAIRS = 0, 1, 2
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def library():
+    """The loaded kernel library (built on first use if it is not there)."""
+    global _LIB
+    if _LIB is None:
+        path = _build.ensure_built()
+        try:
+            lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError("cannot load the HIP kernel library %s: %s" % (path, e))
+        lib.tqk_last_error.restype = ctypes.c_char_p
+        lib.tqk_abi_version.restype = ctypes.c_int
+        _LIB = lib
+    return _LIB
+
+
+def library_path():
+    library()
+    return _LIB._name
+
+
+def _check(status, name):
+    if status != 0:
+        raise KernelError("%s: %s" % (name, library().tqk_last_error().decode("utf-8", "replace")))
+
+
+def _code(dtype):
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise KernelError("unsupported dtype %s (float32 and bfloat16 only)" % dtype)
+
+
+def _dev(t, name, dtype=None, shape=None):
+    if not isinstance(t, torch.Tensor):
+        raise KernelError("%s must be a tensor" % name)
+    if t.device.type != "cuda":
+        raise KernelError("%s is on %s: the kernels run on the GPU only" % (name, t.device))
+    if not t.is_contiguous():
+        raise KernelError("%s must be contiguous" % name)
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError("%s must be %s, got %s" % (name, dtype, t.dtype))
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError("%s must have shape %s, got %s" % (name, tuple(shape), tuple(t.shape)))
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _opt(t, name, dtype=None, shape=None):
+    return ctypes.c_void_p(0) if t is None else _dev(t, name, dtype, shape)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def embed(table, ids, out):
+    """out[t] = float32(table[ids[t]]);  table [V,H], ids [T] int32, out [T,H] float32."""
+    vocab, hidden = table.shape
+    n = ids.shape[0]
+    _check(library().tqk_embed(_dev(table, "table"), _code(table.dtype), _dev(ids, "ids", torch.int32, (n,)),
+                               n, hidden, vocab, _dev(out, "out", torch.float32, (n, hidden)), _stream()),
+           "embed")
+    return out
+
+
+def add_rmsnorm(h, delta, weight, eps, out, rows=None, write_back=False):
+    """out = rmsnorm(h + delta) * weight; with write_back h becomes h + delta.
+
+    h: [T,H] float32 or None.  delta: [T,H] of out's dtype or None.  rows: int32 row
+    indices (then out has one row per index) or None for all rows."""
+    hidden = weight.shape[0]
+    n_rows = out.shape[0]
+    src_rows = (h if h is not None else delta).shape[0]
+    if rows is None and src_rows != n_rows:
+        raise KernelError("add_rmsnorm: %d input rows but %d output rows" % (src_rows, n_rows))
+    _check(library().tqk_add_rmsnorm(
+        _opt(h, "h", torch.float32, (src_rows, hidden)), _opt(delta, "delta", out.dtype, (src_rows, hidden)),
+        _code(out.dtype), _dev(weight, "weight", None, (hidden,)), _code(weight.dtype), ctypes.c_float(eps),
+        _opt(rows, "rows", torch.int32, (n_rows,)), n_rows, hidden, _dev(out, "out", None, (n_rows, hidden)),
+        1 if write_back else 0, _stream()), "add_rmsnorm")
+    return out
+
+
+def gemm(x, w, bias, out):
+    """out[M,N] = x[M,K] w[N,K]^T (+ bias[N]), float32 accumulation, any dtype mix."""
+    m, k = x.shape
+    n = w.shape[0]
+    _check(library().tqk_gemm(
+        _dev(x, "x", None, (m, k)), _code(x.dtype), _dev(w, "w", None, (n, k)), _code(w.dtype),
+        _opt(bias, "bias", None, (n,)), _code(bias.dtype) if bias is not None else 0,
+        _dev(out, "out", None, (m, n)), _code(out.dtype), m, n, k, _stream()), "gemm")
+    return out
+
+
+def rope_store(qkv, bias, cos, sin, rot_dim, style, tok_seq, tok_pos, page_table, keys, values, q_out,
+               n_heads, n_kv_heads, head_dim, write_kv=True):
+    """Bias, rotation of q and k, q to q_out, k and v into the cache pages."""
+    n = qkv.shape[0]
+    total = (n_heads + 2 * n_kv_heads) * head_dim
+    max_pos = 0
+    if style != STYLE_NONE:
+        max_pos = cos.shape[0]
+        _dev(cos, "cos", torch.float32, (max_pos, rot_dim // 2))
+        _dev(sin, "sin", torch.float32, (max_pos, rot_dim // 2))
+    n_seqs, width, n_pages = 0, 0, 0
+    if write_kv:
+        n_seqs, width = page_table.shape
+        n_pages = keys.shape[0]
+        shape = (n_pages, n_kv_heads, 64, head_dim)
+        _dev(keys, "keys", qkv.dtype, shape)
+        _dev(values, "values", qkv.dtype, shape)
+    _check(library().tqk_rope_store(
+        _dev(qkv, "qkv", None, (n, total)), _code(qkv.dtype), _opt(bias, "bias", None, (total,)),
+        _code(bias.dtype) if bias is not None else 0,
+        _opt(cos if style != STYLE_NONE else None, "cos"), _opt(sin if style != STYLE_NONE else None, "sin"),
+        rot_dim, style, max_pos, _opt(tok_seq, "tok_seq", torch.int32, (n,)), _dev(tok_pos, "tok_pos", torch.int32, (n,)),
+        _opt(page_table if write_kv else None, "page_table", torch.int32), width, n_seqs,
+        _opt(keys if write_kv else None, "keys"), _opt(values if write_kv else None, "values"), n_pages,
+        _dev(q_out, "q_out", qkv.dtype, (n, n_heads, head_dim)), n, n_heads, n_kv_heads, head_dim,
+        1 if write_kv else 0, _stream()), "rope_store")
+    return q_out
+
+
+def attention(q, keys, values, tok_seq, tok_pos, page_table, window, scale, out):
+    """Generic softmax attention of q [T,heads,d] over the paged cache; out [T, heads*d]."""
+    n, n_heads, head_dim = q.shape
+    n_pages, n_kv_heads = keys.shape[0], keys.shape[1]
+    n_seqs, width = page_table.shape
+    shape = (n_pages, n_kv_heads, 64, head_dim)
+    _check(library().tqk_attention(
+        _dev(q, "q"), _dev(keys, "keys", q.dtype, shape), _dev(values, "values", q.dtype, shape), _code(q.dtype),
+        _dev(tok_seq, "tok_seq", torch.int32, (n,)), _dev(tok_pos, "tok_pos", torch.int32, (n,)),
+        _dev(page_table, "page_table", torch.int32), width, n_seqs, n_pages, int(window or 0), ctypes.c_float(scale),
+        _dev(out, "out", q.dtype, (n, n_heads * head_dim)), n, n_heads, n_kv_heads, head_dim, _stream()), "attention")
+    return out
+
+
+def swiglu(gate_up, out):
+    """out[t,i] = silu(gate_up[t,i]) * gate_up[t,I+i]"""
+    n, inter = out.shape
+    _check(library().tqk_swiglu(_dev(gate_up, "gate_up", out.dtype, (n, 2 * inter)), _dev(out, "out"),
+                                _code(out.dtype), n, inter, _stream()), "swiglu")
+    return out
+
+
+def argmax(logits, out):
+    """out[r] = lowest index of the largest value of row r; logits [R,V] float32, out [R] int32."""
+    rows, vocab = logits.shape
+    _check(library().tqk_argmax(_dev(logits, "logits", torch.float32), rows, vocab,
+                                _dev(out, "out", torch.int32, (rows,)), _stream()), "argmax")
+    return out
+
+
+def has_skinny():
+    """Whether the library holds the MFMA kernel for products with few rows."""
+    return hasattr(library(), "tqk_skinny_bf16")
+
+
+def skinny_bf16(x, w, out, swiglu=False):
+    """out[M,N] = x[M,K] w[N,K]^T for few rows, bfloat16 in; with swiglu, w holds gate rows
+    then up rows and out[M, N/2] = silu(gate) * up."""
+    m, k = x.shape
+    n = w.shape[0]
+    n_out = n // 2 if swiglu else n
+    _check(library().tqk_skinny_bf16(
+        _dev(x, "x", torch.bfloat16, (m, k)), _dev(w, "w", torch.bfloat16, (n, k)),
+        _dev(out, "out", None, (m, n_out)), _code(out.dtype), m, n, k, 1 if swiglu else 0, _stream()), "skinny_bf16")
+    return out
+
+
+def repeat_penalty(logits, row_req, hist, hist_len, penalty):
+    """In place: for every token in the history of the row's request, once per occurrence,
+    l > 0 ? l / penalty : l * penalty."""
+    rows, vocab = logits.shape
+    n_req, cap = hist.shape
+    _check(library().tqk_repeat_penalty(
+        _dev(logits, "logits", torch.float32), rows, vocab, _dev(row_req, "row_req", torch.int32, (rows,)),
+        _dev(hist, "hist", torch.int32), cap, _dev(hist_len, "hist_len", torch.int32, (n_req,)), n_req,
+        ctypes.c_float(penalty), _stream()), "repeat_penalty")
+    return logits
+
+
+def append_history(tokens, row_req, hist, hist_len):
+    rows = tokens.shape[0]
+    n_req, cap = hist.shape
+    _check(library().tqk_append_history(
+        _dev(tokens, "tokens", torch.int32, (rows,)), _dev(row_req, "row_req", torch.int32, (rows,)),
+        _dev(hist, "hist", torch.int32), cap, _dev(hist_len, "hist_len", torch.int32, (n_req,)), rows, _stream()),
+        "append_history")
+
+
+def sample(logits, temperature, top_k, top_p, uniforms, out):
+    """One draw per row of logits [R,V] float32 with the uniforms [R] float32; out [R] int32."""
+    rows, vocab = logits.shape
+    _check(library().tqk_sample(
+        _dev(logits, "logits", torch.float32), rows, vocab, ctypes.c_float(temperature), int(top_k),
+        ctypes.c_float(top_p), _dev(uniforms, "uniforms", torch.float32, (rows,)),
+        _dev(out, "out", torch.int32, (rows,)), _stream()), "sample")
+    return out

@@ -1,0 +1,98 @@
+"""The attention mixer: grouped-query softmax attention over the cache.
+
+Order of work as in the reference (src/models/turbo_generic.rs:770-833, 1604-1635):
+q, k, v projections (+ bias), head split, position encoding of q and k, keys and
+values into the cache, scores q.k/sqrt(d), mask, softmax, p.v, merge heads, output
+projection without bias.  Query head h reads kv head h // (heads // kv_heads)
+(:195-204).  The three projections are one product with the weights stacked.
+"""
+import math
+
+import torch
+
+from .. import kernels as K
+from .linear import linear
+from .registry import Part, register
+from .spec import KVNeed, TensorSpec
+
+
+@register("mixer", "attention")
+class Attention(Part):
+    """params: hidden, n_heads, n_kv_heads, head_dim, qkv_bias (bool), out_bias (bool),
+    window (None or positions a query sees, itself included), scale (None: 1/sqrt(head_dim)),
+    position (PartSpec)."""
+
+    def __init__(self, params, env):
+        self.env = env
+        self.hidden = int(params["hidden"])
+        self.n_heads = int(params["n_heads"])
+        self.n_kv_heads = int(params["n_kv_heads"])
+        self.head_dim = int(params["head_dim"])
+        self.qkv_bias = bool(params.get("qkv_bias", False))
+        self.out_bias = bool(params.get("out_bias", False))
+        self.window = params.get("window")
+        if self.n_heads % self.n_kv_heads:
+            raise ValueError("attention: %d heads are not a multiple of %d kv heads" % (self.n_heads, self.n_kv_heads))
+        if self.window is not None and self.window < 1:
+            raise ValueError("attention: window must be at least 1, got %r" % (self.window,))
+        scale = params.get("scale")
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        spec = params["position"]
+        key = ("position", spec.kind, tuple(sorted(spec.params.items())))
+        if key not in env.shared:
+            env.shared[key] = env.build("position", spec)
+        self.position = env.shared[key]
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+
+    def tensors(self):
+        q, kv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
+        t = {"q_proj.weight": TensorSpec((q, self.hidden)), "k_proj.weight": TensorSpec((kv, self.hidden)),
+             "v_proj.weight": TensorSpec((kv, self.hidden)), "o_proj.weight": TensorSpec((self.hidden, q))}
+        if self.qkv_bias:
+            t.update({"q_proj.bias": TensorSpec((q,)), "k_proj.bias": TensorSpec((kv,)), "v_proj.bias": TensorSpec((kv,))})
+        if self.out_bias:
+            t["o_proj.bias"] = TensorSpec((self.hidden,))
+        return t
+
+    def load(self, tensors):
+        ws = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
+        dtype = torch.float32 if any(w.dtype == torch.float32 for w in ws) else ws[0].dtype
+        self.w_qkv = torch.cat([w.to(dtype) for w in ws], dim=0).contiguous()
+        if self.qkv_bias:
+            bs = [tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]]
+            bdtype = torch.float32 if any(b.dtype == torch.float32 for b in bs) else bs[0].dtype
+            self.b_qkv = torch.cat([b.to(bdtype) for b in bs], dim=0).contiguous()
+        self.w_o = tensors["o_proj.weight"]
+        self.b_o = tensors.get("o_proj.bias")
+
+    def cache_need(self):
+        return KVNeed(self.n_kv_heads, self.head_dim, self.window)
+
+    def forward(self, x, ctx, entry):
+        n = x.shape[0]
+        qkv = linear(x, self.w_qkv)
+        table = ctx.page_table(entry.group)
+        q = torch.empty((n, self.n_heads, self.head_dim), dtype=x.dtype, device=x.device)
+        if hasattr(self.position, "apply"):
+            # a position encoding of its own: bias first, then it changes q and k in place
+            if self.b_qkv is not None:
+                qkv += self.b_qkv.to(qkv.dtype)
+            qd, kd = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
+            self.position.apply(qkv[:, :qd].unflatten(1, (self.n_heads, self.head_dim)),
+                                qkv[:, qd:qd + kd].unflatten(1, (self.n_kv_heads, self.head_dim)), ctx)
+            cos = sin = bias = None
+            rot_dim, style = 0, K.STYLE_NONE
+        else:
+            cos, sin, rot_dim, style = self.position.tables()
+            bias = self.b_qkv
+        K.rope_store(qkv, bias, cos, sin, rot_dim, style, ctx.dev.tok_seq, ctx.dev.tok_pos, table,
+                     entry.keys, entry.values, q, self.n_heads, self.n_kv_heads, self.head_dim,
+                     write_kv=entry.writes)
+        y = torch.empty((n, self.n_heads * self.head_dim), dtype=x.dtype, device=x.device)
+        attend(q, entry, table, ctx, self.window, self.scale, y)
+        return linear(y, self.w_o, self.b_o)
+
+
+def attend(q, entry, table, ctx, window, scale, out):
+    """Softmax attention of q over the cache entry: picks the kernel for the step."""
+    return K.attention(q, entry.keys, entry.values, ctx.dev.tok_seq, ctx.dev.tok_pos, table, window, scale, out)

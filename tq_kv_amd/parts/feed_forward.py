@@ -1,0 +1,36 @@
+"""Feed-forward parts.  Gated SiLU ("SwiGLU") as the reference's Mlp
+(src/models/turbo_generic.rs:98-111): down(silu(gate(x)) * up(x)), no biases.  Gate and
+up are one product with the weights stacked."""
+import torch
+
+from .. import kernels as K
+from .linear import linear
+from .registry import Part, register
+from .spec import TensorSpec
+
+
+@register("feed_forward", "gated_silu")
+class GatedSiLU(Part):
+    """params: hidden, inter."""
+
+    def __init__(self, params, env):
+        self.hidden = int(params["hidden"])
+        self.inter = int(params["inter"])
+        self.w_gate_up = self.w_down = None
+
+    def tensors(self):
+        return {"gate_proj.weight": TensorSpec((self.inter, self.hidden)),
+                "up_proj.weight": TensorSpec((self.inter, self.hidden)),
+                "down_proj.weight": TensorSpec((self.hidden, self.inter))}
+
+    def load(self, tensors):
+        ws = [tensors["gate_proj.weight"], tensors["up_proj.weight"]]
+        dtype = torch.float32 if any(w.dtype == torch.float32 for w in ws) else ws[0].dtype
+        self.w_gate_up = torch.cat([w.to(dtype) for w in ws], dim=0).contiguous()
+        self.w_down = tensors["down_proj.weight"]
+
+    def forward(self, x, ctx):
+        gate_up = linear(x, self.w_gate_up)
+        act = torch.empty((x.shape[0], self.inter), dtype=x.dtype, device=x.device)
+        K.swiglu(gate_up, act)
+        return linear(act, self.w_down)

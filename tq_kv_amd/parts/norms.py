@@ -1,0 +1,41 @@
+"""Norms.  RMSNorm as the reference computes it (src/models/turbo_generic.rs:41-51):
+x / sqrt(mean(x^2) + eps) * weight in float32, cast last; the weight is used as it
+is stored (no 1 + w)."""
+import torch
+
+from .. import kernels as K
+from .registry import Part, register
+from .spec import TensorSpec
+
+
+@register("norm", "rms_norm")
+class RMSNorm(Part):
+    """params: size, eps."""
+
+    def __init__(self, params, env):
+        self.size = int(params["size"])
+        self.eps = float(params["eps"])
+        self.env = env
+        self.weight = None
+
+    def tensors(self):
+        return {"weight": TensorSpec((self.size,), init="one_plus_normal")}
+
+    def load(self, tensors):
+        self.weight = tensors["weight"]
+
+    def forward(self, x):
+        """x: [T, size] of the activation dtype -> its norm, same dtype."""
+        out = torch.empty_like(x)
+        return K.add_rmsnorm(None, x, self.weight, self.eps, out)
+
+    def add_norm(self, h, delta):
+        """h: [T, size] float32 residual stream, delta: update of the activation dtype or
+        None.  h += delta in place; returns norm(h) in the activation dtype."""
+        out = torch.empty(h.shape, dtype=self.env.act_dtype, device=h.device)
+        return K.add_rmsnorm(h, delta, self.weight, self.eps, out, write_back=delta is not None)
+
+    def gather_add_norm(self, h, delta, rows):
+        """norm(h[rows] + delta[rows]) for the int32 row indices `rows`; h is left as it is."""
+        out = torch.empty((rows.shape[0], self.size), dtype=self.env.act_dtype, device=h.device)
+        return K.add_rmsnorm(h, delta, self.weight, self.eps, out, rows=rows)

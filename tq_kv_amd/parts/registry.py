@@ -1,0 +1,74 @@
+"""The registry of part kinds and the interface each category of part has.
+
+A part is built from a PartSpec (kind + parameters) and a BuildEnv.  It names its
+tensors, takes them when they are loaded, and computes.  No part knows which
+model it is in: sizes and constants come in as parameters only.
+
+Categories and what each must offer beyond `tensors()` and `load()`:
+
+  norm          forward(x) -> y;  add_norm(h, delta) -> y  (h += delta in place, then
+                norm of h);  gather_add_norm(h, delta, rows) -> y for chosen rows only
+  position      the way a mixer turns positions into a change of q and k: either
+                `tables()` (cos, sin, rot_dim, style) for the fused kernel or
+                `apply(q, k, positions)` for a position encoding of its own
+  mixer         cache_need() -> KVNeed | StateNeed | None;
+                forward(x, ctx, cache_entry) -> y, x and y [tokens, hidden]
+  feed_forward  forward(x, ctx) -> y
+  block         the arrangement: forward(h, delta, ctx, cache_entry) -> delta, where h
+                is the float32 residual stream and delta the update not yet added
+"""
+from typing import Callable, Dict
+
+from .spec import PartSpec
+
+CATEGORIES = ("norm", "position", "mixer", "feed_forward", "block")
+_REGISTRY: Dict[str, Dict[str, Callable]] = {c: {} for c in CATEGORIES}
+
+
+def register(category, kind):
+    """Class decorator: make `kind` buildable in `category`."""
+    if category not in _REGISTRY:
+        raise KeyError("unknown part category '%s' (known: %s)" % (category, ", ".join(CATEGORIES)))
+
+    def deco(cls):
+        _REGISTRY[category][kind] = cls
+        cls.category = category
+        cls.kind = kind
+        return cls
+    return deco
+
+
+def known(category):
+    return sorted(_REGISTRY[category])
+
+
+class BuildEnv:
+    """What a part needs to know about the run: device, activation dtype, and a place
+    where parts without weights (position tables) are shared between layers."""
+
+    def __init__(self, device, act_dtype):
+        self.device = device
+        self.act_dtype = act_dtype
+        self.shared = {}
+
+    def build(self, category, spec: PartSpec):
+        kinds = _REGISTRY[category]
+        if spec.kind not in kinds:
+            raise KeyError("unknown %s kind '%s' (known: %s)" % (category, spec.kind, ", ".join(sorted(kinds))))
+        return kinds[spec.kind](dict(spec.params), self)
+
+
+class Part:
+    """Base of every part."""
+    category = None
+    kind = None
+
+    def tensors(self):
+        """name (relative to the part's prefix) -> TensorSpec"""
+        return {}
+
+    def load(self, tensors):
+        """Take the loaded tensors (same names as tensors())."""
+
+    def cache_need(self):
+        return None

@@ -1,0 +1,5 @@
+from .params import GenerationParams
+from .rng import uniform
+from .sampler import Sampler
+
+__all__ = ["GenerationParams", "uniform", "Sampler"]
