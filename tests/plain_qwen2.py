@@ -99,11 +99,12 @@ def attention_core(q, k, v, visible):
     return att @ v
 
 
-def attention(x, w, prefix, cfg, window):
+def attention(x, w, prefix, cfg, window, offset=0):
     """src/models/turbo_generic.rs:770-833 and 1604-1635 for one whole sequence.
 
-    Projections with bias, head split, rotation of q and k at positions 0..T-1,
-    causal (and windowed) softmax attention, merge heads, o_proj without bias.
+    Projections with bias, head split, rotation of q and k at positions
+    offset..offset+T-1 (the reference's index_pos, :749-750), causal (and windowed)
+    softmax attention, merge heads, o_proj without bias.
     """
     t = x.shape[0]
     nh, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
@@ -113,7 +114,8 @@ def attention(x, w, prefix, cfg, window):
     q = q.reshape(t, nh, d).transpose(0, 1)
     k = k.reshape(t, nkv, d).transpose(0, 1)
     v = v.reshape(t, nkv, d).transpose(0, 1)
-    cos, sin = rope_tables(d, cfg["rope_theta"], t)
+    cos, sin = rope_tables(d, cfg["rope_theta"], offset + t)
+    cos, sin = cos[offset:], sin[offset:]
     q = rope_half(q, cos, sin)
     k = rope_half(k, cos, sin)
     y = attention_core(q, k, v, visibility(t, window))
@@ -141,28 +143,29 @@ def layer_window(cfg, layer):
     return None
 
 
-def decoder_layer(x, w, layer, cfg):
+def decoder_layer(x, w, layer, cfg, offset=0):
     """src/models/turbo_generic.rs:1959-1981.  x + attn(norm(x)); x + mlp(norm(x))."""
     p = "model.layers.%d." % layer
     eps = cfg["rms_norm_eps"]
     h = rms_norm(x, w[p + "input_layernorm.weight"], eps)
-    x = x + attention(h, w, p + "self_attn.", cfg, layer_window(cfg, layer))
+    x = x + attention(h, w, p + "self_attn.", cfg, layer_window(cfg, layer), offset)
     h = rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
     return x + swiglu_mlp(h, w, p + "mlp.")
 
 
-def forward(weights, cfg, tokens):
+def forward(weights, cfg, tokens, offset=0):
     """src/models/turbo_generic.rs:1950-1987 for one sequence, but the logits of every
     position are returned ([T, V]) instead of the last row only.
 
     weights: name -> tensor (any float dtype; read as f32).  cfg: dict of config.json
-    keys.  Tied embeddings: lm_head is the embedding matrix (:2079-2084).
+    keys.  Tied embeddings: lm_head is the embedding matrix (:2079-2084).  offset: the
+    position of the first token (0 in every real use; tests shift it).
     """
     w = {k: v.to(torch.float32) for k, v in weights.items()}
     ids = torch.as_tensor(tokens, dtype=torch.long)
     x = w["model.embed_tokens.weight"][ids]
     for layer in range(cfg["num_hidden_layers"]):
-        x = decoder_layer(x, w, layer, cfg)
+        x = decoder_layer(x, w, layer, cfg, offset)
     x = rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return linear(x, head)
@@ -202,4 +205,82 @@ def generate_greedy(weights, cfg, prompt, max_tokens, eos_ids=()):
         emitted.append(nxt)
         tokens.append(nxt)
         nxt = greedy(forward(weights, cfg, tokens)[-1])
+    return emitted
+
+
+def keep_top_k_top_p(z, top_k, top_p):
+    """Which tokens stay after "top-k then top-p" (src/engine.rs:356-360 names the method;
+    its ties and cut are defined by this framework): the k largest z, lower ids first
+    among equals; of those, every token at least as probable as the one at which the
+    cumulative probability, from the largest down, first reaches top_p of their total.
+    z: float64 [V] (already penalised and divided by the temperature).  Returns bool [V]."""
+    v = z.numel()
+    order = sorted(range(v), key=lambda i: (-float(z[i]), i))
+    if 0 < top_k < v:
+        order = order[:top_k]
+    w = torch.exp(z - z.max())
+    keep = torch.zeros(v, dtype=torch.bool)
+    if top_p < 1.0:
+        total = sum(float(w[i]) for i in order)
+        cum, cut = 0.0, order[-1]
+        for i in order:
+            cum += float(w[i])
+            if cum >= top_p * total:
+                cut = i
+                break
+        order = [i for i in order if float(z[i]) >= float(z[cut])]
+    keep[order] = True
+    return keep
+
+
+def sample_token(logits, generated, temperature, top_k, top_p, penalty, u):
+    """One draw as src/engine.rs:353-373, 403-423 orders it: repeat penalty over the
+    generated tokens, argmax if temperature <= 0, else top-k then top-p at the
+    temperature; the draw itself (this framework's definition): the first kept token, in
+    order of id, whose cumulative kept probability exceeds u times the kept total."""
+    z = apply_repeat_penalty(logits.to(torch.float32), generated, penalty) if penalty != 1.0 else logits.to(torch.float32)
+    if temperature <= 0:
+        return greedy(z)
+    z = z.to(torch.float64) / temperature
+    keep = keep_top_k_top_p(z, top_k, top_p)
+    w = torch.where(keep, torch.exp(z - z.max()), torch.zeros_like(z))
+    cum = torch.cumsum(w, 0)
+    target = u * float(cum[-1])
+    hits = torch.nonzero((cum > target) & keep)
+    return int(hits[0, 0]) if hits.numel() else int(torch.nonzero(keep)[-1, 0])
+
+
+def draw_uniform(seed, request, step):
+    """The uniform number of draw `step` of request `request`: three rounds of the
+    splitmix64 finaliser over (seed, request, step), top 24 bits.  (Defined by this
+    framework; the reference seeds one generator per request, src/engine.rs:362.)"""
+    mask = (1 << 64) - 1
+
+    def mix(x):
+        x = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & mask
+        x = ((x ^ (x >> 27)) * 0x94D049BB133111EB) & mask
+        return x ^ (x >> 31)
+    golden = 0x9E3779B97F4A7C15
+    x = mix((seed + golden) & mask)
+    x = mix(((x ^ request) + golden) & mask)
+    x = mix(((x ^ step) + golden) & mask)
+    return (x >> 40) / float(1 << 24)
+
+
+def generate(weights, cfg, prompt, max_tokens, temperature=0.0, top_k=0, top_p=1.0, penalty=1.0, seed=0,
+             request=0, eos_ids=()):
+    """src/engine.rs:364-438 for one request with any sampling settings."""
+    tokens, emitted, step = list(prompt), [], 0
+    nxt = sample_token(forward(weights, cfg, tokens)[-1], emitted, temperature, top_k, top_p, penalty,
+                       draw_uniform(seed, request, step))
+    while len(emitted) < max_tokens:
+        if nxt in eos_ids:
+            break
+        emitted.append(nxt)
+        tokens.append(nxt)
+        if len(emitted) >= max_tokens:
+            break
+        step += 1
+        nxt = sample_token(forward(weights, cfg, tokens)[-1], emitted, temperature, top_k, top_p, penalty,
+                           draw_uniform(seed, request, step))
     return emitted

@@ -1,0 +1,143 @@
+"""The generation loop's decisions, with a stand-in engine and sampler (no GPU): which
+tokens are fed, emitted and stopped on, when slots come back, how requests are cut into
+batches."""
+import pytest
+
+from tq_kv_amd import GenerationError, GenerationParams, generate
+from tq_kv_amd.engine.generate import plan_batches
+
+
+class FakeEngine:
+    """Its "logits" for a sequence are just (slot, tokens seen so far); it records steps."""
+    max_positions = 10000
+
+    def __init__(self, max_tokens=64 * 64, n_slots=8):
+        self.max_tokens = max_tokens
+        self.free = list(range(n_slots - 1, -1, -1))
+        self.seen = {}
+        self.steps = []
+        self.closed = []
+
+    def open(self):
+        s = self.free.pop()
+        self.seen[s] = []
+        return s
+
+    def close(self, slot):
+        assert slot in self.seen, "slot closed twice"
+        del self.seen[slot]
+        self.closed.append(slot)
+        self.free.append(slot)
+
+    def step(self, items):
+        self.steps.append([(s, list(t)) for s, t, _ in items])
+        out = []
+        for s, toks, want in items:
+            self.seen[s].extend(toks)
+            assert want == [len(toks) - 1]
+            out.append(list(self.seen[s]))
+        return out
+
+
+class ScriptSampler:
+    """Draws for request r the next token of scripts[r], whatever the logits."""
+
+    def __init__(self, scripts, request_ids):
+        self.scripts = [list(scripts[r]) for r in request_ids]
+        self.calls = []
+
+    def sample(self, logits, rows):
+        assert len(logits) == len(rows)
+        self.calls.append(list(rows))
+        return [self.scripts[r].pop(0) for r in rows]
+
+
+def run(prompts, scripts, max_tokens, eos=(), **kw):
+    eng = kw.pop("engine", None) or FakeEngine()
+    events = []
+    out = generate(eng, prompts, GenerationParams(max_tokens=max_tokens, temperature=0.0), eos_ids=eos,
+                   on_tokens=events.append, make_sampler=lambda p, ids: ScriptSampler(scripts, ids), **kw)
+    return out, eng, events
+
+
+def test_one_request_prompt_then_one_token_each():
+    out, eng, events = run([[5, 6, 7]], [[10, 11, 12, 13]], 3)
+    assert out == [[10, 11, 12]]
+    # the prompt whole, then each emitted token but the last is fed (src/engine.rs:364-397)
+    assert eng.steps == [[(0, [5, 6, 7])], [(0, [10])], [(0, [11])]]
+    assert events == [[(0, 10)], [(0, 11)], [(0, 12)]]
+    assert eng.seen == {} and eng.closed == [0]
+
+
+def test_stop_token_ends_without_being_emitted():
+    out, eng, _ = run([[1, 2]], [[10, 11, 99, 12]], 8, eos=(99,))
+    assert out == [[10, 11]] and eng.steps[-1] == [(0, [11])]
+    out, eng, _ = run([[1, 2]], [[99]], 8, eos=(99,))
+    assert out == [[]] and len(eng.steps) == 1
+
+
+def test_zero_max_tokens_emits_nothing():
+    out, eng, _ = run([[1, 2]], [[10]], 0)
+    assert out == [[]] and eng.seen == {}
+
+
+def test_shorter_requests_leave_the_batch_and_free_their_slot():
+    scripts = [[10, 99], [20, 21, 22, 23, 24], [30, 31, 99]]
+    out, eng, events = run([[1], [2, 2], [3, 3, 3]], scripts, 4, eos=(99,))
+    assert out == [[10], [20, 21, 22, 23], [30, 31]]
+    assert eng.steps[0] == [(0, [1]), (1, [2, 2]), (2, [3, 3, 3])]
+    assert eng.steps[1] == [(0, [10]), (1, [20]), (2, [30])]
+    assert eng.steps[2] == [(1, [21]), (2, [31])]
+    assert eng.steps[3] == [(1, [22])] and len(eng.steps) == 4
+    assert eng.closed == [0, 2, 1] and eng.seen == {}
+    assert events[0] == [(0, 10), (1, 20), (2, 30)] and events[-1] == [(1, 23)]
+
+
+def test_batches_follow_one_another_and_reuse_slots():
+    prompts = [[1] * 10, [2] * 10, [3] * 10, [4] * 10, [5] * 10]
+    scripts = [[10 + i] * 5 for i in range(5)]
+    out, eng, _ = run(prompts, scripts, 2, max_batch=2)
+    assert out == [[10, 10], [11, 11], [12, 12], [13, 13], [14, 14]]
+    firsts = [s for s in eng.steps if len(s[0][1]) == 10]
+    assert [len(s) for s in firsts] == [2, 2, 1]
+    assert {slot for s in eng.steps for slot, _ in s} == {0, 1}       # the same two slots serve all five
+    assert eng.seen == {}
+
+
+def test_plan_batches_by_cache_room():
+    # room of a request: prompt + max_new - 1 positions in whole pages of 64
+    assert plan_batches([10, 10, 10], 5, 64 * 2, 8) == [[0, 1], [2]]
+    assert plan_batches([64, 1], 2, 64 * 3, 8) == [[0, 1]]            # 65 -> 128, 2 -> 64
+    assert plan_batches([60, 60, 60, 60], 5, 64 * 64, 3) == [[0, 1, 2], [3]]
+    with pytest.raises(GenerationError, match="cache positions"):
+        plan_batches([200], 5, 64 * 2, 8)
+
+
+def test_errors():
+    with pytest.raises(GenerationError, match="Empty prompt"):
+        run([[]], [[1]], 3)
+    eng = FakeEngine()
+    eng.max_positions = 12
+    with pytest.raises(GenerationError, match="positions"):
+        run([[1] * 10], [[1] * 9], 4, engine=eng)
+
+
+def test_slots_come_back_when_a_step_fails():
+    class Boom(FakeEngine):
+        def step(self, items):
+            if len(self.steps) == 2:
+                raise RuntimeError("boom")
+            return super().step(items)
+    eng = Boom()
+    with pytest.raises(RuntimeError):
+        run([[1], [2]], [[10] * 9, [20] * 9], 6, engine=eng)
+    assert eng.seen == {} and sorted(eng.free) == list(range(8))
+
+
+def test_params_have_the_reference_defaults():
+    p = GenerationParams()
+    assert (p.max_tokens, p.temperature, p.top_p, p.top_k, p.repeat_penalty, p.seed) == (512, 0.7, 0.9, 40, 1.1, 0)
+    assert GenerationParams(temperature=0.0).greedy and not p.greedy
+    with pytest.raises(ValueError):
+        GenerationParams(top_p=0.0)
+    assert "temperature=0.7" in repr(p)

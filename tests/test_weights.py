@@ -1,0 +1,124 @@
+"""Weights: the safetensors reader and writer, the by-name loader's one error, the dtype
+policy, the random-weights mode."""
+import json
+import os
+
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from helpers import TINY_A, TINY_B
+from tq_kv_amd import Model
+from tq_kv_amd.weights import WeightError, WeightFileError, load_folder, open_folder, target_dtype, write_file
+
+
+def test_writer_and_reader_agree_with_the_safetensors_package(tmp_path):
+    t = {"a": torch.randn(3, 5).to(torch.bfloat16), "b": torch.arange(7, dtype=torch.int32), "c": torch.randn(2, 2, 2)}
+    write_file(str(tmp_path / "x.safetensors"), t)
+    back = load_file(str(tmp_path / "x.safetensors"))
+    assert set(back) == set(t) and all(torch.equal(back[k], t[k]) for k in t)
+    save_file({k: v.contiguous() for k, v in t.items()}, str(tmp_path / "y.safetensors"))
+    (tmp_path / "x.safetensors").unlink()
+    mine = open_folder(str(tmp_path))
+    assert set(mine) == set(t)
+    for k in t:
+        assert mine[k].dtype == t[k].dtype and mine[k].shape == tuple(t[k].shape) and torch.equal(mine[k].read(), t[k])
+
+
+def test_folder_errors(tmp_path):
+    with pytest.raises(WeightFileError, match="No .safetensors files found"):
+        open_folder(str(tmp_path))
+    (tmp_path / "bad.safetensors").write_bytes(b"\x05\x00")
+    with pytest.raises(WeightFileError, match="too short"):
+        open_folder(str(tmp_path))
+    (tmp_path / "bad.safetensors").write_bytes((1 << 40).to_bytes(8, "little") + b"{}")
+    with pytest.raises(WeightFileError, match="header length"):
+        open_folder(str(tmp_path))
+
+
+def _folder(tmp_path, cfg, seed=0, dtype=torch.bfloat16):
+    return Model.write_random_folder(str(tmp_path / "m"), cfg, seed=seed, store_dtype=dtype)
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    folder = _folder(tmp_path, TINY_B)
+    path = os.path.join(folder, "model.safetensors")
+    t = load_file(path)
+    del t["model.layers.1.self_attn.k_proj.bias"], t["lm_head.weight"]
+    t["model.layers.0.mlp.up_proj.weight"] = torch.zeros(224, 95, dtype=torch.bfloat16)
+    t["model.layers.2.rogue.weight"] = torch.zeros(3, dtype=torch.bfloat16)
+    t["model.norm.weight"] = torch.zeros(96, dtype=torch.int32)
+    save_file(t, path)
+    model = Model.from_config_dict(TINY_B, "float32", "cpu")
+    with pytest.raises(WeightError) as e:
+        load_folder(folder, model.tensor_specs(), torch.float32, "cpu")
+    msg = str(e.value)
+    assert "Missing tensor: model.layers.1.self_attn.k_proj.bias" in msg and "Missing tensor: lm_head.weight" in msg
+    assert "Unexpected tensor: model.layers.2.rogue.weight" in msg
+    assert "model.layers.0.mlp.up_proj.weight is [224, 95], expected [224, 96]" in msg
+    assert "Wrong dtype: model.norm.weight" in msg
+    assert e.value.missing == ["model.layers.1.self_attn.k_proj.bias", "lm_head.weight"]
+    assert len(e.value.wrong_shape) == 1 and len(e.value.unexpected) == 1
+
+
+def test_tied_model_refuses_a_head_and_untied_needs_one(tmp_path):
+    folder = _folder(tmp_path, TINY_A)
+    path = os.path.join(folder, "model.safetensors")
+    t = load_file(path)
+    assert "lm_head.weight" not in t
+    t["lm_head.weight"] = t["model.embed_tokens.weight"].clone()
+    save_file(t, path)
+    model = Model.from_config_dict(TINY_A, "float32", "cpu")
+    with pytest.raises(WeightError, match="Unexpected tensor: lm_head.weight"):
+        load_folder(folder, model.tensor_specs(), torch.float32, "cpu")
+
+
+def test_dtype_policy(tmp_path):
+    bf, f32, f16 = torch.bfloat16, torch.float32, torch.float16
+    assert target_dtype(bf, "float", bf) == bf and target_dtype(f16, "float", bf) == bf
+    assert target_dtype(f32, "float", bf) == f32                  # stored in 32-bit stays so
+    assert target_dtype(bf, "float", f32) == f32 and target_dtype(f16, "float", f32) == f32
+    assert target_dtype(torch.int64, "int32", bf) == torch.int32
+    folder = _folder(tmp_path, TINY_A)
+    path = os.path.join(folder, "model.safetensors")
+    t = load_file(path)
+    t["model.norm.weight"] = t["model.norm.weight"].to(f32) + 1e-4     # not representable in bf16
+    save_file(t, path)
+    model = Model.from_config_dict(TINY_A, "bfloat16", "cpu")
+    got = load_folder(folder, model.tensor_specs(), bf, "cpu")
+    assert got["model.norm.weight"].dtype == f32 and torch.equal(got["model.norm.weight"], t["model.norm.weight"])
+    assert got["model.embed_tokens.weight"].dtype == bf
+    got = load_folder(folder, model.tensor_specs(), f32, "cpu")
+    assert all(v.dtype == f32 for v in got.values())
+    assert torch.equal(got["model.embed_tokens.weight"], t["model.embed_tokens.weight"].to(f32))
+
+
+def test_random_folder_is_seeded_and_has_the_stated_distributions(tmp_path):
+    a = load_file(os.path.join(Model.write_random_folder(str(tmp_path / "a"), TINY_B, seed=1), "model.safetensors"))
+    b = load_file(os.path.join(Model.write_random_folder(str(tmp_path / "b"), TINY_B, seed=1), "model.safetensors"))
+    c = load_file(os.path.join(Model.write_random_folder(str(tmp_path / "c"), TINY_B, seed=2), "model.safetensors"))
+    assert set(a) == set(Model.from_config_dict(TINY_B, "float32", "cpu").tensor_specs())
+    assert all(torch.equal(a[k], b[k]) for k in a)
+    assert not torch.equal(a["lm_head.weight"], c["lm_head.weight"])
+    assert json.load(open(tmp_path / "a" / "config.json")) == TINY_B
+    w = a["model.embed_tokens.weight"].float()
+    assert abs(w.mean().item()) < 2e-3 and w.std().item() == pytest.approx(0.02, rel=0.05)
+    n = a["model.layers.0.input_layernorm.weight"].float()
+    assert n.mean().item() == pytest.approx(1.0, abs=0.01) and n.std().item() == pytest.approx(0.02, rel=0.3)
+    bias = a["model.layers.2.self_attn.q_proj.bias"].float()
+    assert bias.std().item() == pytest.approx(0.02, rel=0.3)
+    # a tensor's stream depends on the seed and its name only, not on the other tensors
+    tied = load_file(os.path.join(Model.write_random_folder(str(tmp_path / "d"), dict(TINY_B, tie_word_embeddings=True), seed=1),
+                                  "model.safetensors"))
+    assert "lm_head.weight" not in tied and torch.equal(tied["model.norm.weight"], a["model.norm.weight"])
+
+
+def test_model_lists_tensors_by_the_reference_names():
+    names = set(Model.from_config_dict(TINY_A, "float32", "cpu").tensor_specs())
+    want = {"model.embed_tokens.weight", "model.norm.weight"}
+    for l in range(2):
+        p = "model.layers.%d." % l
+        want |= {p + "self_attn.%s_proj.weight" % x for x in "qkvo"} | {p + "self_attn.%s_proj.bias" % x for x in "qkv"}
+        want |= {p + "mlp.%s_proj.weight" % x for x in ("gate", "up", "down")}
+        want |= {p + "input_layernorm.weight", p + "post_attention_layernorm.weight"}
+    assert names == want
