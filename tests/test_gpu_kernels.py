@@ -1,0 +1,326 @@
+"""Each kernel alone against a plain float32 torch expression of the same operation, at
+sizes other than the tiny models': widths and vocabularies that are no power of two,
+head sizes in steps of 16, odd numbers of heads and groups.  Inputs are made so that a
+fault shows: one far key that dominates, keys just inside and just outside a window,
+pages in scrambled order, NaN in everything that must not be read."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_qwen2 as plain
+from tq_kv_amd import kernels as K
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": dict(atol=1e-5, rtol=1e-5), "bfloat16": dict(atol=2e-2, rtol=2e-2)}
+
+
+def rand(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def ints(values):
+    return torch.tensor(values, dtype=torch.int32, device=DEV)
+
+
+def test_library_is_built_and_loaded():
+    assert K.library().tqk_abi_version() == 1
+    assert K.library_path().endswith(".so")
+    with pytest.raises(K.KernelError, match="GPU only"):
+        K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
+    with pytest.raises(K.KernelError, match="shape"):
+        K.swiglu(torch.zeros(2, 5, device=DEV), torch.zeros(2, 2, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed(dtype):
+    table = rand(301, 72, seed=1, dtype=DT[dtype])
+    ids = ints([0, 300, 17, 17, 5])
+    out = torch.full((5, 72), float("nan"), device=DEV)
+    K.embed(table, ids, out)
+    assert torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden", [72, 1000, 3584])
+def test_add_rmsnorm(dtype, hidden):
+    act = DT[dtype]
+    h = rand(7, hidden, seed=2, scale=2.0)
+    delta = rand(7, hidden, seed=3, dtype=act)
+    w = (1 + rand(hidden, seed=4, scale=0.1)).to(act)
+    eps = 3e-5
+    want_h = h + delta.float()
+    want = plain.rms_norm(want_h, w.float(), eps)
+    h1 = h.clone()
+    out = torch.empty(7, hidden, dtype=act, device=DEV)
+    K.add_rmsnorm(h1, delta, w, eps, out, write_back=True)
+    assert torch.equal(h1, want_h)
+    torch.testing.assert_close(out.float(), want, **TOL[dtype])
+    # without a delta h is only read; a float32 weight with bfloat16 activations is taken too
+    h2 = h.clone()
+    K.add_rmsnorm(h2, None, w.float(), eps, out)
+    assert torch.equal(h2, h)
+    torch.testing.assert_close(out.float(), plain.rms_norm(h, w.float(), eps), **TOL[dtype])
+    # chosen rows only, h untouched
+    rows = ints([6, 0, 3])
+    out3 = torch.empty(3, hidden, dtype=act, device=DEV)
+    K.add_rmsnorm(h2, delta, w, eps, out3, rows=rows)
+    assert torch.equal(h2, h)
+    torch.testing.assert_close(out3.float(), want[rows.long()], **TOL[dtype])
+    # norm of an activation tensor alone
+    K.add_rmsnorm(None, delta, w, eps, out)
+    torch.testing.assert_close(out.float(), plain.rms_norm(delta.float(), w.float(), eps), **TOL[dtype])
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 100, 33), (65, 129, 200), (130, 64, 48)])
+@pytest.mark.parametrize("xd,wd,yd", [("float32", "float32", "float32"), ("bfloat16", "bfloat16", "bfloat16"),
+                                      ("bfloat16", "bfloat16", "float32"), ("bfloat16", "float32", "bfloat16")])
+def test_gemm_generic(m, n, k, xd, wd, yd):
+    x, w, b = rand(m, k, seed=5, dtype=DT[xd]), rand(n, k, seed=6, dtype=DT[wd]), rand(n, seed=7, dtype=DT[wd])
+    out = torch.empty(m, n, dtype=DT[yd], device=DEV)
+    K.gemm(x, w, None, out)
+    want = x.double() @ w.double().t()
+    tol = dict(atol=1e-4, rtol=1e-5) if yd == "float32" else dict(atol=0.1, rtol=2e-2)
+    torch.testing.assert_close(out.double(), want, **tol)
+    K.gemm(x, w, b, out)
+    torch.testing.assert_close(out.double(), want + b.double(), **tol)
+
+
+def test_gemm_generic_rows_do_not_depend_on_the_batch():
+    x, w = rand(70, 96, seed=8), rand(130, 96, seed=9)
+    full = torch.empty(70, 130, device=DEV)
+    K.gemm(x, w, None, full)
+    one = torch.empty(1, 130, device=DEV)
+    K.gemm(x[41:42].contiguous(), w, None, one)
+    assert torch.equal(one[0], full[41])
+
+
+def make_cache(n_pages, nkv, d, dtype):
+    nan = float("nan")
+    return (torch.full((n_pages, nkv, 64, d), nan, dtype=dtype, device=DEV),
+            torch.full((n_pages, nkv, 64, d), nan, dtype=dtype, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("style,rot", [("halves", 48), ("pairs", 48), ("halves", 32), ("none", 0)])
+def test_rope_store(dtype, style, rot):
+    act = DT[dtype]
+    nh, nkv, d, n_pages = 5, 2, 48, 6
+    # two sequences: 3 tokens at positions 62..64 (crossing a page), 2 tokens at 130, 131
+    tok_seq, tok_pos = ints([0, 0, 0, 1, 1]), ints([62, 63, 64, 130, 131])
+    table = ints([[4, 1, -1], [0, 5, 2]])
+    qkv = rand(5, (nh + 2 * nkv) * d, seed=10, dtype=act)
+    bias = rand((nh + 2 * nkv) * d, seed=11, dtype=act)
+    keys, values = make_cache(n_pages, nkv, d, act)
+    q = torch.empty(5, nh, d, dtype=act, device=DEV)
+    if style == "none":
+        cos = sin = None
+        code = K.STYLE_NONE
+    else:
+        c, s = plain.rope_tables(rot, 777.0, 140)
+        cos, sin = c.to(DEV), s.to(DEV)
+        code = K.STYLE_HALVES if style == "halves" else K.STYLE_PAIRS
+    K.rope_store(qkv, bias, cos, sin, rot, code, tok_seq, tok_pos, table, keys, values, q, nh, nkv, d)
+
+    x = (qkv.float() + bias.float()).cpu()
+    pos = tok_pos.cpu().long()
+
+    def rotate(v):                       # v: [tokens, heads, d]
+        if style == "none":
+            return v
+        c, s = plain.rope_tables(rot, 777.0, 140)
+        c, s = c[pos][:, None, :], s[pos][:, None, :]
+        r = v[..., :rot]
+        if style == "halves":            # src/models/turbo_generic.rs:417-427
+            x0, x1 = r[..., :rot // 2], r[..., rot // 2:]
+            out = torch.cat([x0 * c - x1 * s, x0 * s + x1 * c], -1)
+        else:                            # :430-443
+            x0, x1 = r[..., 0::2], r[..., 1::2]
+            out = torch.stack([x0 * c - x1 * s, x0 * s + x1 * c], -1).flatten(-2)
+        return torch.cat([out, v[..., rot:]], -1)       # elements beyond rot_dim pass through (:752-761)
+    want_q = rotate(x[:, :nh * d].reshape(5, nh, d))
+    want_k = rotate(x[:, nh * d:(nh + nkv) * d].reshape(5, nkv, d))
+    want_v = x[:, (nh + nkv) * d:].reshape(5, nkv, d)
+    torch.testing.assert_close(q.float().cpu(), want_q, **TOL[dtype])
+    written = torch.zeros(n_pages, 64, dtype=torch.bool)
+    for t in range(5):
+        page = table.cpu()[tok_seq[t].item(), pos[t].item() // 64].item()
+        slot = pos[t].item() % 64
+        written[page, slot] = True
+        torch.testing.assert_close(keys[page, :, slot].float().cpu(), want_k[t], **TOL[dtype])
+        torch.testing.assert_close(values[page, :, slot].float().cpu(), want_v[t], **TOL[dtype])
+    # nothing else was touched
+    assert torch.isnan(keys.float().cpu().transpose(1, 2)[~written]).all()
+    assert torch.isnan(values.float().cpu().transpose(1, 2)[~written]).all()
+    # a run that reads another run's cache writes none
+    keys2, values2 = make_cache(n_pages, nkv, d, act)
+    K.rope_store(qkv, bias, cos, sin, rot, code, tok_seq, tok_pos, table, keys2, values2, q, nh, nkv, d, write_kv=False)
+    assert torch.isnan(keys2.float()).all()
+    torch.testing.assert_close(q.float().cpu(), want_q, **TOL[dtype])
+
+
+def paged(k, v, page_ids, n_pages, dtype):
+    """Lay k, v [nkv, S, d] out in pages given by page_ids; everything else is NaN."""
+    nkv, s, d = k.shape
+    keys, values = make_cache(n_pages, nkv, d, dtype)
+    for i, p in enumerate(page_ids):
+        n = min(64, s - 64 * i)
+        if p >= 0 and n > 0:
+            keys[p, :, :n] = k[:, 64 * i:64 * i + n].to(dtype)
+            values[p, :, :n] = v[:, 64 * i:64 * i + n].to(dtype)
+    return keys, values
+
+
+def attention_reference(q, k, v, pos, window, scale):
+    """q [T, nh, d] at absolute positions pos over k, v [nkv, S, d]: plain softmax attention."""
+    nh = q.shape[1]
+    n_rep = nh // k.shape[0]
+    kk, vv = plain.repeat_kv(k, n_rep), plain.repeat_kv(v, n_rep)
+    att = torch.einsum("thd,hsd->hts", q, kk) * scale
+    j = torch.arange(k.shape[1])[None, :]
+    vis = j <= pos[:, None]
+    if window:
+        vis = vis & (j > pos[:, None] - window)
+    att = torch.where(vis[None], att, torch.full_like(att, float("-inf")))
+    return torch.einsum("hts,hsd->thd", plain.softmax_last(att), vv).reshape(q.shape[0], -1)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,d", [(6, 2, 48), (5, 5, 16), (4, 1, 128), (3, 1, 80)])
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_generic(dtype, nh, nkv, d, window):
+    act = DT[dtype]
+    s = 300
+    k, v = rand(nkv, s, d, seed=12).cpu(), rand(nkv, s, d, seed=13).cpu()
+    # queries: a prompt chunk at positions 200..259 of sequence 0, and single tokens elsewhere
+    pos = torch.tensor(list(range(200, 260)) + [0, 63, 64, 299])
+    q = rand(len(pos), nh, d, seed=14).cpu()
+    # make single keys stand out: for the query at 259 the far key 3, the key at the window's
+    # edge (259-69 = 190) and the one just outside it (189)
+    q[59] = 0.0
+    q[59, :, 0] = 30.0
+    k[:, :, 0] *= 0.01
+    k[:, 3, 0], k[:, 190, 0], k[:, 189, 0] = 9.0, 8.0, 8.5
+    k, v, q = k.to(act).float(), v.to(act).float(), q.to(act).float()
+    page_ids = [7, 2, 9, 0, 5]
+    keys, values = paged(k, v, page_ids, 11, act)
+    table = ints([page_ids])
+    tok_seq = torch.zeros(len(pos), dtype=torch.int32, device=DEV)
+    out = torch.empty(len(pos), nh * d, dtype=act, device=DEV)
+    scale = 1 / math.sqrt(d)
+    K.attention(q.to(act).to(DEV), keys, values, tok_seq, pos.to(torch.int32).to(DEV), table, window, scale, out)
+    want = attention_reference(q, k, v, pos, window, scale)
+    torch.testing.assert_close(out.float().cpu(), want, **TOL[dtype])
+    # the designed query really tells the cases apart
+    other = attention_reference(q, k, v, pos, 0 if window else 70, scale)
+    assert (other[59] - want[59]).abs().max() > 0.1
+
+
+def test_attention_generic_two_sequences_share_nothing():
+    nh, nkv, d = 4, 2, 32
+    ka, va = rand(nkv, 100, d, seed=15).cpu(), rand(nkv, 100, d, seed=16).cpu()
+    kb, vb = rand(nkv, 70, d, seed=17).cpu(), rand(nkv, 70, d, seed=18).cpu()
+    keys, values = make_cache(6, nkv, d, torch.float32)
+    for (k, v, ids) in ((ka, va, [4, 1]), (kb, vb, [0, 3])):
+        kk, vv = paged(k, v, ids, 6, torch.float32)
+        for p in ids:
+            keys[p], values[p] = kk[p], vv[p]
+    table = ints([[4, 1], [0, 3]])
+    q = rand(3, nh, d, seed=19)
+    out = torch.empty(3, nh * d, device=DEV)
+    K.attention(q, keys, values, ints([0, 1, 1]), ints([99, 69, 5]), table, 0, 0.2, out)
+    qa = q.cpu()
+    want = torch.cat([attention_reference(qa[:1], ka, va, torch.tensor([99]), 0, 0.2),
+                      attention_reference(qa[1:], kb, vb, torch.tensor([69, 5]), 0, 0.2)])
+    torch.testing.assert_close(out.cpu(), want, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_swiglu(dtype):
+    act = DT[dtype]
+    gu = rand(9, 2 * 250, seed=20, scale=3.0, dtype=act)
+    out = torch.empty(9, 250, dtype=act, device=DEV)
+    K.swiglu(gu, out)
+    want = F.silu(gu.float()[:, :250]) * gu.float()[:, 250:]
+    torch.testing.assert_close(out.float(), want, **TOL[dtype])
+
+
+def test_argmax_and_ties():
+    logits = rand(6, 5003, seed=21)
+    logits[1, 77] = logits[1, 4000] = 50.0          # a tie: the lower id wins
+    logits[2, 5002] = 60.0                          # the last element
+    logits[3] = -float("inf")
+    logits[3, 9] = -1e30
+    logits[4] = 1.0                                  # all equal
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    K.argmax(logits, out)
+    want = [plain.greedy(r) for r in logits.cpu()]
+    assert out.tolist() == want and want[1] == 77 and want[2] == 5002 and want[3] == 9 and want[4] == 0
+
+
+def test_repeat_penalty():
+    logits = rand(3, 1001, seed=22)
+    base = logits.clone().cpu()
+    hist = ints([[5, 9, 5, 1000, 5, 0, 0, 0], [0] * 8, [7, 7, 7, 7, 7, 7, 7, 7]])
+    hist_len = ints([5, 0, 8])
+    K.repeat_penalty(logits, ints([0, 1, 2]), hist, hist_len, 1.3)
+    for r in range(3):
+        want = plain.apply_repeat_penalty(base[r], hist[r, :hist_len[r]].tolist(), 1.3)
+        torch.testing.assert_close(logits[r].cpu(), want, atol=0, rtol=1e-6)
+    # rows may point at any request
+    logits2 = base.clone().to(DEV)
+    K.repeat_penalty(logits2, ints([2, 2, 0]), hist, hist_len, 2.0)
+    torch.testing.assert_close(logits2[1].cpu(), plain.apply_repeat_penalty(base[1], [7] * 8, 2.0), atol=0, rtol=1e-6)
+    tokens = ints([11, 12, 13])
+    K.append_history(tokens, ints([0, 1, 2]), hist, hist_len)
+    assert hist_len.tolist() == [6, 1, 8] and hist[0, 5].item() == 11 and hist[1, 0].item() == 12   # request 2 is full
+
+
+def draw(logits, temperature, top_k, top_p, us):
+    rows = logits.repeat(len(us), 1).contiguous()
+    out = torch.empty(len(us), dtype=torch.int32, device=DEV)
+    K.sample(rows, temperature, top_k, top_p, torch.tensor(us, dtype=torch.float32, device=DEV), out)
+    return out.tolist()
+
+
+def test_sample_inverse_cdf_and_cuts():
+    probs = torch.tensor([0.1, 0.4, 0.2, 0.3])
+    logits = torch.log(probs)[None].to(DEV)
+    us = [0.0, 0.09, 0.11, 0.49, 0.51, 0.69, 0.71, 0.999]
+    assert draw(logits, 1.0, 0, 1.0, us) == [0, 0, 1, 1, 2, 2, 3, 3]
+    # top-k 2 keeps ids 1 and 3 (0.4, 0.3): the cut between them is at 4/7
+    assert draw(logits, 1.0, 2, 1.0, [0.0, 0.56, 0.58, 0.99]) == [1, 1, 3, 3]
+    # top-p 0.69 keeps 0.4 + 0.3; 0.71 needs the 0.2 as well
+    assert draw(logits, 1.0, 0, 0.69, [0.0, 0.56, 0.58, 0.99]) == [1, 1, 3, 3]
+    assert draw(logits, 1.0, 0, 0.71, [0.0, 0.43, 0.46, 0.66, 0.68, 0.99]) == [1, 1, 2, 2, 3, 3]
+    # top-k 3 then top-p 0.5 of the kept 0.9: 0.4 < 0.45 <= 0.7
+    assert draw(logits, 1.0, 3, 0.5, [0.0, 0.56, 0.58, 0.99]) == [1, 1, 3, 3]
+    # temperature: the weights become p^(1/T)
+    w = probs ** 2
+    cut = (w[0] / w.sum()).item()
+    assert draw(logits, 0.5, 0, 1.0, [cut - 0.01, cut + 0.01]) == [0, 1]
+    # equal logits: top-k keeps the lower ids
+    flat = torch.zeros(1, 7, device=DEV)
+    assert draw(flat, 1.0, 3, 1.0, [0.0, 0.32, 0.34, 0.65, 0.67, 0.99]) == [0, 0, 1, 1, 2, 2]
+
+
+@pytest.mark.parametrize("vocab,top_k,top_p,temperature", [(5003, 0, 1.0, 0.8), (5003, 40, 0.9, 0.7), (1000, 0, 0.5, 1.3),
+                                                           (151936, 40, 0.9, 0.7), (151936, 0, 0.95, 1.0), (300, 1000, 1.0, 1.0)])
+def test_sample_agrees_with_the_plain_rule(vocab, top_k, top_p, temperature):
+    logits = rand(1, vocab, seed=23, scale=3.0)
+    us = [0.001, 0.13, 0.37, 0.5, 0.77, 0.93, 0.9999]
+    got = draw(logits, temperature, top_k, top_p, us)
+    want = [plain.sample_token(logits[0].cpu(), [], temperature, top_k, top_p, 1.0, u) for u in us]
+    assert got == want
+
+
+def test_sample_frequencies_follow_the_softmax():
+    logits = torch.tensor([[0.0, 1.0, -1.0, 2.0, 0.5]], device=DEV)
+    n = 4000
+    us = ((torch.arange(n) + 0.5) / n).tolist()
+    got = torch.bincount(torch.tensor(draw(logits, 1.0, 0, 1.0, us)), minlength=5).float() / n
+    torch.testing.assert_close(got, torch.softmax(logits[0].cpu(), 0), atol=1e-3, rtol=0)

@@ -1,0 +1,277 @@
+"""Each part alone against its plain counterpart, and the generality of the
+arrangement: a run order that names a layer twice, a run that reads another run's
+cache, a norm after the mixer, and a toy mixer with state of its own that is defined
+here, registered, built and stepped without a change to the framework."""
+import pytest
+import torch
+
+import gpu_common as G
+import helpers
+import plain_qwen2 as plain
+from tq_kv_amd import Engine, Model
+from tq_kv_amd.cache import Cache
+from tq_kv_amd.engine.context import StepContext
+from tq_kv_amd.parts import (BuildEnv, KVNeed, LayerSpec, ModelSpec, Part, PartSpec, Run, StateNeed, TensorSpec,
+                             register)
+from tq_kv_amd.weights import random_tensors
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda")
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": dict(atol=1e-5, rtol=1e-5), "bfloat16": dict(atol=2e-2, rtol=2e-2)}
+
+
+def load_random(part, dtype, seed, std=0.1):
+    specs = {n: TensorSpec(s.shape, s.init, std if s.init == "normal" else 0.1) for n, s in part.tensors().items()}
+    t = random_tensors(specs, seed, DT[dtype], "cpu")
+    part.load({k: v.to(DEV) for k, v in t.items()})
+    return {k: v.float() for k, v in t.items()}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_rms_norm_part(dtype):
+    env = BuildEnv(DEV, DT[dtype])
+    norm = env.build("norm", PartSpec("rms_norm", {"size": 200, "eps": 1e-4}))
+    w = load_random(norm, dtype, 1)
+    h = torch.randn(5, 200, device=DEV)
+    d = torch.randn(5, 200, device=DEV).to(DT[dtype])
+    want_h = h + d.float()
+    got = norm.add_norm(h, d)
+    assert torch.equal(h, want_h) and got.dtype == DT[dtype]
+    torch.testing.assert_close(got.float().cpu(), plain.rms_norm(want_h.cpu(), w["weight"], 1e-4), **TOL[dtype])
+    torch.testing.assert_close(norm.forward(d).float().cpu(), plain.rms_norm(d.float().cpu(), w["weight"], 1e-4), **TOL[dtype])
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    got = norm.gather_add_norm(h, d, rows)
+    torch.testing.assert_close(got.float().cpu(), plain.rms_norm((want_h + d.float()).cpu()[[4, 1]], w["weight"], 1e-4), **TOL[dtype])
+
+
+def test_rotary_part_tables():
+    env = BuildEnv(DEV, torch.float32)
+    rot = env.build("position", PartSpec("rotary", {"theta": 1e6, "rot_dim": 48, "max_positions": 300, "style": "halves"}))
+    cos, sin, rot_dim, _ = rot.tables()
+    c, s = plain.rope_tables(48, 1e6, 300)
+    assert rot_dim == 48 and torch.equal(cos.cpu(), c) and torch.equal(sin.cpu(), s)
+    with pytest.raises(ValueError):
+        env.build("position", PartSpec("rotary", {"theta": 1e4, "rot_dim": 7, "max_positions": 8}))
+
+
+def step_ctx(cache, items):
+    """items: [(slot, tokens)]; reserves, builds the context; the caller commits."""
+    sizes = [(s, len(t)) for s, t in items]
+    cache.reserve(sizes)
+    ctx = StepContext([(s, cache.length(s), t) for s, t in items], [[] for _ in items], cache, DEV)
+    return ctx, sizes
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,d,window", [(6, 2, 48, None), (3, 1, 32, 20), (4, 4, 16, 70)])
+def test_attention_part(dtype, nh, nkv, d, window):
+    hidden = 88
+    env = BuildEnv(DEV, DT[dtype])
+    pos = PartSpec("rotary", {"theta": 1e4, "rot_dim": d, "max_positions": 256, "style": "halves"})
+    att = env.build("mixer", PartSpec("attention", {"hidden": hidden, "n_heads": nh, "n_kv_heads": nkv, "head_dim": d,
+                                                    "qkv_bias": True, "window": window, "position": pos}))
+    assert att.cache_need() == KVNeed(nkv, d, window)
+    w = load_random(att, dtype, 2)
+    cfg = {"num_attention_heads": nh, "num_key_value_heads": nkv, "head_dim": d, "rope_theta": 1e4}
+    cache = Cache([att.cache_need()], [None], 64 * 16, 4, DT[dtype], DEV)
+    xs = [torch.randn(n, hidden).to(DT[dtype]) for n in (150, 40)]     # outputs of size about 1
+    slots = [cache.acquire(), cache.acquire()]
+    # sequence 0 in two chunks and then single tokens, sequence 1 whole, in shared steps
+    plan = [[(0, 0, 100), (1, 0, 40)], [(0, 100, 140)]] + [[(0, t, t + 1)] for t in range(140, 150)]
+    got = [[], []]
+    for step in plan:
+        ctx, sizes = step_ctx(cache, [(slots[i], [0] * (b - a)) for i, a, b in step])
+        x = torch.cat([xs[i][a:b] for i, a, b in step]).to(DEV)
+        y = att.forward(x, ctx, cache.entry(0))
+        cache.commit(sizes)
+        off = 0
+        for i, a, b in step:
+            got[i].append(y[off:off + b - a])
+            off += b - a
+    for i in range(2):
+        want = plain.attention(xs[i].float(), w, "", cfg, window)
+        torch.testing.assert_close(torch.cat(got[i]).float().cpu(), want, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_feed_forward_part(dtype):
+    env = BuildEnv(DEV, DT[dtype])
+    ff = env.build("feed_forward", PartSpec("gated_silu", {"hidden": 72, "inter": 200}))
+    w = load_random(ff, dtype, 3)
+    x = torch.randn(9, 72).to(DT[dtype])
+    torch.testing.assert_close(ff.forward(x.to(DEV), None).float().cpu(), plain.swiglu_mlp(x.float(), w, ""), **TOL[dtype])
+
+
+def tiny_spec(cfg, order=None, post_norms=False, mixers=None):
+    """A ModelSpec put together by hand from the parts (what an architecture file does)."""
+    h, d = cfg["hidden_size"], cfg["head_dim"]
+    norm = PartSpec("rms_norm", {"size": h, "eps": cfg["rms_norm_eps"]})
+    pos = PartSpec("rotary", {"theta": cfg["rope_theta"], "rot_dim": d, "max_positions": cfg["max_position_embeddings"],
+                              "style": "halves"})
+    layers = []
+    for l in range(cfg["num_hidden_layers"]):
+        mixer = (mixers or {}).get(l) or PartSpec("attention", {
+            "hidden": h, "n_heads": cfg["num_attention_heads"], "n_kv_heads": cfg["num_key_value_heads"], "head_dim": d,
+            "qkv_bias": True, "window": plain.layer_window(cfg, l), "position": pos})
+        names = {"mixer": "self_attn.", "feed_forward": "mlp.", "mixer_norm": "input_layernorm.",
+                 "ff_norm": "post_attention_layernorm."}
+        params = {"mixer": mixer, "feed_forward": PartSpec("gated_silu", {"hidden": h, "inter": cfg["intermediate_size"]}),
+                  "mixer_norm": norm, "ff_norm": norm, "names": names}
+        if post_norms:
+            params.update({"post_mixer_norm": norm, "post_ff_norm": norm})
+            names.update({"post_mixer_norm": "post_mixer_norm.", "post_ff_norm": "post_ff_norm."})
+        layers.append(LayerSpec("model.layers.%d." % l, PartSpec("pre_norm", params)))
+    return ModelSpec(architecture="test", vocab_size=cfg["vocab_size"], hidden_size=h,
+                     max_positions=cfg["max_position_embeddings"], embedding_name="model.embed_tokens.weight",
+                     layers=layers, order=order or [Run(l) for l in range(len(layers))], final_norm=norm,
+                     final_norm_prefix="model.norm.", head_name="lm_head.weight")
+
+
+def run_all(model, prompt, cut):
+    eng = Engine(model, max_tokens=1024)
+    s = eng.open()
+    outs = [eng.step([(s, prompt[:cut], list(range(cut)))])]
+    for t in range(cut, len(prompt)):
+        outs.append(eng.step([(s, [prompt[t]], [0])]))
+    eng.close(s)
+    eng.cache.check()
+    return torch.cat(outs).cpu()
+
+
+def test_block_is_the_plain_decoder_layer_and_a_layer_may_run_twice():
+    cfg = dict(helpers.TINY_B)
+    _, w = G.plain_model("B", True)
+    prompt = helpers.random_tokens(40, cfg["vocab_size"], 1)
+    # order 0, 1, 2, 1: layer 1 runs twice, each run with a cache of its own
+    model = Model(tiny_spec(cfg, order=[Run(0), Run(1), Run(2), Run(1)]), "float32", DEV)
+    assert len(model.needs) == 4
+    model.load({k: v.to(DEV) for k, v in w.items()})
+    # the same thing for the plain implementation: a four-layer model whose layer 3 is layer 1
+    # (both windowed, as l >= max_window_layers)
+    w4 = dict(w)
+    for k, v in w.items():
+        if k.startswith("model.layers.1."):
+            w4[k.replace("layers.1.", "layers.3.")] = v
+    want = plain.forward(w4, dict(cfg, num_hidden_layers=4), prompt)
+    torch.testing.assert_close(run_all(model, prompt, 25), want, atol=2e-5, rtol=2e-5)
+
+
+def test_a_run_reads_another_runs_cache():
+    cfg = dict(helpers.TINY_A)
+    _, w = G.plain_model("A", True)
+    prompt = helpers.random_tokens(30, cfg["vocab_size"], 2)
+    model = Model(tiny_spec(cfg, order=[Run(0), Run(1, cache_of=0)]), "float32", DEV)
+    model.load({k: v.to(DEV) for k, v in w.items() if k != "lm_head.weight"} | {"lm_head.weight": w["model.embed_tokens.weight"].to(DEV)})
+    assert len(model.needs) == 2 and Engine(model, max_tokens=256).cache.kv_groups[0].runs == [0]
+    # plain: layer 1 attends with its own queries over layer 0's rotated keys and values
+    nh, nkv, d, eps = 4, 2, 16, cfg["rms_norm_eps"]
+    x = w["model.embed_tokens.weight"][prompt]
+    t = len(prompt)
+    cos, sin = plain.rope_tables(d, cfg["rope_theta"], t)
+    p0, p1 = "model.layers.0.", "model.layers.1."
+    h = plain.rms_norm(x, w[p0 + "input_layernorm.weight"], eps)
+    k0 = plain.rope_half(plain.linear(h, w[p0 + "self_attn.k_proj.weight"], w[p0 + "self_attn.k_proj.bias"]).reshape(t, nkv, d).transpose(0, 1), cos, sin)
+    v0 = plain.linear(h, w[p0 + "self_attn.v_proj.weight"], w[p0 + "self_attn.v_proj.bias"]).reshape(t, nkv, d).transpose(0, 1)
+    x = plain.decoder_layer(x, w, 0, cfg)
+    h = plain.rms_norm(x, w[p1 + "input_layernorm.weight"], eps)
+    q1 = plain.rope_half(plain.linear(h, w[p1 + "self_attn.q_proj.weight"], w[p1 + "self_attn.q_proj.bias"]).reshape(t, nh, d).transpose(0, 1), cos, sin)
+    y = plain.attention_core(q1, k0, v0, plain.visibility(t)).transpose(0, 1).reshape(t, nh * d)
+    x = x + plain.linear(y, w[p1 + "self_attn.o_proj.weight"])
+    x = x + plain.swiglu_mlp(plain.rms_norm(x, w[p1 + "post_attention_layernorm.weight"], eps), w, p1 + "mlp.")
+    want = plain.linear(plain.rms_norm(x, w["model.norm.weight"], eps), w["model.embed_tokens.weight"])
+    torch.testing.assert_close(run_all(model, prompt, 17), want, atol=2e-5, rtol=2e-5)
+
+
+def test_norms_after_mixer_and_feed_forward():
+    # the optional norms of src/models/turbo_generic.rs:1965-1968, 1976-1979
+    cfg = dict(helpers.TINY_A, num_hidden_layers=1)
+    model = Model(tiny_spec(cfg, post_norms=True), "float32", DEV)
+    specs = {n: TensorSpec(s.shape, s.init, 0.2 if s.init == "normal" else 0.1) for n, s in model.tensor_specs().items()}
+    w = random_tensors(specs, 5, torch.float32, "cpu")
+    model.load({k: v.to(DEV) for k, v in w.items()})
+    prompt = helpers.random_tokens(12, cfg["vocab_size"], 3)
+    p, eps = "model.layers.0.", cfg["rms_norm_eps"]
+    x = w["model.embed_tokens.weight"][prompt]
+    a = plain.attention(plain.rms_norm(x, w[p + "input_layernorm.weight"], eps), w, p + "self_attn.", cfg, None)
+    x = x + plain.rms_norm(a, w[p + "post_mixer_norm.weight"], eps)
+    f = plain.swiglu_mlp(plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], eps), w, p + "mlp.")
+    x = x + plain.rms_norm(f, w[p + "post_ff_norm.weight"], eps)
+    want = plain.linear(plain.rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"])
+    torch.testing.assert_close(run_all(model, prompt, 7), want, atol=2e-5, rtol=2e-5)
+
+
+# ---- a toy mixer with state of its own -------------------------------------------------------
+@register("mixer", "toy_decay")
+class ToyDecay(Part):
+    """y_t = W s_t with s_t = decay * s_{t-1} + x_t: a recurrence with a fixed-size state per
+    sequence, kept in the cache's state rows.  Plain torch on the device; it exists to show
+    that the framework's interfaces carry a mixer that is not attention."""
+
+    def __init__(self, params, env):
+        self.hidden, self.decay = params["hidden"], params["decay"]
+
+    def tensors(self):
+        return {"mix.weight": TensorSpec((self.hidden, self.hidden))}
+
+    def load(self, tensors):
+        self.w = tensors["mix.weight"]
+
+    def cache_need(self):
+        return StateNeed((self.hidden,))
+
+    def forward(self, x, ctx, entry):
+        out = torch.empty_like(x)
+        for b in range(ctx.n_seqs):
+            a, e = int(ctx.host.cu[b]), int(ctx.host.cu[b + 1])
+            s = entry.state[int(ctx.host.seq_slot[b])]
+            for t in range(a, e):
+                s.mul_(self.decay).add_(x[t].float())
+                out[t] = (self.w.float() @ s).to(x.dtype)
+        return out
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped():
+    cfg = dict(helpers.TINY_A, num_hidden_layers=3)
+    toy = PartSpec("toy_decay", {"hidden": cfg["hidden_size"], "decay": 0.5})
+    model = Model(tiny_spec(cfg, mixers={1: toy}), "float32", DEV)       # attention, toy, attention
+    assert model.needs[1] == StateNeed((64,)) and isinstance(model.needs[0], KVNeed)
+    assert "model.layers.1.self_attn.mix.weight" in model.tensor_specs()
+    specs = {n: TensorSpec(s.shape, s.init, 0.2 if s.init == "normal" else 0.1) for n, s in model.tensor_specs().items()}
+    w = random_tensors(specs, 6, torch.float32, "cpu")
+    model.load({k: v.to(DEV) for k, v in w.items()})
+    eng = Engine(model, max_tokens=1024)
+    assert len(eng.cache.state_groups) == 1 and len(eng.cache.kv_groups) == 1
+
+    def plain_forward(tokens):
+        x = w["model.embed_tokens.weight"][tokens]
+        eps = cfg["rms_norm_eps"]
+        for l in range(3):
+            p = "model.layers.%d." % l
+            h = plain.rms_norm(x, w[p + "input_layernorm.weight"], eps)
+            if l == 1:
+                s, ys = torch.zeros(64), []
+                for t in range(len(tokens)):
+                    s = 0.5 * s + h[t]
+                    ys.append(w[p + "self_attn.mix.weight"] @ s)
+                x = x + torch.stack(ys)
+            else:
+                x = x + plain.attention(h, w, p + "self_attn.", cfg, None)
+            x = x + plain.swiglu_mlp(plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], eps), w, p + "mlp.")
+        return plain.linear(plain.rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"])
+
+    a, b = helpers.random_tokens(20, 256, 4), helpers.random_tokens(9, 256, 5)
+    for round_ in range(2):                      # twice: the second time on used slots, whose state must be zero again
+        sa, sb = eng.open(), eng.open()
+        out = eng.step([(sa, a[:12], list(range(12))), (sb, b[:4], list(range(4)))])
+        got_a, got_b = [out[:12]], [out[12:]]
+        for t in range(5):
+            out = eng.step([(sa, [a[12 + t]], [0]), (sb, [b[4 + t]], [0])])
+            got_a.append(out[:1]), got_b.append(out[1:])
+        eng.close(sb)
+        for t in range(17, 20):
+            got_a.append(eng.step([(sa, [a[t]], [0])]))
+        eng.close(sa)
+        torch.testing.assert_close(torch.cat(got_a).cpu(), plain_forward(a), atol=2e-5, rtol=2e-5)
+        torch.testing.assert_close(torch.cat(got_b).cpu(), plain_forward(b), atol=2e-5, rtol=2e-5)
+    eng.cache.check()
