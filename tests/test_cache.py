@@ -50,7 +50,7 @@ def test_groups_have_storage_of_their_own():
     full = next(g for g in c.kv_groups if g.need.window is None)
     win = next(g for g in c.kv_groups if g.need.window == 100)
     assert full.runs == [0, 3] and win.runs == [1, 2]
-    assert full.keys.shape == (2, 8, 2, PAGE, 16) and win.values.shape == (2, 8, 2, PAGE, 16)
+    assert full.keys.shape == (2, 8, 2, PAGE, 16) and win.values.shape == (2, 8, 2, 16, PAGE)
     assert c.entry(3).keys.data_ptr() == full.keys[1].data_ptr()
     assert c.entry(1).group is win and c.entry(1).writes
 

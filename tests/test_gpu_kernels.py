@@ -101,8 +101,9 @@ def test_gemm_generic_rows_do_not_depend_on_the_batch():
 
 def make_cache(n_pages, nkv, d, dtype):
     nan = float("nan")
+    # keys [pages, kv heads, 64, d]; values are kept transposed inside a page
     return (torch.full((n_pages, nkv, 64, d), nan, dtype=dtype, device=DEV),
-            torch.full((n_pages, nkv, 64, d), nan, dtype=dtype, device=DEV))
+            torch.full((n_pages, nkv, d, 64), nan, dtype=dtype, device=DEV))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -152,10 +153,10 @@ def test_rope_store(dtype, style, rot):
         slot = pos[t].item() % 64
         written[page, slot] = True
         torch.testing.assert_close(keys[page, :, slot].float().cpu(), want_k[t], **TOL[dtype])
-        torch.testing.assert_close(values[page, :, slot].float().cpu(), want_v[t], **TOL[dtype])
+        torch.testing.assert_close(values[page, :, :, slot].float().cpu(), want_v[t], **TOL[dtype])
     # nothing else was touched
     assert torch.isnan(keys.float().cpu().transpose(1, 2)[~written]).all()
-    assert torch.isnan(values.float().cpu().transpose(1, 2)[~written]).all()
+    assert torch.isnan(values.float().cpu().permute(0, 3, 1, 2)[~written]).all()
     # a run that reads another run's cache writes none
     keys2, values2 = make_cache(n_pages, nkv, d, act)
     K.rope_store(qkv, bias, cos, sin, rot, code, tok_seq, tok_pos, table, keys2, values2, q, nh, nkv, d, write_kv=False)
@@ -171,7 +172,7 @@ def paged(k, v, page_ids, n_pages, dtype):
         n = min(64, s - 64 * i)
         if p >= 0 and n > 0:
             keys[p, :, :n] = k[:, 64 * i:64 * i + n].to(dtype)
-            values[p, :, :n] = v[:, 64 * i:64 * i + n].to(dtype)
+            values[p, :, :, :n] = v[:, 64 * i:64 * i + n].transpose(1, 2).to(dtype)
     return keys, values
 
 
@@ -324,3 +325,89 @@ def test_sample_frequencies_follow_the_softmax():
     us = ((torch.arange(n) + 0.5) / n).tolist()
     got = torch.bincount(torch.tensor(draw(logits, 1.0, 0, 1.0, us)), minlength=5).float() / n
     torch.testing.assert_close(got, torch.softmax(logits[0].cpu(), 0), atol=1e-3, rtol=0)
+
+
+@pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("n,k", [(100, 96), (3584, 3584), (1000, 18944), (4608, 1536), (48, 32)])
+def test_skinny_product(m, n, k):
+    x, w = rand(m, k, seed=30, dtype=torch.bfloat16), rand(n, k, seed=31, scale=0.05, dtype=torch.bfloat16)
+    want = x.double() @ w.double().t()
+    out = torch.full((m, n), float("nan"), device=DEV)
+    K.skinny_bf16(x, w, out)
+    torch.testing.assert_close(out.double(), want, atol=2e-3, rtol=1e-3)
+    out16 = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    K.skinny_bf16(x, w, out16)
+    assert torch.equal(out16, out.to(torch.bfloat16))
+    # a row's result does not depend on the other rows
+    if m > 1:
+        one = torch.empty(1, n, device=DEV)
+        K.skinny_bf16(x[m - 1:].contiguous(), w, one)
+        assert torch.equal(one[0], out[m - 1])
+
+
+@pytest.mark.parametrize("m", [1, 8, 40, 64])
+@pytest.mark.parametrize("inter,k", [(112, 64), (18944, 3584), (200, 1536)])
+def test_skinny_gated(m, inter, k):
+    x, w = rand(m, k, seed=32, dtype=torch.bfloat16), rand(2 * inter, k, seed=33, scale=0.05, dtype=torch.bfloat16)
+    gu = (x.double() @ w.double().t()).float().to(torch.bfloat16).float()
+    want = (F.silu(gu[:, :inter]) * gu[:, inter:])
+    out = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    K.skinny_bf16(x, w, out, swiglu=True)
+    torch.testing.assert_close(out.float(), want, atol=2e-2, rtol=2e-2)
+
+
+def test_skinny_refuses_what_it_does_not_take():
+    x, w = rand(65, 64, dtype=torch.bfloat16), rand(16, 64, dtype=torch.bfloat16)
+    with pytest.raises(K.KernelError, match="at most 64"):
+        K.skinny_bf16(x, w, torch.empty(65, 16, device=DEV))
+    with pytest.raises(K.KernelError, match="multiple of 32"):
+        K.skinny_bf16(rand(2, 48, dtype=torch.bfloat16), rand(16, 48, dtype=torch.bfloat16), torch.empty(2, 16, device=DEV))
+
+
+@pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (3, 1, 96), (40, 2, 64), (4, 1, 256)])
+@pytest.mark.parametrize("window", [0, 70])
+@pytest.mark.parametrize("target_waves", [1, 64, 100000])
+def test_attention_decode(nh, nkv, d, window, target_waves):
+    # three sequences of lengths 300, 64 and 1, pages scrambled, everything unread is NaN
+    lens = [300, 64, 1]
+    n_pages = 12
+    keys, values = make_cache(n_pages, nkv, d, torch.bfloat16)
+    tables = [[7, 2, 9, 0, 5], [4, -1, -1, -1, -1], [11, -1, -1, -1, -1]]
+    ks, vs = [], []
+    for i, n in enumerate(lens):
+        k, v = rand(nkv, n, d, seed=40 + i).cpu(), rand(nkv, n, d, seed=50 + i).cpu()
+        if n == 300:
+            k[:, :, 0] *= 0.01
+            k[:, 3, 0], k[:, 230, 0], k[:, 229, 0] = 9.0, 8.0, 8.5     # far key, window edge (299-69), just outside
+        k, v = k.to(torch.bfloat16).float(), v.to(torch.bfloat16).float()
+        kk, vv = paged(k, v, tables[i], n_pages, torch.bfloat16)
+        for p in tables[i]:
+            if p >= 0:
+                keys[p], values[p] = kk[p], vv[p]
+        ks.append(k), vs.append(v)
+    q = rand(3, nh, d, seed=60).cpu()
+    q[0] = 0.0
+    q[0, :, 0] = 30.0
+    q = q.to(torch.bfloat16)
+    pos = torch.tensor([n - 1 for n in lens])
+    out = torch.empty(3, nh * d, dtype=torch.bfloat16, device=DEV)
+    scale = 1 / math.sqrt(d)
+    K.attention_decode(q.to(DEV), keys, values, pos.to(torch.int32).to(DEV), ints(tables), window, scale, out,
+                       target_waves=target_waves)
+    for i in range(3):
+        want = attention_reference(q[i:i + 1].float(), ks[i], vs[i], pos[i:i + 1], window, scale)
+        torch.testing.assert_close(out[i:i + 1].float().cpu(), want, atol=2e-2, rtol=2e-2)
+    other = attention_reference(q[:1].float(), ks[0], vs[0], pos[:1], 0 if window else 70, scale)
+    assert (other - out[:1].float().cpu()).abs().max() > 0.1
+    # the plain kernel agrees
+    out2 = torch.empty_like(out)
+    K.attention(q.to(DEV), keys, values, ints([0, 1, 2]), pos.to(torch.int32).to(DEV), ints(tables), window, scale, out2)
+    torch.testing.assert_close(out.float(), out2.float(), atol=2e-2, rtol=2e-2)
+
+
+def test_attention_decode_refuses_other_head_sizes():
+    assert not K.attention_decode_supported(48) and K.attention_decode_supported(128)
+    keys, values = make_cache(2, 1, 48, torch.bfloat16)
+    with pytest.raises(K.KernelError, match="head_dim 48"):
+        K.attention_decode(rand(1, 1, 48, dtype=torch.bfloat16), keys, values, ints([0]), ints([[0]]), 0, 1.0,
+                           torch.empty(1, 48, dtype=torch.bfloat16, device=DEV))

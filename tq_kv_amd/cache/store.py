@@ -4,7 +4,9 @@ the order, fixed-size state beside them.
 Runs of the order with the same need (same kv heads, head size and window) form a
 group.  A group has storage of its own: one pool of pages of PAGE positions,
 
-    keys, values: [runs in group, pages, kv heads, PAGE, head_dim]
+    keys:   [runs in group, pages, kv heads, PAGE, head_dim]
+    values: [runs in group, pages, kv heads, head_dim, PAGE]   (transposed inside a page:
+            the attention kernels read 8 consecutive positions of one element at once)
 
 and, per slot, the list of pages that hold the slot's positions.  A group with a
 window gives pages back as soon as every position in them has left the window; a
@@ -59,7 +61,7 @@ class KVGroup:
         self.pool = FreeList(n_pages, "page")
         shape = (len(self.runs), n_pages, need.n_kv_heads, PAGE, need.head_dim)
         self.keys = torch.zeros(shape, dtype=dtype, device=device)
-        self.values = torch.zeros(shape, dtype=dtype, device=device)
+        self.values = torch.zeros(shape[:3] + (need.head_dim, PAGE), dtype=dtype, device=device)
         self.pages = {}               # slot -> list of page ids, -1 where given back
 
     def first_needed(self, length):

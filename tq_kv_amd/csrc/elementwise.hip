@@ -107,15 +107,24 @@ __global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restri
     const TA* src = qkv + (size_t)t * total + (size_t)head * head_dim;
     const TB* b = bias ? bias + (size_t)head * head_dim : nullptr;
 
+    // q rows and key rows are contiguous in head_dim; values are kept transposed inside a
+    // page, [kv head][head_dim][position in page], so that the matrix cores can read 8
+    // consecutive positions of one element as 16 contiguous bytes.
     TA* dst;
+    size_t dst_stride = 1;
     if (kind == 0) {
         dst = q_out + ((size_t)t * n_heads + head) * head_dim;
     } else {
         const int kvh = kind == 1 ? head - n_heads : head - n_heads - n_kv_heads;
         const int page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
         if (page < 0) return;                          // the host never lets this happen
-        TA* base = kind == 1 ? keys : values;
-        dst = base + (((size_t)page * n_kv_heads + kvh) * TQK_PAGE + (pos % TQK_PAGE)) * head_dim;
+        const size_t base = ((size_t)page * n_kv_heads + kvh) * TQK_PAGE * head_dim;
+        if (kind == 1) {
+            dst = keys + base + (size_t)(pos % TQK_PAGE) * head_dim;
+        } else {
+            dst = values + base + (pos % TQK_PAGE);
+            dst_stride = TQK_PAGE;
+        }
     }
 
     const int half_rot = rot_dim / 2;
@@ -132,7 +141,7 @@ __global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restri
             const float s = sin_table[(size_t)pos * half_rot + p];
             x = first ? x * c - y * s : y * s + x * c;
         }
-        dst[i] = from_float<TA>(x);
+        dst[(size_t)i * dst_stride] = from_float<TA>(x);
     }
 }
 

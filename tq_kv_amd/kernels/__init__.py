@@ -117,7 +117,8 @@ def gemm(x, w, bias, out):
 
 def rope_store(qkv, bias, cos, sin, rot_dim, style, tok_seq, tok_pos, page_table, keys, values, q_out,
                n_heads, n_kv_heads, head_dim, write_kv=True):
-    """Bias, rotation of q and k, q to q_out, k and v into the cache pages."""
+    """Bias, rotation of q and k, q to q_out, k and v into the cache pages
+    (keys [pages, kv heads, 64, d], values [pages, kv heads, d, 64])."""
     n = qkv.shape[0]
     total = (n_heads + 2 * n_kv_heads) * head_dim
     max_pos = 0
@@ -129,9 +130,8 @@ def rope_store(qkv, bias, cos, sin, rot_dim, style, tok_seq, tok_pos, page_table
     if write_kv:
         n_seqs, width = page_table.shape
         n_pages = keys.shape[0]
-        shape = (n_pages, n_kv_heads, 64, head_dim)
-        _dev(keys, "keys", qkv.dtype, shape)
-        _dev(values, "values", qkv.dtype, shape)
+        _dev(keys, "keys", qkv.dtype, (n_pages, n_kv_heads, 64, head_dim))
+        _dev(values, "values", qkv.dtype, (n_pages, n_kv_heads, head_dim, 64))
     _check(library().tqk_rope_store(
         _dev(qkv, "qkv", None, (n, total)), _code(qkv.dtype), _opt(bias, "bias", None, (total,)),
         _code(bias.dtype) if bias is not None else 0,
@@ -149,9 +149,9 @@ def attention(q, keys, values, tok_seq, tok_pos, page_table, window, scale, out)
     n, n_heads, head_dim = q.shape
     n_pages, n_kv_heads = keys.shape[0], keys.shape[1]
     n_seqs, width = page_table.shape
-    shape = (n_pages, n_kv_heads, 64, head_dim)
     _check(library().tqk_attention(
-        _dev(q, "q"), _dev(keys, "keys", q.dtype, shape), _dev(values, "values", q.dtype, shape), _code(q.dtype),
+        _dev(q, "q"), _dev(keys, "keys", q.dtype, (n_pages, n_kv_heads, 64, head_dim)),
+        _dev(values, "values", q.dtype, (n_pages, n_kv_heads, head_dim, 64)), _code(q.dtype),
         _dev(tok_seq, "tok_seq", torch.int32, (n,)), _dev(tok_pos, "tok_pos", torch.int32, (n,)),
         _dev(page_table, "page_table", torch.int32), width, n_seqs, n_pages, int(window or 0), ctypes.c_float(scale),
         _dev(out, "out", q.dtype, (n, n_heads * head_dim)), n, n_heads, n_kv_heads, head_dim, _stream()), "attention")
@@ -219,4 +219,32 @@ def sample(logits, temperature, top_k, top_p, uniforms, out):
         _dev(logits, "logits", torch.float32), rows, vocab, ctypes.c_float(temperature), int(top_k),
         ctypes.c_float(top_p), _dev(uniforms, "uniforms", torch.float32, (rows,)),
         _dev(out, "out", torch.int32, (rows,)), _stream()), "sample")
+    return out
+
+
+def attention_decode_supported(head_dim):
+    return bool(library().tqk_attention_decode_supported(int(head_dim)))
+
+
+def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, target_waves=2048):
+    """Attention of one new token per sequence (q [B, heads, d] bfloat16, row b belongs to
+    sequence b at position tok_pos[b]) over the paged cache; out [B, heads*d]."""
+    n, n_heads, head_dim = q.shape
+    n_pages, n_kv_heads = keys.shape[0], keys.shape[1]
+    n_seqs, width = page_table.shape
+    if n_seqs != n:
+        raise KernelError("attention_decode: %d query rows for %d sequences (one token each is required)" % (n, n_seqs))
+    q_blocks = (n_heads // n_kv_heads + 15) // 16
+    want_parts = max(1, min(width, target_waves // max(1, n * n_kv_heads * q_blocks)))
+    per_part = (width + want_parts - 1) // want_parts
+    n_parts = (width + per_part - 1) // per_part
+    part_out = torch.empty((n, n_heads, n_parts, head_dim), dtype=torch.float32, device=q.device)
+    part_ml = torch.empty((n, n_heads, n_parts, 2), dtype=torch.float32, device=q.device)
+    _check(library().tqk_attention_decode(
+        _dev(q, "q", torch.bfloat16), _dev(keys, "keys", torch.bfloat16, (n_pages, n_kv_heads, 64, head_dim)),
+        _dev(values, "values", torch.bfloat16, (n_pages, n_kv_heads, head_dim, 64)),
+        _dev(tok_pos, "tok_pos", torch.int32, (n,)), _dev(page_table, "page_table", torch.int32), width, n, n_pages,
+        int(window or 0), ctypes.c_float(scale), per_part, n_parts, _dev(part_out, "part_out"), _dev(part_ml, "part_ml"),
+        _dev(out, "out", torch.bfloat16, (n, n_heads * head_dim)), n_heads, n_kv_heads, head_dim, _stream()),
+        "attention_decode")
     return out

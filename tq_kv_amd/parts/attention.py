@@ -93,6 +93,17 @@ class Attention(Part):
         return linear(y, self.w_o, self.b_o)
 
 
+# The bfloat16 attention kernels can be switched off one by one (tests compare each with
+# the plain kernel); nothing else reads these.
+POLICY = {"decode_mfma": True, "prefill_mfma": True}
+
+
 def attend(q, entry, table, ctx, window, scale, out):
-    """Softmax attention of q over the cache entry: picks the kernel for the step."""
+    """Softmax attention of q over the cache entry: picks the kernel for the step.
+
+    float32, or a head size the MFMA kernels do not take: the plain kernel, one wave per
+    (token, head).  bfloat16 and one token per sequence: the partitioned decoding kernel."""
+    head_dim = q.shape[2]
+    if q.dtype == torch.bfloat16 and ctx.all_decode and POLICY["decode_mfma"] and K.attention_decode_supported(head_dim):
+        return K.attention_decode(q, entry.keys, entry.values, ctx.dev.tok_pos, table, window, scale, out)
     return K.attention(q, entry.keys, entry.values, ctx.dev.tok_seq, ctx.dev.tok_pos, table, window, scale, out)

@@ -3,8 +3,7 @@
 up are one product with the weights stacked."""
 import torch
 
-from .. import kernels as K
-from .linear import linear
+from .linear import gated_silu_linear, linear
 from .registry import Part, register
 from .spec import TensorSpec
 
@@ -30,7 +29,4 @@ class GatedSiLU(Part):
         self.w_down = tensors["down_proj.weight"]
 
     def forward(self, x, ctx):
-        gate_up = linear(x, self.w_gate_up)
-        act = torch.empty((x.shape[0], self.inter), dtype=x.dtype, device=x.device)
-        K.swiglu(gate_up, act)
-        return linear(act, self.w_down)
+        return linear(gated_silu_linear(x, self.w_gate_up), self.w_down)

@@ -19,6 +19,23 @@ from .. import kernels as K
 POLICY = {"skinny": True, "library": True, "skinny_max_rows": 64}
 
 
+def _skinny_ok(x, weight):
+    return (POLICY["skinny"] and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+            and x.shape[1] % 32 == 0 and x.shape[0] <= POLICY["skinny_max_rows"] and K.has_skinny())
+
+
+def gated_silu_linear(x, weight_gate_up):
+    """silu(x Wg^T) * (x Wu^T) with Wg stacked on Wu: [M, K] x [2I, K] -> [M, I].  For few
+    rows of bfloat16 the gate and the up row of an output are computed by the same wave
+    and never written; otherwise one product and the SwiGLU kernel."""
+    m = x.shape[0]
+    inter = weight_gate_up.shape[0] // 2
+    act = torch.empty((m, inter), dtype=x.dtype, device=x.device)
+    if _skinny_ok(x, weight_gate_up):
+        return K.skinny_bf16(x, weight_gate_up, act, swiglu=True)
+    return K.swiglu(linear(x, weight_gate_up), act)
+
+
 def linear(x, weight, bias=None, out_dtype=None):
     """x: [M,K]; weight: [N,K]; bias: [N] or None.  Returns [M,N] of out_dtype
     (default: x's dtype)."""
@@ -29,7 +46,7 @@ def linear(x, weight, bias=None, out_dtype=None):
     out_dtype = out_dtype or x.dtype
     both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
     if both_bf16 and bias is None:
-        if POLICY["skinny"] and K.has_skinny() and k % 32 == 0 and m <= POLICY["skinny_max_rows"]:
+        if _skinny_ok(x, weight):
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
             return K.skinny_bf16(x, weight, out)
         if POLICY["library"] and out_dtype == torch.bfloat16 and m > POLICY["skinny_max_rows"]:
