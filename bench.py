@@ -1,0 +1,116 @@
+"""Decode and prefill throughput of the Qwen2.5-7B shape with random bfloat16 weights on
+one MI355X: `python bench.py [--gpus 1] [--steps K] [--warmup W]` prints one JSON line.
+
+A step is one decode step of the whole batch through the generation loop (step
+function, sampling, host round trip for the stop check).  The reference measures
+tokens per second of one chat request including its prompt (src/main.rs:1123-1143);
+here decoding is timed alone and the prompt pass is reported beside it.
+"""
+import argparse
+import json
+import sys
+import time
+
+PEAK = {"hbm_gbs": 8000.0, "bf16_flops": 2.5e15}     # MI355X: HBM3E 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s
+SHAPE = "qwen2.5:7b"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
+    ap.add_argument("--shape", default=SHAPE)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this library runs on one GPU; --gpus %d is not supported" % args.gpus)
+        return 2
+
+    import torch
+
+    from tq_kv_amd import Engine, GenerationParams, Model, generate
+    from tq_kv_amd.config import catalog
+
+    raw = dict(catalog.find(args.shape))
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    layers = raw["num_hidden_layers"]
+    H, I, V = raw["hidden_size"], raw["intermediate_size"], raw["vocab_size"]
+    nh, nkv, d = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"]
+    ctx_len = raw["max_position_embeddings"]
+    model = Model.random(raw, seed=0, dtype="bfloat16", device="cuda:0")
+    max_batch = 64 if not args.no_points else args.batch
+    total_new = args.steps + args.warmup + 2
+    engine = Engine(model, max_tokens=max_batch * ((args.prompt_len + total_new + 63) // 64 * 64))
+    gen = torch.Generator().manual_seed(0)
+
+    def prompts(n):
+        return torch.randint(0, V, (n, args.prompt_len), generator=gen).tolist()
+
+    # -- prefill of one prompt --------------------------------------------------------------
+    p = prompts(1)[0]
+    times = []
+    for i in range(4):
+        slot = engine.open()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([(slot, p, [len(p) - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.close(slot)
+    prefill_s = min(times[1:])
+    T = args.prompt_len
+    linear_params = layers * (H * (nh + 2 * nkv) * d + nh * d * H + 3 * H * I)
+    prefill_flops = 2.0 * T * linear_params + layers * 4.0 * nh * d * (T * (T + 1) / 2) + 2.0 * H * V
+    prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+               "frac": round(prefill_flops / prefill_s / PEAK["bf16_flops"], 4)}
+
+    # -- decoding ---------------------------------------------------------------------------
+    def decode(batch, steps, warmup):
+        """Tokens per second over `steps` decode steps of `batch` sequences after their prompts."""
+        marks = []
+
+        def on_tokens(pairs):
+            torch.cuda.synchronize()
+            marks.append(time.perf_counter())
+        params = GenerationParams(max_tokens=warmup + steps + 1, temperature=0.0, repeat_penalty=1.0)
+        out = generate(engine, prompts(batch), params, on_tokens=on_tokens, max_batch=batch)
+        assert all(len(o) == warmup + steps + 1 for o in out)
+        # marks[i] is taken after the tokens of draw i are known; draw i+1 needs decode step i+1
+        seconds = marks[warmup + steps] - marks[warmup]
+        return batch * steps / seconds, seconds / steps
+
+    tps, sec_per_step = decode(args.batch, args.steps, args.warmup)
+    points = {}
+    if not args.no_points:
+        points["decode_b1"] = round(decode(1, min(args.steps, 64), 8)[0], 1)
+        points["decode_b64"] = round(decode(64, min(args.steps, 32), 4)[0], 1)
+
+    weight_bytes = 2.0 * (linear_params + H * V)                      # every weight the step uses, once
+    mean_ctx = args.prompt_len + args.warmup + args.steps / 2.0
+    kv_bytes = args.batch * mean_ctx * layers * 2 * nkv * d * 2.0        # keys and values of the live requests
+    achieved = (weight_bytes + kv_bytes) / sec_per_step / 1e9
+    line = {
+        "metric": "decode tok/s @ batch %d, %s shape" % (args.batch, args.shape), "value": round(tps, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"model": args.shape, "global_batch": args.batch, "seq_len": ctx_len, "parallelism": "single-gpu",
+                   "layers": layers, "layers_of_shape": full_layers, "hidden": H, "heads": nh, "kv_heads": nkv,
+                   "head_dim": d, "intermediate": I, "vocab": V, "prompt_len": args.prompt_len,
+                   "new_tokens": args.warmup + args.steps + 1, "weights": "random N(0,0.02)", "sampling": "greedy"},
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK["hbm_gbs"], "unit": "GB/s",
+                     "frac": round(achieved / PEAK["hbm_gbs"], 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -24,14 +24,18 @@ class HostStaging:
         self.buf = None
         self.event = None
 
-    def upload(self, packed):
+    def upload(self, packed, into=None):
+        """Copy the packed array to the device: into `into` (a device buffer of the same
+        size that a captured graph reads) or into a new tensor."""
         n = packed.shape[0]
         if self.event is not None:
             self.event.synchronize()
         if self.buf is None or self.buf.shape[0] < n:
             self.buf = torch.empty(max(4096, 2 * n), dtype=torch.int32, pin_memory=True)
         self.buf[:n].numpy()[:] = packed
-        dev = torch.empty(n, dtype=torch.int32, device=self.device)
+        dev = into if into is not None else torch.empty(n, dtype=torch.int32, device=self.device)
+        if dev.shape[0] != n:
+            raise ValueError("the step's arrays take %d values, the buffer holds %d" % (n, dev.shape[0]))
         dev.copy_(self.buf[:n], non_blocking=True)
         self.event = torch.cuda.Event()
         self.event.record()
@@ -42,7 +46,7 @@ class StepContext:
     """items: [(slot, start, tokens)] with `start` the sequence's length before the step;
     want: for each item the indices among its tokens whose logits are wanted."""
 
-    def __init__(self, items, want, cache, device, staging=None):
+    def __init__(self, items, want, cache, device, staging=None, width_step=1, into=None):
         self.n_seqs = len(items)
         lens = [len(toks) for _, _, toks in items]
         self.n_tokens = int(sum(lens))
@@ -70,6 +74,13 @@ class StepContext:
         self.groups = list(cache.kv_groups) if cache is not None else []
         slots = [slot for slot, _, _ in items]
         self.host_tables = [cache.page_table(g, slots) for g in self.groups]
+        if width_step > 1:
+            # widths in steps, so that a captured graph serves until a sequence outgrows them
+            for i, t in enumerate(self.host_tables):
+                width = (t.shape[1] + width_step - 1) // width_step * width_step
+                wide = np.full((t.shape[0], width), -1, dtype=np.int32)
+                wide[:, :t.shape[1]] = t
+                self.host_tables[i] = wide
 
         names = ["tokens", "tok_seq", "tok_pos", "seq_slot", "seq_start", "seq_new", "cu", "want_rows"]
         parts = [getattr(host, n) for n in names] + [t.reshape(-1) for t in self.host_tables]
@@ -80,8 +91,13 @@ class StepContext:
         packed = np.zeros(max(total, 4), dtype=np.int32)
         for off, p in zip(offsets, parts):
             packed[off:off + p.shape[0]] = p
+        self.packed = packed
+        if into is not None and not isinstance(into, torch.Tensor):
+            return                                   # host arrays only
         if staging is not None:
-            flat = staging.upload(packed)
+            flat = staging.upload(packed, into)
+        elif into is not None:
+            flat = into.copy_(torch.from_numpy(packed))
         else:
             flat = torch.from_numpy(packed).to(device)
         self.flat = flat
@@ -92,6 +108,11 @@ class StepContext:
         self._tables = {}
         for g, off, t in zip(self.groups, offsets[len(names):], self.host_tables):
             self._tables[id(g)] = flat[off:off + t.size].view(t.shape)
+
+    def shape_key(self):
+        """What fixes the layout of the device arrays (and so what a captured graph of the
+        step depends on): numbers of tokens, sequences and wanted rows, table widths."""
+        return (self.n_tokens, self.n_seqs, int(self.host.want_rows.shape[0]), tuple(t.shape[1] for t in self.host_tables))
 
     def page_table(self, group):
         """[sequences of the step, width] int32 page ids of a cache group, on the device."""

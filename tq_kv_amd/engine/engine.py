@@ -17,17 +17,28 @@ class StepError(ValueError):
     pass
 
 
+_NoUpload = object()       # StepContext(into=_NoUpload): build the host arrays only
+
+
 class Engine:
     """model: a loaded Model.  max_tokens: positions live sequences may hold together,
     each sequence counted up to a multiple of 64.  max_slots: most live sequences."""
 
-    def __init__(self, model, max_tokens, max_slots=256):
+    GRAPH_WIDTH_STEP = 8       # page-table widths of graphed steps grow in steps of 8 pages
+    MAX_GRAPHS = 32
+
+    def __init__(self, model, max_tokens, max_slots=256, use_graphs=True):
         self.model = model
         self.max_tokens = int(max_tokens)
         self.cache = Cache(model.needs, model.cache_of, self.max_tokens, max_slots, model.dtype, model.device)
         self.staging = HostStaging(model.device) if model.device.type == "cuda" else None
         self.vocab_size = model.spec.vocab_size
         self.max_positions = model.spec.max_positions
+        # Steps of one token per sequence are captured as HIP graphs and replayed: the step
+        # is some hundred short kernels, and launching them one by one from the host would
+        # cost more than running them.  Only if every part says its forward can be captured.
+        self.use_graphs = bool(use_graphs) and model.device.type == "cuda" and model.graph_safe
+        self.graphs = {}
 
     # -- sequences --------------------------------------------------------
     def open(self):
@@ -42,10 +53,12 @@ class Engine:
         return self.cache.length(slot)
 
     # -- the step ---------------------------------------------------------
-    def step(self, items):
+    def step(self, items, borrow=False):
         """items: [(slot, tokens, want)].  tokens: the sequence's next tokens (at least one);
         want: indices among them whose logits are wanted (may be empty).  Returns float32
-        logits [sum of len(want), vocab] in the order of items and of want."""
+        logits [sum of len(want), vocab] in the order of items and of want.  borrow: the
+        caller is done with the logits before the next step (they may live in a buffer that
+        the next step writes again)."""
         if not items:
             raise StepError("a step needs at least one sequence")
         seen = set()
@@ -63,8 +76,39 @@ class Engine:
                                 % (self.cache.length(slot) + len(tokens), self.max_positions))
         sizes = [(slot, len(tokens)) for slot, tokens, _ in items]
         self.cache.reserve(sizes)
-        ctx = StepContext([(slot, self.cache.length(slot), tokens) for slot, tokens, _ in items],
-                          [want for _, _, want in items], self.cache, self.model.device, self.staging)
-        logits = self.model.forward(ctx, self.cache)
+        ctx_items = [(slot, self.cache.length(slot), tokens) for slot, tokens, _ in items]
+        wants = [want for _, _, want in items]
+        if self.use_graphs and all(n == 1 for _, n in sizes) and len(items) <= self.model.graph_max_rows:
+            logits = self._graphed_step(ctx_items, wants)
+            if not borrow:
+                logits = logits.clone()
+        else:
+            ctx = StepContext(ctx_items, wants, self.cache, self.model.device, self.staging)
+            logits = self.model.forward(ctx, self.cache)
         self.cache.commit(sizes)
         return logits
+
+    def _graphed_step(self, ctx_items, wants):
+        """A step of one token per sequence through a captured graph.  The graph reads the
+        step's arrays (tokens, positions, page tables) from one device buffer that is
+        overwritten before every replay; its kernels take every size from those arrays or
+        from the shapes the graph was captured for."""
+        probe = StepContext(ctx_items, wants, self.cache, None, None, self.GRAPH_WIDTH_STEP, into=_NoUpload)
+        key = probe.shape_key()
+        entry = self.graphs.get(key)
+        if entry is None:
+            ctx = StepContext(ctx_items, wants, self.cache, self.model.device, self.staging, self.GRAPH_WIDTH_STEP)
+            logits = self.model.forward(ctx, self.cache)          # this step's work, and the warm-up
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_logits = self.model.forward(ctx, self.cache)
+            if len(self.graphs) >= self.MAX_GRAPHS:
+                self.graphs.pop(next(iter(self.graphs)))
+            self.graphs[key] = (graph, ctx, static_logits)
+            return logits
+        graph, ctx, static_logits = entry
+        self.graphs[key] = self.graphs.pop(key)                     # most recently used last
+        self.staging.upload(probe.packed, into=ctx.flat)
+        graph.replay()
+        return static_logits

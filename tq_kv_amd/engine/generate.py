@@ -74,6 +74,7 @@ def generate(engine, prompts, params=None, eos_ids=(), on_tokens=None, max_batch
 
 def _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, sampler):
     slots = {}
+    borrow = {"borrow": True} if getattr(engine, "use_graphs", False) else {}
     try:
         for r in batch:
             slots[r] = engine.open()
@@ -99,7 +100,7 @@ def _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, sampler)
             live = feed
             if not live:
                 break
-            logits = engine.step([(slots[batch[b]], [drawn[b]], [0]) for b in live])
+            logits = engine.step([(slots[batch[b]], [drawn[b]], [0]) for b in live], **borrow)
             drawn = dict(zip(live, sampler.sample(logits, live)))
     finally:
         for slot in slots.values():

@@ -43,6 +43,11 @@ class Model:
         self.embedding = None
         self.head = None
         self.loaded = False
+        # a step can be captured as a graph if every part's forward launches the same kernels
+        # whatever the step's data are; steps of more rows than the skinny products take
+        # would bring library calls into the graph and are run directly
+        self.graph_safe = all(getattr(b, "graph_safe", False) for b in self.blocks) and getattr(self.final_norm, "graph_safe", False)
+        self.graph_max_rows = 64
 
     # -- tensors ----------------------------------------------------------
     def tensor_specs(self):

@@ -24,6 +24,7 @@ class Attention(Part):
 
     def __init__(self, params, env):
         self.env = env
+        self.graph_safe = True
         self.hidden = int(params["hidden"])
         self.n_heads = int(params["n_heads"])
         self.n_kv_heads = int(params["n_kv_heads"])
@@ -42,6 +43,7 @@ class Attention(Part):
         if key not in env.shared:
             env.shared[key] = env.build("position", spec)
         self.position = env.shared[key]
+        self.graph_safe = not hasattr(self.position, "apply") or getattr(self.position, "graph_safe", False)
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
 
     def tensors(self):

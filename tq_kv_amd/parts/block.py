@@ -38,6 +38,7 @@ class PreNormBlock(Part):
         self.ff_norm = self.parts["ff_norm"]
         self.post_mixer_norm = self.parts.get("post_mixer_norm")
         self.post_ff_norm = self.parts.get("post_ff_norm")
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in self.parts.values())
 
     def tensors(self):
         out = {}

@@ -11,6 +11,7 @@ from .spec import TensorSpec
 @register("feed_forward", "gated_silu")
 class GatedSiLU(Part):
     """params: hidden, inter."""
+    graph_safe = True
 
     def __init__(self, params, env):
         self.hidden = int(params["hidden"])

@@ -11,6 +11,7 @@ from .spec import TensorSpec
 @register("norm", "rms_norm")
 class RMSNorm(Part):
     """params: size, eps."""
+    graph_safe = True
 
     def __init__(self, params, env):
         self.size = int(params["size"])

@@ -62,6 +62,10 @@ class Part:
     """Base of every part."""
     category = None
     kind = None
+    # True if forward() launches the same kernels with the same arguments whatever the
+    # step's data are (it reads positions, tables and slots on the device only), so that a
+    # step can be captured once as a graph and replayed.
+    graph_safe = False
 
     def tensors(self):
         """name (relative to the part's prefix) -> TensorSpec"""
