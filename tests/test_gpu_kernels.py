@@ -411,3 +411,48 @@ def test_attention_decode_refuses_other_head_sizes():
     with pytest.raises(K.KernelError, match="head_dim 48"):
         K.attention_decode(rand(1, 1, 48, dtype=torch.bfloat16), keys, values, ints([0]), ints([[0]]), 0, 1.0,
                            torch.empty(1, 48, dtype=torch.bfloat16, device=DEV))
+
+
+@pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (3, 1, 96)])
+@pytest.mark.parametrize("window", [0, 70, 12])
+def test_attention_prefill(nh, nkv, d, window):
+    # sequence 0: 150 new queries at positions 150..299 behind 150 cached ones; sequence 1: a
+    # whole prompt of 70; sequence 2: one token at position 0.  Pages scrambled, unread places NaN.
+    spans = [(150, 300), (0, 70), (0, 1)]
+    n_pages = 12
+    keys, values = make_cache(n_pages, nkv, d, torch.bfloat16)
+    tables = [[7, 2, 9, 0, 5], [4, 10, -1, -1, -1], [11, -1, -1, -1, -1]]
+    ks, vs, qs = [], [], []
+    for i, (a, b) in enumerate(spans):
+        k, v = rand(nkv, b, d, seed=70 + i).cpu(), rand(nkv, b, d, seed=80 + i).cpu()
+        qq = rand(b - a, nh, d, seed=90 + i).cpu()
+        if i == 0:
+            k[:, :, 0] *= 0.01
+            k[:, 3, 0], k[:, 230, 0], k[:, 229, 0] = 9.0, 8.0, 8.5     # far key; edge of the window of 70 for 299; outside
+            qq[-1] = 0.0
+            qq[-1, :, 0] = 30.0
+        k, v = k.to(torch.bfloat16).float(), v.to(torch.bfloat16).float()
+        kk, vv = paged(k, v, tables[i], n_pages, torch.bfloat16)
+        for p in tables[i]:
+            if p >= 0:
+                keys[p], values[p] = kk[p], vv[p]
+        ks.append(k), vs.append(v), qs.append(qq.to(torch.bfloat16))
+    q = torch.cat(qs).to(DEV)
+    pos = torch.cat([torch.arange(a, b) for a, b in spans])
+    tile_seq, tile_tok0, tile_count, off = [], [], [], 0
+    for i, (a, b) in enumerate(spans):
+        for s0 in range(0, b - a, 64):
+            tile_seq.append(i), tile_tok0.append(off + s0), tile_count.append(min(64, b - a - s0))
+        off += b - a
+    out = torch.empty(q.shape[0], nh * d, dtype=torch.bfloat16, device=DEV)
+    scale = 1 / math.sqrt(d)
+    K.attention_prefill(q, keys, values, pos.to(torch.int32).to(DEV), ints(tables), ints(tile_seq), ints(tile_tok0),
+                        ints(tile_count), ints([a for a, _ in spans]), ints([b - a for a, b in spans]), window, scale, out)
+    off = 0
+    for i, (a, b) in enumerate(spans):
+        want = attention_reference(qs[i].float(), ks[i], vs[i], torch.arange(a, b), window, scale)
+        torch.testing.assert_close(out[off:off + b - a].float().cpu(), want, atol=2e-2, rtol=2e-2)
+        off += b - a
+    if window != 70:
+        other = attention_reference(qs[0][-1:].float(), ks[0], vs[0], torch.tensor([299]), 70, scale)
+        assert (other - out[149:150].float().cpu()).abs().max() > 0.1

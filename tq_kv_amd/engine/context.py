@@ -11,6 +11,9 @@ import numpy as np
 import torch
 
 
+TILE = 64      # queries per tile of the prompt attention kernel
+
+
 class _Arrays:
     pass
 
@@ -67,6 +70,16 @@ class StepContext:
                     raise IndexError("wanted place %d is outside the %d tokens of sequence %d" % (j, lens[i], i))
                 rows.append(int(host.cu[i]) + int(j))
         host.want_rows = np.asarray(rows, dtype=np.int32)
+        # tiles of up to TILE consecutive queries of one sequence, for the prompt attention kernel
+        t_seq, t_tok0, t_count = [], [], []
+        for i, n in enumerate(lens):
+            for a in range(0, n, TILE):
+                t_seq.append(i)
+                t_tok0.append(int(host.cu[i]) + a)
+                t_count.append(min(TILE, n - a))
+        host.tile_seq = np.asarray(t_seq, dtype=np.int32)
+        host.tile_tok0 = np.asarray(t_tok0, dtype=np.int32)
+        host.tile_count = np.asarray(t_count, dtype=np.int32)
         self.host = host
         self.all_decode = all(n == 1 for n in lens)
         self.max_new = max(lens)
@@ -82,7 +95,8 @@ class StepContext:
                 wide[:, :t.shape[1]] = t
                 self.host_tables[i] = wide
 
-        names = ["tokens", "tok_seq", "tok_pos", "seq_slot", "seq_start", "seq_new", "cu", "want_rows"]
+        names = ["tokens", "tok_seq", "tok_pos", "seq_slot", "seq_start", "seq_new", "cu", "want_rows",
+                 "tile_seq", "tile_tok0", "tile_count"]
         parts = [getattr(host, n) for n in names] + [t.reshape(-1) for t in self.host_tables]
         offsets, total = [], 0
         for p in parts:

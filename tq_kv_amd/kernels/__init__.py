@@ -248,3 +248,27 @@ def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, t
         _dev(out, "out", torch.bfloat16, (n, n_heads * head_dim)), n_heads, n_kv_heads, head_dim, _stream()),
         "attention_decode")
     return out
+
+
+def attention_prefill_supported(head_dim):
+    return bool(library().tqk_attention_prefill_supported(int(head_dim)))
+
+
+def attention_prefill(q, keys, values, tok_pos, page_table, tile_seq, tile_tok0, tile_count, seq_start, seq_new,
+                      window, scale, out):
+    """Causal attention of tiles of up to 64 consecutive queries (q [T, heads, d] bfloat16)
+    over the paged cache; out [T, heads*d]."""
+    n, n_heads, head_dim = q.shape
+    n_pages, n_kv_heads = keys.shape[0], keys.shape[1]
+    n_seqs, width = page_table.shape
+    n_tiles = tile_seq.shape[0]
+    _check(library().tqk_attention_prefill(
+        _dev(q, "q", torch.bfloat16), _dev(keys, "keys", torch.bfloat16, (n_pages, n_kv_heads, 64, head_dim)),
+        _dev(values, "values", torch.bfloat16, (n_pages, n_kv_heads, head_dim, 64)),
+        _dev(tok_pos, "tok_pos", torch.int32, (n,)), _dev(page_table, "page_table", torch.int32), width, n_seqs, n_pages,
+        _dev(tile_seq, "tile_seq", torch.int32, (n_tiles,)), _dev(tile_tok0, "tile_tok0", torch.int32, (n_tiles,)),
+        _dev(tile_count, "tile_count", torch.int32, (n_tiles,)), n_tiles,
+        _dev(seq_start, "seq_start", torch.int32, (n_seqs,)), _dev(seq_new, "seq_new", torch.int32, (n_seqs,)),
+        int(window or 0), ctypes.c_float(scale), _dev(out, "out", torch.bfloat16, (n, n_heads * head_dim)),
+        n, n_heads, n_kv_heads, head_dim, _stream()), "attention_prefill")
+    return out

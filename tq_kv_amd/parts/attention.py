@@ -104,8 +104,13 @@ def attend(q, entry, table, ctx, window, scale, out):
     """Softmax attention of q over the cache entry: picks the kernel for the step.
 
     float32, or a head size the MFMA kernels do not take: the plain kernel, one wave per
-    (token, head).  bfloat16 and one token per sequence: the partitioned decoding kernel."""
+    (token, head).  bfloat16 and one token per sequence: the partitioned decoding kernel;
+    bfloat16 otherwise: the tiled prompt kernel."""
     head_dim = q.shape[2]
     if q.dtype == torch.bfloat16 and ctx.all_decode and POLICY["decode_mfma"] and K.attention_decode_supported(head_dim):
         return K.attention_decode(q, entry.keys, entry.values, ctx.dev.tok_pos, table, window, scale, out)
+    if q.dtype == torch.bfloat16 and POLICY["prefill_mfma"] and K.attention_prefill_supported(head_dim):
+        d = ctx.dev
+        return K.attention_prefill(q, entry.keys, entry.values, d.tok_pos, table, d.tile_seq, d.tile_tok0, d.tile_count,
+                                   d.seq_start, d.seq_new, window, scale, out)
     return K.attention(q, entry.keys, entry.values, ctx.dev.tok_seq, ctx.dev.tok_pos, table, window, scale, out)
