@@ -46,7 +46,7 @@ def test_embed(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("hidden", [72, 1000, 3584])
+@pytest.mark.parametrize("hidden", [70, 72, 1000, 3584, 9000])
 def test_add_rmsnorm(dtype, hidden):
     act = DT[dtype]
     h = rand(7, hidden, seed=2, scale=2.0)
@@ -99,6 +99,15 @@ def test_gemm_generic_rows_do_not_depend_on_the_batch():
     assert torch.equal(one[0], full[41])
 
 
+def value_place(p):
+    """Where position p of a page lies in a row of values: inside each 32 positions, the 4
+    positions 4g..4g+3 of the first 16 are followed by 16+4g..16+4g+3 of the second 16."""
+    return (p & 32) | (((p >> 2) & 3) << 3) | (((p >> 4) & 1) << 2) | (p & 3)
+
+
+PLACES = [value_place(p) for p in range(64)]
+
+
 def make_cache(n_pages, nkv, d, dtype):
     nan = float("nan")
     # keys [pages, kv heads, 64, d]; values are kept transposed inside a page
@@ -148,15 +157,17 @@ def test_rope_store(dtype, style, rot):
     want_v = x[:, (nh + nkv) * d:].reshape(5, nkv, d)
     torch.testing.assert_close(q.float().cpu(), want_q, **TOL[dtype])
     written = torch.zeros(n_pages, 64, dtype=torch.bool)
+    written_v = torch.zeros(n_pages, 64, dtype=torch.bool)
     for t in range(5):
         page = table.cpu()[tok_seq[t].item(), pos[t].item() // 64].item()
         slot = pos[t].item() % 64
         written[page, slot] = True
+        written_v[page, value_place(slot)] = True
         torch.testing.assert_close(keys[page, :, slot].float().cpu(), want_k[t], **TOL[dtype])
-        torch.testing.assert_close(values[page, :, :, slot].float().cpu(), want_v[t], **TOL[dtype])
+        torch.testing.assert_close(values[page, :, :, value_place(slot)].float().cpu(), want_v[t], **TOL[dtype])
     # nothing else was touched
     assert torch.isnan(keys.float().cpu().transpose(1, 2)[~written]).all()
-    assert torch.isnan(values.float().cpu().permute(0, 3, 1, 2)[~written]).all()
+    assert torch.isnan(values.float().cpu().permute(0, 3, 1, 2)[~written_v]).all()
     # a run that reads another run's cache writes none
     keys2, values2 = make_cache(n_pages, nkv, d, act)
     K.rope_store(qkv, bias, cos, sin, rot, code, tok_seq, tok_pos, table, keys2, values2, q, nh, nkv, d, write_kv=False)
@@ -172,7 +183,7 @@ def paged(k, v, page_ids, n_pages, dtype):
         n = min(64, s - 64 * i)
         if p >= 0 and n > 0:
             keys[p, :, :n] = k[:, 64 * i:64 * i + n].to(dtype)
-            values[p, :, :, :n] = v[:, 64 * i:64 * i + n].transpose(1, 2).to(dtype)
+            values[p][:, :, PLACES[:n]] = v[:, 64 * i:64 * i + n].transpose(1, 2).to(dtype).to(DEV)
     return keys, values
 
 
@@ -366,8 +377,8 @@ def test_skinny_refuses_what_it_does_not_take():
 
 @pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (3, 1, 96), (40, 2, 64), (4, 1, 256)])
 @pytest.mark.parametrize("window", [0, 70])
-@pytest.mark.parametrize("target_waves", [1, 64, 100000])
-def test_attention_decode(nh, nkv, d, window, target_waves):
+@pytest.mark.parametrize("target_blocks", [1, 24, 100000])
+def test_attention_decode(nh, nkv, d, window, target_blocks):
     # three sequences of lengths 300, 64 and 1, pages scrambled, everything unread is NaN
     lens = [300, 64, 1]
     n_pages = 12
@@ -393,7 +404,7 @@ def test_attention_decode(nh, nkv, d, window, target_waves):
     out = torch.empty(3, nh * d, dtype=torch.bfloat16, device=DEV)
     scale = 1 / math.sqrt(d)
     K.attention_decode(q.to(DEV), keys, values, pos.to(torch.int32).to(DEV), ints(tables), window, scale, out,
-                       target_waves=target_waves)
+                       target_blocks=target_blocks)
     for i in range(3):
         want = attention_reference(q[i:i + 1].float(), ks[i], vs[i], pos[i:i + 1], window, scale)
         torch.testing.assert_close(out[i:i + 1].float().cpu(), want, atol=2e-2, rtol=2e-2)

@@ -1,10 +1,14 @@
 // Attention for decoding: one new token per sequence attends over its sequence's pages
 // of the cache.  bfloat16 in, MFMA, float32 softmax.  Bound by the bytes of keys and
-// values, so the work is cut for memory: one wave per (sequence, kv head, partition of
-// the positions); all query heads that share the kv head ride in the same wave, so the
-// keys and values are read once for the whole group (the reference expands them per
-// query head instead, src/models/turbo_generic.rs:195-204, 1620-1621).  A second kernel
-// merges the partitions.  Formulas as src/models/turbo_generic.rs:1622-1631, :56-62.
+// values, so the work is cut for memory: a block of 4 waves per (sequence, kv head,
+// partition of the pages), each wave taking every fourth page of the partition; all
+// query heads that share the kv head ride in the same wave, so keys and values are
+// read once for the whole group (the reference expands them per query head instead,
+// src/models/turbo_generic.rs:195-204, 1620-1621).  The waves' results are merged
+// through LDS; with one partition the block writes the result itself, with more a
+// second kernel merges the partitions in their order.  (Merging in the last block to
+// finish, behind a device-wide fence, was measured to cost more than the second launch.)
+// Formulas as src/models/turbo_generic.rs:1622-1631, :56-62.
 //
 // Matrix-core mapping (v_mfma_f32_16x16x32_bf16, D[16x16] += A[16x32] B[32x16]):
 //   scores^T[key][head] = K[key][:] . Q^T[:][head]
@@ -15,33 +19,37 @@
 //       B needs for head l%16 eight keys per lane: the lane already holds them, the four
 //       of one group of 16 keys and the four of the next (slot j<4: key 4g+j, j>=4: key
 //       16+4g+j-4), so P never leaves its registers.  A must pair the same keys with the
-//       slots: values are stored transposed in a page ([head_dim][64 positions]), so the
-//       four keys of a slot group are 8 contiguous bytes of an element's row.
+//       slots: the cache keeps values transposed and in exactly this order inside a page
+//       (value_place in common.h), 16 contiguous bytes per lane.
 // Keys outside [lo, pos] get probability exactly 0 and their values are replaced by 0
 // before the product, so nothing stored at such places can reach the result.
 #include "common.h"
 #include "tq_kernels.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
-typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
 
 union pack8 {
     bf16x8_t v;
-    bf16x4_t h[2];
     uint16_t u[8];
+    uint4 q;
 };
 
+#define AD_WAVES 4
+
 template <int D>
-__global__ __launch_bounds__(TQK_WAVE)
+__global__ __launch_bounds__(AD_WAVES * TQK_WAVE)
 void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ keys,
                              const bf16_t* __restrict__ values, const int32_t* __restrict__ tok_pos,
                              const int32_t* __restrict__ page_table, int table_width, int window, float scale,
                              int pages_per_part, int n_parts, int n_heads, int n_kv_heads, int q_blocks,
-                             float* __restrict__ part_out, float* __restrict__ part_ml) {
+                             float* __restrict__ part_out, float* __restrict__ part_ml,
+                             bf16_t* __restrict__ out) {
     constexpr int KB = D / 32;          // k-blocks of the score product
     constexpr int DB = D / 16;          // 16-element blocks of the output
-    const int lane = threadIdx.x;
+    constexpr int ROW = DB * 4 + 2;     // floats a lane hands over: its out^T values, m, l
+    __shared__ float xch[(AD_WAVES - 1) * TQK_WAVE * ROW];
+    const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
     const int col = lane % 16, g = lane / 16;
     const int part = blockIdx.x;
     const int kvh = blockIdx.y / q_blocks, qb = blockIdx.y % q_blocks;
@@ -64,10 +72,9 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 #pragma unroll
     for (int i = 0; i < DB; ++i) o[i] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    if (start_page <= last_page) {
+    if (start_page + wave <= last_page) {
         pack8 zero;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) zero.u[i] = 0;
+        zero.q = make_uint4(0, 0, 0, 0);
         // the heads' queries: B operand of the score product
         bf16x8_t bq[KB];
         const bf16_t* qrow = q + ((size_t)seq * n_heads + head) * D + g * 8;
@@ -77,7 +84,7 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 
         const int32_t* pages = page_table + (size_t)seq * table_width;
         const size_t page_stride = (size_t)n_kv_heads * TQK_PAGE * D;
-        for (int pg = start_page; pg <= last_page; ++pg) {
+        for (int pg = start_page + wave; pg <= last_page; pg += AD_WAVES) {
             const int page = pages[pg];
             if (page < 0) continue;                     // the host never lets this happen
             const bf16_t* kp = keys + (size_t)page * page_stride + (size_t)kvh * TQK_PAGE * D;
@@ -85,17 +92,27 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
             const int key0 = pg * TQK_PAGE;
             const bool edge = key0 < lo || key0 + TQK_PAGE - 1 > pos;
 
+            // all of the page's loads first, so that they are in flight together
+            bf16x8_t ka[4][KB], va[DB][2];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+                    ka[t][kb] = *reinterpret_cast<const bf16x8_t*>(kp + (size_t)(t * 16 + col) * D + kb * 32 + g * 8);
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int pr = 0; pr < 2; ++pr)
+                    va[db][pr] = *reinterpret_cast<const bf16x8_t*>(vp + (size_t)(db * 16 + col) * TQK_PAGE + pr * 32 + g * 8);
+
             // scores^T for the page's four groups of 16 keys
             floatx4_t s[4];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-                const bf16_t* krow = kp + (size_t)(t * 16 + col) * D + g * 8;
 #pragma unroll
-                for (int kb = 0; kb < KB; ++kb) {
-                    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(krow + kb * 32);
-                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq[kb], s[t], 0, 0, 0);
-                }
+                for (int kb = 0; kb < KB; ++kb)
+                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[t][kb], bq[kb], s[t], 0, 0, 0);
             }
             // mask, scale, running maximum (the lane's head is its column; its keys are
             // key0 + 16 t + 4 g + r)
@@ -130,12 +147,10 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 o[db][0] *= alpha; o[db][1] *= alpha; o[db][2] *= alpha; o[db][3] *= alpha;
-                const bf16_t* vrow = vp + (size_t)(db * 16 + col) * TQK_PAGE + g * 4;
 #pragma unroll
                 for (int pr = 0; pr < 2; ++pr) {
                     pack8 av;
-                    av.h[0] = *reinterpret_cast<const bf16x4_t*>(vrow + (2 * pr) * 16);
-                    av.h[1] = *reinterpret_cast<const bf16x4_t*>(vrow + (2 * pr + 1) * 16);
+                    av.v = va[db][pr];
                     if (edge) {
 #pragma unroll
                         for (int i = 0; i < 8; ++i) {
@@ -151,15 +166,49 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
         l += __shfl_xor(l, 32, TQK_WAVE);
     }
 
-    // partial result of this partition: out^T[element db*16 + 4g + r][head col]
-    if (head_live) {
-        const size_t row = ((size_t)seq * n_heads + head) * n_parts + part;
-        float* po = part_out + row * D;
+    // the waves' results into wave 0, in wave order
+    if (wave > 0) {
+        float* mine = xch + ((size_t)(wave - 1) * TQK_WAVE + lane) * ROW;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) po[db * 16 + g * 4 + r] = o[db][r];
-        if (g == 0) { part_ml[row * 2] = m; part_ml[row * 2 + 1] = l; }
+            for (int r = 0; r < 4; ++r) mine[db * 4 + r] = o[db][r];
+        mine[DB * 4] = m;
+        mine[DB * 4 + 1] = l;
+    }
+    __syncthreads();
+    const size_t row = ((size_t)seq * n_heads + head) * n_parts + part;
+    if (wave == 0) {
+        for (int w = 1; w < AD_WAVES; ++w) {
+            const float* theirs = xch + ((size_t)(w - 1) * TQK_WAVE + lane) * ROW;
+            const float m2 = theirs[DB * 4], l2 = theirs[DB * 4 + 1];
+            if (m2 == -INFINITY) continue;
+            const float mn = fmaxf(m, m2);
+            const float a1 = m == -INFINITY ? 0.f : expf(m - mn), a2 = expf(m2 - mn);
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[db][r] = o[db][r] * a1 + theirs[db * 4 + r] * a2;
+            l = l * a1 + l2 * a2;
+            m = mn;
+        }
+        if (!head_live) return;
+        if (n_parts == 1) {
+            // the only partition: this is the result, out[head, element db*16 + 4g + r]
+            bf16_t* po = out + ((size_t)seq * n_heads + head) * D;
+            const float inv = 1.f / l;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) po[db * 16 + g * 4 + r] = from_float<bf16_t>(o[db][r] * inv);
+        } else {
+            float* po = part_out + row * D;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) po[db * 16 + g * 4 + r] = o[db][r];
+            if (g == 0) { part_ml[row * 2] = m; part_ml[row * 2 + 1] = l; }
+        }
     }
 }
 
@@ -170,13 +219,14 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_out, const
     const float* ml = part_ml + row * n_parts * 2;
     float M = -INFINITY;
     for (int p = 0; p < n_parts; ++p) M = fmaxf(M, ml[p * 2]);
-    float denom = 0.f;
-    for (int p = 0; p < n_parts; ++p) denom += ml[p * 2] == -INFINITY ? 0.f : expf(ml[p * 2] - M) * ml[p * 2 + 1];
     for (int c = threadIdx.x; c < head_dim; c += blockDim.x) {
-        float acc = 0.f;
+        float acc = 0.f, denom = 0.f;
         for (int p = 0; p < n_parts; ++p) {
-            if (ml[p * 2] == -INFINITY) continue;
-            acc += expf(ml[p * 2] - M) * part_out[(row * n_parts + p) * head_dim + c];
+            const float mp = ml[p * 2];
+            if (mp == -INFINITY) continue;
+            const float wgt = expf(mp - M);
+            denom += wgt * ml[p * 2 + 1];
+            acc += wgt * part_out[(row * n_parts + p) * head_dim + c];
         }
         out[row * head_dim + c] = from_float<bf16_t>(acc / denom);
     }
@@ -190,7 +240,8 @@ extern "C" int tqk_attention_decode(const void* q, const void* keys, const void*
                                     const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window,
                                     float scale, int pages_per_part, int n_parts, void* part_out, void* part_ml,
                                     void* out, int n_heads, int n_kv_heads, int head_dim, void* stream) {
-    TQK_REQUIRE(q && keys && values && tok_pos && page_table && part_out && part_ml && out, "tqk_attention_decode: null pointer");
+    TQK_REQUIRE(q && keys && values && tok_pos && page_table && out, "tqk_attention_decode: null pointer");
+    TQK_REQUIRE(n_parts == 1 || (part_out && part_ml), "tqk_attention_decode: more than one partition needs part_out and part_ml");
     TQK_REQUIRE(n_seqs >= 0 && n_heads > 0 && n_kv_heads > 0, "tqk_attention_decode: bad sizes");
     TQK_REQUIRE(n_heads % n_kv_heads == 0, "tqk_attention_decode: %d heads are not a multiple of %d kv heads", n_heads, n_kv_heads);
     TQK_REQUIRE(tqk_attention_decode_supported(head_dim), "tqk_attention_decode: head_dim %d is not one of 32, 64, 96, 128, 256", head_dim);
@@ -198,14 +249,14 @@ extern "C" int tqk_attention_decode(const void* q, const void* keys, const void*
     TQK_REQUIRE(pages_per_part > 0 && n_parts > 0 && (long long)n_parts * pages_per_part >= table_width,
                 "tqk_attention_decode: %d partitions of %d pages do not cover %d pages", n_parts, pages_per_part, table_width);
     TQK_REQUIRE(window >= 0, "tqk_attention_decode: negative window");
-    TQK_REQUIRE(n_seqs <= 65535 && n_kv_heads * ((n_heads / n_kv_heads + 15) / 16) <= 65535, "tqk_attention_decode: grid too large");
+    const int q_blocks = (n_heads / n_kv_heads + 15) / 16;
+    TQK_REQUIRE(n_seqs <= 65535 && n_kv_heads * q_blocks <= 65535, "tqk_attention_decode: grid too large");
     if (n_seqs == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    const int q_blocks = (n_heads / n_kv_heads + 15) / 16;
     dim3 grid(n_parts, n_kv_heads * q_blocks, n_seqs);
-#define LAUNCH(DD) attention_decode_kernel<DD><<<grid, TQK_WAVE, 0, s>>>( \
+#define LAUNCH(DD) attention_decode_kernel<DD><<<grid, AD_WAVES * TQK_WAVE, 0, s>>>( \
         (const bf16_t*)q, (const bf16_t*)keys, (const bf16_t*)values, tok_pos, page_table, table_width, window, scale, \
-        pages_per_part, n_parts, n_heads, n_kv_heads, q_blocks, (float*)part_out, (float*)part_ml)
+        pages_per_part, n_parts, n_heads, n_kv_heads, q_blocks, (float*)part_out, (float*)part_ml, (bf16_t*)out)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;
@@ -215,6 +266,7 @@ extern "C" int tqk_attention_decode(const void* q, const void* keys, const void*
     }
 #undef LAUNCH
     if (tqk_check_launch("tqk_attention_decode")) return -1;
+    if (n_parts == 1) return 0;
     attention_merge_kernel<<<n_seqs * n_heads, head_dim >= 128 ? 128 : 64, 0, s>>>(
         (const float*)part_out, (const float*)part_ml, n_parts, head_dim, (bf16_t*)out);
     return tqk_check_launch("tqk_attention_decode merge");

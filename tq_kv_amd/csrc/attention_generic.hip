@@ -14,7 +14,8 @@
 // score of key j of the block, the softmax runs online over blocks, then lane c
 // accumulates output element c (+64, +128, ...) over the block's keys.  The order of
 // operations for a query depends only on its position, never on the batch.
-// Cache pages: keys [kv head][position][head_dim], values [kv head][head_dim][position].
+// Cache pages: keys [kv head][position][head_dim], values [kv head][head_dim][place of
+// the position] (value_place in common.h).
 #include "common.h"
 #include "tq_kernels.h"
 
@@ -79,7 +80,7 @@ void attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ key
             if (a * TQK_WAVE < head_dim) {
                 for (int jj = first_key; jj < n_keys; ++jj) {
                     const float pj = __shfl(p, jj, TQK_WAVE);
-                    if (c < head_dim) sum = fmaf(pj, to_float(vb[(size_t)c * TQK_PAGE + jj]), sum);
+                    if (c < head_dim) sum = fmaf(pj, to_float(vb[(size_t)c * TQK_PAGE + value_place(jj)]), sum);
                 }
             }
             acc[a] = sum;

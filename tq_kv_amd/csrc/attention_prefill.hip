@@ -14,8 +14,8 @@
 // Matrix-core mapping as in the decoding kernel: scores^T = K Q^T puts a query in a
 // lane's column and 4 keys of each group of 16 in its registers, which is exactly the
 // operand layout that out^T = V^T P^T needs, so the probabilities never move.
-// LDS rows are padded (keys by 8 elements, values by 8 positions) so that the 16 lanes
-// of a read phase fall into different banks.
+// LDS rows are padded (keys by 8 elements, values by 8 places) so that the lanes of a
+// read phase fall into different banks.
 #include "common.h"
 #include "tq_kernels.h"
 
@@ -117,7 +117,7 @@ void attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __rest
             if (tail) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
-                    if (key0 + vpart * 8 + i >= seq_end) v.u[i] = 0;      // nothing stored there may count
+                    if (key0 + value_position(vpart * 8 + i) >= seq_end) v.u[i] = 0;   // nothing stored there may count
             }
             *reinterpret_cast<uint4*>(&v_lds[vrow * VSTRIDE + vpart * 8]) = v.q;
         }
@@ -172,13 +172,12 @@ void attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __rest
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
             o[db][0] *= alpha; o[db][1] *= alpha; o[db][2] *= alpha; o[db][3] *= alpha;
-            const uint16_t* vrow = &v_lds[(db * 16 + col) * VSTRIDE + g * 4];
+            // the lane's 8 keys of each half page lie together (value_place)
+            const uint16_t* vrow = &v_lds[(db * 16 + col) * VSTRIDE + g * 8];
 #pragma unroll
             for (int pr = 0; pr < 2; ++pr) {
-                pf_pack8 av;
-                av.h[0] = *reinterpret_cast<const bf16x4_t*>(vrow + (2 * pr) * 16);
-                av.h[1] = *reinterpret_cast<const bf16x4_t*>(vrow + (2 * pr + 1) * 16);
-                o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av.v, pb[pr].v, o[db], 0, 0, 0);
+                const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(vrow + pr * 32);
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pb[pr].v, o[db], 0, 0, 0);
             }
         }
     }

@@ -25,6 +25,20 @@ template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { bf16_t r; r.bits = float_to_bf16_bits(v); return r; }
 
+// ---- places of values inside a page ---------------------------------------------
+// A page of values is [kv head][head_dim][64 places]: an element's values of the page's
+// 64 positions lie together, but not in order of position.  Position p (0..63) lies at
+// place value_place(p): inside each group of 32 positions, the 4 positions 4g..4g+3 of
+// the first 16 are followed by the 4 positions 16+4g..16+4g+3 of the second 16.  These
+// are the 8 keys one lane feeds to the matrix cores in the product P.V (see
+// attention_decode.hip), so a lane reads its 8 values as 16 contiguous bytes.
+__device__ __host__ __forceinline__ int value_place(int p) {
+    return (p & 32) | (((p >> 2) & 3) << 3) | (((p >> 4) & 1) << 2) | (p & 3);
+}
+__device__ __host__ __forceinline__ int value_position(int place) {
+    return (place & 32) | (((place >> 2) & 1) << 4) | (((place >> 3) & 3) << 2) | (place & 3);
+}
+
 // ---- reductions ---------------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

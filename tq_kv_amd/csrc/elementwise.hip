@@ -63,6 +63,67 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__
     }
 }
 
+// The same for rows of up to VPT * 4 * blockDim elements, a multiple of 4: every value is
+// read once, in vectors of 4, and stays in registers between the two passes.
+template <typename TA> struct Vec4;
+template <> struct Vec4<float> { float4 v; __device__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; } };
+template <> struct Vec4<bf16_t> { uint2 v; __device__ float get(int i) const {
+    const uint32_t word = i < 2 ? v.x : v.y;
+    return __uint_as_float((i & 1) ? (word & 0xffff0000u) : (word << 16)); } };
+
+template <typename T> __device__ __forceinline__ void store4(T* p, float a, float b, float c, float d);
+template <> __device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
+    *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+}
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float a, float b, float c, float d) {
+    uint2 o;
+    o.x = (uint32_t)float_to_bf16_bits(a) | ((uint32_t)float_to_bf16_bits(b) << 16);
+    o.y = (uint32_t)float_to_bf16_bits(c) | ((uint32_t)float_to_bf16_bits(d) << 16);
+    *reinterpret_cast<uint2*>(p) = o;
+}
+
+template <typename TA, typename TW, int VPT>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TA* __restrict__ delta,
+                                       const TW* __restrict__ weight, float eps,
+                                       const int32_t* __restrict__ rows, int hidden,
+                                       TA* __restrict__ out, int write_back) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t row = rows ? (size_t)rows[r] : (size_t)r;
+    float* hr = h ? h + row * hidden : nullptr;
+    const TA* dr = delta ? delta + row * hidden : nullptr;
+    TA* o = out + (size_t)r * hidden;
+    float v[VPT][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int i = (j * blockDim.x + threadIdx.x) * 4;
+        if (i < hidden) {
+            float4 hv = hr ? *reinterpret_cast<const float4*>(hr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (dr) {
+                Vec4<TA> d;
+                d.v = *reinterpret_cast<const decltype(d.v)*>(dr + i);
+                hv.x += d.get(0); hv.y += d.get(1); hv.z += d.get(2); hv.w += d.get(3);
+            }
+            if (write_back) *reinterpret_cast<float4*>(hr + i) = hv;
+            v[j][0] = hv.x; v[j][1] = hv.y; v[j][2] = hv.z; v[j][3] = hv.w;
+            ss += hv.x * hv.x + hv.y * hv.y + hv.z * hv.z + hv.w * hv.w;
+        }
+    }
+    const float total = block_sum(ss, scratch);
+    const float rms = sqrtf(total / (float)hidden + eps);
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int i = (j * blockDim.x + threadIdx.x) * 4;
+        if (i < hidden) {
+            Vec4<TW> w;
+            w.v = *reinterpret_cast<const decltype(w.v)*>(weight + i);
+            store4<TA>(o + i, (v[j][0] / rms) * w.get(0), (v[j][1] / rms) * w.get(1),
+                       (v[j][2] / rms) * w.get(2), (v[j][3] / rms) * w.get(3));
+        }
+    }
+}
+
 extern "C" int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const void* weight,
                                int weight_dtype, float eps, const int32_t* rows, int n_rows,
                                int hidden, void* out, int write_back, void* stream) {
@@ -70,16 +131,37 @@ extern "C" int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const
     TQK_REQUIRE(h || delta, "tqk_add_rmsnorm: neither h nor delta given");
     TQK_REQUIRE(!write_back || (h && !rows), "tqk_add_rmsnorm: write_back needs h and no row list");
     TQK_REQUIRE(n_rows >= 0 && hidden > 0, "tqk_add_rmsnorm: bad sizes rows=%d hidden=%d", n_rows, hidden);
+    TQK_REQUIRE(act_dtype == TQK_F32 || act_dtype == TQK_BF16, "tqk_add_rmsnorm: unknown activation dtype %d", act_dtype);
+    TQK_REQUIRE(weight_dtype == TQK_F32 || weight_dtype == TQK_BF16, "tqk_add_rmsnorm: unknown weight dtype %d", weight_dtype);
     if (n_rows == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    const bool aligned = ((((uintptr_t)h) | ((uintptr_t)delta) | ((uintptr_t)weight) | ((uintptr_t)out)) & 15) == 0;
+    const int code = act_dtype * 2 + weight_dtype;
+    if (hidden % 4 == 0 && hidden <= 8192 && aligned) {
+        const int threads = 256;
+#define LAUNCHV(TA, TW, VPT) add_rmsnorm_vec_kernel<TA, TW, VPT><<<n_rows, threads, 0, s>>>( \
+        h, (const TA*)delta, (const TW*)weight, eps, rows, hidden, (TA*)out, write_back)
+#define PICK(TA, TW) do { if (hidden <= 1024) LAUNCHV(TA, TW, 1); else if (hidden <= 2048) LAUNCHV(TA, TW, 2); \
+        else if (hidden <= 4096) LAUNCHV(TA, TW, 4); else LAUNCHV(TA, TW, 8); } while (0)
+        switch (code) {
+            case 0: PICK(float, float); break;
+            case 1: PICK(float, bf16_t); break;
+            case 2: PICK(bf16_t, float); break;
+            case 3: PICK(bf16_t, bf16_t); break;
+        }
+#undef PICK
+#undef LAUNCHV
+        return tqk_check_launch("tqk_add_rmsnorm");
+    }
     const int threads = hidden >= 2048 ? 512 : 256;
 #define LAUNCH(TA, TW) add_rmsnorm_kernel<TA, TW><<<n_rows, threads, 0, s>>>( \
         h, (const TA*)delta, (const TW*)weight, eps, rows, hidden, (TA*)out, write_back)
-    if (act_dtype == TQK_F32 && weight_dtype == TQK_F32) LAUNCH(float, float);
-    else if (act_dtype == TQK_F32 && weight_dtype == TQK_BF16) LAUNCH(float, bf16_t);
-    else if (act_dtype == TQK_BF16 && weight_dtype == TQK_F32) LAUNCH(bf16_t, float);
-    else if (act_dtype == TQK_BF16 && weight_dtype == TQK_BF16) LAUNCH(bf16_t, bf16_t);
-    else return tqk_fail("tqk_add_rmsnorm: unknown dtypes act=%d weight=%d", act_dtype, weight_dtype);
+    switch (code) {
+        case 0: LAUNCH(float, float); break;
+        case 1: LAUNCH(float, bf16_t); break;
+        case 2: LAUNCH(bf16_t, float); break;
+        case 3: LAUNCH(bf16_t, bf16_t); break;
+    }
 #undef LAUNCH
     return tqk_check_launch("tqk_add_rmsnorm");
 }
@@ -108,8 +190,8 @@ __global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restri
     const TB* b = bias ? bias + (size_t)head * head_dim : nullptr;
 
     // q rows and key rows are contiguous in head_dim; values are kept transposed inside a
-    // page, [kv head][head_dim][position in page], so that the matrix cores can read 8
-    // consecutive positions of one element as 16 contiguous bytes.
+    // page, [kv head][head_dim][place of the position], so that the matrix cores can read
+    // the 8 positions a lane needs of one element as 16 contiguous bytes.
     TA* dst;
     size_t dst_stride = 1;
     if (kind == 0) {
@@ -122,7 +204,7 @@ __global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restri
         if (kind == 1) {
             dst = keys + base + (size_t)(pos % TQK_PAGE) * head_dim;
         } else {
-            dst = values + base + (pos % TQK_PAGE);
+            dst = values + base + value_place(pos % TQK_PAGE);
             dst_stride = TQK_PAGE;
         }
     }

@@ -25,39 +25,70 @@
 #define SAMP_THREADS 1024
 
 // ---- argmax ----------------------------------------------------------------------
-__global__ __launch_bounds__(SAMP_THREADS)
-void argmax_kernel(const float* __restrict__ logits, int vocab, int32_t* __restrict__ out) {
-    __shared__ float best_v[SAMP_THREADS / TQK_WAVE];
-    __shared__ int best_i[SAMP_THREADS / TQK_WAVE];
-    const float* row = logits + (size_t)blockIdx.x * vocab;
-    float bv = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-        const float v = row[i];
-        if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }   // NaN compares false and is skipped
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(bv, o, TQK_WAVE);
-        const int oi = __shfl_xor(bi, o, TQK_WAVE);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
-    const int lane = threadIdx.x % TQK_WAVE, wave = threadIdx.x / TQK_WAVE;
-    if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w = 1; w < SAMP_THREADS / TQK_WAVE; ++w)
-            if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
-        out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
-    }
+// Two stages, so that a handful of rows still spread over the chip: blocks of 256 threads
+// each find the best of a chunk of a row, then one block per row finds the best chunk.
+// "Best" is the largest value, the lowest index among equals; NaN never wins.
+#define AM_CHUNK 4096
+#define AM_THREADS 256
+
+__device__ __forceinline__ void better(float& bv, int& bi, float ov, int oi) {
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
 }
 
-extern "C" int tqk_argmax(const float* logits, int n_rows, int vocab, int32_t* out, void* stream) {
-    TQK_REQUIRE(logits && out, "tqk_argmax: null pointer");
+__device__ __forceinline__ void block_best(float& bv, int& bi, float* sv, int* si) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) better(bv, bi, __shfl_xor(bv, o, TQK_WAVE), __shfl_xor(bi, o, TQK_WAVE));
+    const int lane = threadIdx.x % TQK_WAVE, wave = threadIdx.x / TQK_WAVE;
+    if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0)
+        for (int w = 1; w < (int)(blockDim.x / TQK_WAVE); ++w) better(bv, bi, sv[w], si[w]);
+}
+
+__global__ __launch_bounds__(AM_THREADS)
+void argmax_chunk_kernel(const float* __restrict__ logits, int vocab, int n_chunks,
+                         float* __restrict__ best_v, int32_t* __restrict__ best_i) {
+    __shared__ float sv[AM_THREADS / TQK_WAVE];
+    __shared__ int si[AM_THREADS / TQK_WAVE];
+    const float* row = logits + (size_t)blockIdx.y * vocab;
+    const int begin = blockIdx.x * AM_CHUNK, end = min(vocab, begin + AM_CHUNK);
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = begin + threadIdx.x; i < end; i += AM_THREADS) better(bv, bi, row[i], i);
+    block_best(bv, bi, sv, si);
+    if (threadIdx.x == 0) { best_v[(size_t)blockIdx.y * n_chunks + blockIdx.x] = bv; best_i[(size_t)blockIdx.y * n_chunks + blockIdx.x] = bi; }
+}
+
+__global__ __launch_bounds__(AM_THREADS)
+void argmax_final_kernel(const float* __restrict__ best_v, const int32_t* __restrict__ best_i, int n_chunks,
+                         int32_t* __restrict__ out) {
+    __shared__ float sv[AM_THREADS / TQK_WAVE];
+    __shared__ int si[AM_THREADS / TQK_WAVE];
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int c = threadIdx.x; c < n_chunks; c += AM_THREADS)
+        better(bv, bi, best_v[(size_t)blockIdx.x * n_chunks + c], best_i[(size_t)blockIdx.x * n_chunks + c]);
+    block_best(bv, bi, sv, si);
+    if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+}
+
+extern "C" int tqk_argmax_scratch_floats(int n_rows, int vocab) {
+    return 2 * n_rows * ((vocab + AM_CHUNK - 1) / AM_CHUNK);
+}
+
+extern "C" int tqk_argmax(const float* logits, int n_rows, int vocab, int32_t* out, float* scratch, void* stream) {
+    TQK_REQUIRE(logits && out && scratch, "tqk_argmax: null pointer");
     TQK_REQUIRE(n_rows >= 0 && vocab > 0, "tqk_argmax: bad sizes rows=%d vocab=%d", n_rows, vocab);
+    TQK_REQUIRE(n_rows <= 65535, "tqk_argmax: too many rows for the grid");
     if (n_rows == 0) return 0;
-    argmax_kernel<<<n_rows, SAMP_THREADS, 0, (hipStream_t)stream>>>(logits, vocab, out);
-    return tqk_check_launch("tqk_argmax");
+    const int n_chunks = (vocab + AM_CHUNK - 1) / AM_CHUNK;
+    float* best_v = scratch;
+    int32_t* best_i = reinterpret_cast<int32_t*>(scratch + (size_t)n_rows * n_chunks);
+    hipStream_t s = (hipStream_t)stream;
+    argmax_chunk_kernel<<<dim3(n_chunks, n_rows), AM_THREADS, 0, s>>>(logits, vocab, n_chunks, best_v, best_i);
+    if (tqk_check_launch("tqk_argmax")) return -1;
+    argmax_final_kernel<<<n_rows, AM_THREADS, 0, s>>>(best_v, best_i, n_chunks, out);
+    return tqk_check_launch("tqk_argmax final");
 }
 
 // ---- helpers for one-block-per-row passes ---------------------------------------

@@ -168,7 +168,8 @@ extern "C" int tqk_skinny_bf16(const void* x, const void* w, void* y, int y_dtyp
     TQK_REQUIRE(!epilogue || y_dtype == TQK_BF16, "tqk_skinny_bf16: the gated epilogue writes bfloat16");
     TQK_REQUIRE((((uintptr_t)x) & 15) == 0 && (((uintptr_t)w) & 15) == 0, "tqk_skinny_bf16: x and w must be 16-byte aligned");
     if (M == 0) return 0;
-    // waves per block: enough waves on the chip to keep HBM busy (a few thousand), no more
+    // waves per block: about a thousand waves on the chip keep HBM busy (measured: with more,
+    // each wave's share of K gets so short that start-up and the reduction dominate), no more
     // than there are chunks of K, a power of two, and such that four blocks of x rows fit the
     // LDS reduction.  M plays no part, so a row's sum has the same order in any batch.
     const int n_out = epilogue ? N / 2 : N;
@@ -176,7 +177,7 @@ extern "C" int tqk_skinny_bf16(const void* x, const void* w, void* y, int y_dtyp
     const int chunks = K / (SK_UNROLL * 32) > 0 ? K / (SK_UNROLL * 32) : 1;
     const int max_waves = epilogue ? 8 : 16;
     int waves = 1;
-    while (waves < max_waves && blocks * waves < 4096 && waves * 2 <= chunks) waves *= 2;
+    while (waves < max_waves && blocks * waves < 1024 && waves * 2 <= chunks) waves *= 2;
     hipStream_t s = (hipStream_t)stream;
     const int mb = (M + 15) / 16;
     switch (mb) {

@@ -45,7 +45,8 @@ int tqk_skinny_bf16(const void* x, const void* w, void* y, int y_dtype, int M, i
  * tok_pos[t] (style 0: none, 1: halves (j, j+rot/2), 2: pairs (2j, 2j+1)), write q to
  * q_out [tokens, heads, head_dim] and, if write_kv, k and v into the pages of the
  * token's sequence: keys [n_pages, kv_heads, 64, head_dim], values transposed inside a
- * page, [n_pages, kv_heads, head_dim, 64]. */
+ * page, [n_pages, kv_heads, head_dim, 64], position p of the page at place
+ * (p & 32) | ((p >> 2 & 3) << 3) | ((p >> 4 & 1) << 2) | (p & 3). */
 int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, int bias_dtype,
                    const float* cos_table, const float* sin_table, int rot_dim, int style,
                    int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
@@ -62,9 +63,10 @@ int tqk_attention(const void* q, const void* keys, const void* values, int act_d
                   int n_tokens, int n_heads, int n_kv_heads, int head_dim, void* stream);
 
 /* Decoding: sequence b's one new token (query row b, position tok_pos[b]) over its pages,
- * bfloat16, MFMA; the positions are cut into n_parts partitions of pages_per_part pages,
- * partial results go to part_out [seqs, heads, n_parts, head_dim] and part_ml
- * [seqs, heads, n_parts, 2] (float32) and are merged into out [seqs, heads*head_dim]. */
+ * bfloat16, MFMA; the pages are cut into n_parts partitions of pages_per_part pages.  With
+ * one partition the result goes straight to out [seqs, heads*head_dim]; with more, the
+ * partitions' results go to part_out [seqs, heads, n_parts, head_dim] and part_ml [seqs,
+ * heads, n_parts, 2] (float32) and a second kernel merges them into out. */
 int tqk_attention_decode_supported(int head_dim);
 int tqk_attention_decode(const void* q, const void* keys, const void* values, const int32_t* tok_pos,
                          const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window,
@@ -86,8 +88,10 @@ int tqk_attention_prefill(const void* q, const void* keys, const void* values, c
 /* out[t, i] = silu(gate_up[t, i]) * gate_up[t, inter + i] */
 int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, void* stream);
 
-/* out[r] = lowest index of the largest value of logits[r, :] */
-int tqk_argmax(const float* logits, int n_rows, int vocab, int32_t* out, void* stream);
+/* out[r] = lowest index of the largest value of logits[r, :]; scratch: at least
+ * tqk_argmax_scratch_floats(n_rows, vocab) floats of device memory. */
+int tqk_argmax_scratch_floats(int n_rows, int vocab);
+int tqk_argmax(const float* logits, int n_rows, int vocab, int32_t* out, float* scratch, void* stream);
 
 /* For every generated token of the row's request, once per occurrence:
  * l > 0 ? l / penalty : l * penalty.  hist [n_req, hist_cap], hist_len [n_req]. */

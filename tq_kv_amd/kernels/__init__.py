@@ -169,8 +169,9 @@ def swiglu(gate_up, out):
 def argmax(logits, out):
     """out[r] = lowest index of the largest value of row r; logits [R,V] float32, out [R] int32."""
     rows, vocab = logits.shape
+    scratch = torch.empty((library().tqk_argmax_scratch_floats(rows, vocab),), dtype=torch.float32, device=logits.device)
     _check(library().tqk_argmax(_dev(logits, "logits", torch.float32), rows, vocab,
-                                _dev(out, "out", torch.int32, (rows,)), _stream()), "argmax")
+                                _dev(out, "out", torch.int32, (rows,)), _dev(scratch, "scratch"), _stream()), "argmax")
     return out
 
 
@@ -226,7 +227,7 @@ def attention_decode_supported(head_dim):
     return bool(library().tqk_attention_decode_supported(int(head_dim)))
 
 
-def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, target_waves=2048):
+def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, target_blocks=512):
     """Attention of one new token per sequence (q [B, heads, d] bfloat16, row b belongs to
     sequence b at position tok_pos[b]) over the paged cache; out [B, heads*d]."""
     n, n_heads, head_dim = q.shape
@@ -235,16 +236,19 @@ def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, t
     if n_seqs != n:
         raise KernelError("attention_decode: %d query rows for %d sequences (one token each is required)" % (n, n_seqs))
     q_blocks = (n_heads // n_kv_heads + 15) // 16
-    want_parts = max(1, min(width, target_waves // max(1, n * n_kv_heads * q_blocks)))
+    groups = max(1, n * n_kv_heads * q_blocks)
+    want_parts = max(1, min(width, (target_blocks + groups - 1) // groups))
     per_part = (width + want_parts - 1) // want_parts
     n_parts = (width + per_part - 1) // per_part
-    part_out = torch.empty((n, n_heads, n_parts, head_dim), dtype=torch.float32, device=q.device)
-    part_ml = torch.empty((n, n_heads, n_parts, 2), dtype=torch.float32, device=q.device)
+    part_out = part_ml = None
+    if n_parts > 1:
+        part_out = torch.empty((n, n_heads, n_parts, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n, n_heads, n_parts, 2), dtype=torch.float32, device=q.device)
     _check(library().tqk_attention_decode(
         _dev(q, "q", torch.bfloat16), _dev(keys, "keys", torch.bfloat16, (n_pages, n_kv_heads, 64, head_dim)),
         _dev(values, "values", torch.bfloat16, (n_pages, n_kv_heads, head_dim, 64)),
         _dev(tok_pos, "tok_pos", torch.int32, (n,)), _dev(page_table, "page_table", torch.int32), width, n, n_pages,
-        int(window or 0), ctypes.c_float(scale), per_part, n_parts, _dev(part_out, "part_out"), _dev(part_ml, "part_ml"),
+        int(window or 0), ctypes.c_float(scale), per_part, n_parts, _opt(part_out, "part_out"), _opt(part_ml, "part_ml"),
         _dev(out, "out", torch.bfloat16, (n, n_heads * head_dim)), n_heads, n_kv_heads, head_dim, _stream()),
         "attention_decode")
     return out
