@@ -349,11 +349,16 @@ def test_skinny_product(m, n, k):
     out16 = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
     K.skinny_bf16(x, w, out16)
     assert torch.equal(out16, out.to(torch.bfloat16))
-    # a row's result does not depend on the other rows
-    if m > 1:
+    # a row's result does not depend on the other rows (the kernel has one order of summation
+    # for up to 16 rows and one for more)
+    if 1 < m <= 16:
         one = torch.empty(1, n, device=DEV)
         K.skinny_bf16(x[m - 1:].contiguous(), w, one)
         assert torch.equal(one[0], out[m - 1])
+    if m > 17:
+        few = torch.empty(17, n, device=DEV)
+        K.skinny_bf16(x[m - 17:].contiguous(), w, few)
+        assert torch.equal(few[16], out[m - 1])
 
 
 @pytest.mark.parametrize("m", [1, 8, 40, 64])

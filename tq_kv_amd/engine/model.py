@@ -47,7 +47,7 @@ class Model:
         # whatever the step's data are; steps of more rows than the skinny products take
         # would bring library calls into the graph and are run directly
         self.graph_safe = all(getattr(b, "graph_safe", False) for b in self.blocks) and getattr(self.final_norm, "graph_safe", False)
-        self.graph_max_rows = 64
+        self.graph_max_rows = 16
 
     # -- tensors ----------------------------------------------------------
     def tensor_specs(self):
