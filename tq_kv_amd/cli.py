@@ -5,6 +5,7 @@ option names and defaults as there where they exist.
     tq bench <model> ...      tokens per second of one request (src/main.rs:926-1151)
     tq replay ...             trace replay (see tq_kv_amd/replay.py)
     tq list                   the shapes that can be run with random weights
+    tq random-weights ...     write a model folder with seeded random weights
 
 <model> is a folder with config.json and *.safetensors, or the name of a shape of the
 catalog ("qwen2.5:7b", "tiny:a"), which is run with seeded random weights.  The
@@ -66,6 +67,11 @@ def build_parser():
     r.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     r.add_argument("--out", required=True)
     r.add_argument("--max-tokens", type=int, required=True)
+    rw = sub.add_parser("random-weights", help="Write a model folder (config.json, model.safetensors) with random weights")
+    rw.add_argument("shape", help="Name of a shape (see `tq list`) or path of a config.json")
+    rw.add_argument("out", help="Folder to write")
+    rw.add_argument("--seed", type=int, default=0)
+    rw.add_argument("--store", choices=["bfloat16", "float32"], default="bfloat16", help="dtype the tensors are stored in")
     ls = sub.add_parser("list", help="List the shapes of the catalog")
     ls.add_argument("-a", "--available", action="store_true", help="(accepted for likeness; all shapes are always listed)")
     return ap
@@ -163,6 +169,20 @@ def cmd_bench(args):
     return 0
 
 
+def cmd_random_weights(args):
+    import torch
+
+    from .engine import Model
+    shape = args.shape
+    if os.path.isfile(shape):
+        with open(shape) as f:
+            shape = json.load(f)
+    folder = Model.write_random_folder(args.out, shape, seed=args.seed,
+                                       store_dtype=torch.bfloat16 if args.store == "bfloat16" else torch.float32)
+    print("wrote %s" % folder)
+    return 0
+
+
 def cmd_list(args):
     from .config import catalog
     for name, tag in catalog.entries():
@@ -189,6 +209,8 @@ def main(argv=None):
         return cmd_bench(args)
     if args.command == "list":
         return cmd_list(args)
+    if args.command == "random-weights":
+        return cmd_random_weights(args)
     if args.command == "replay":
         from .replay import main as replay_main
         return replay_main(["--model", args.model, "--dtype", args.dtype, "--out", args.out, "--max-tokens", str(args.max_tokens)])
