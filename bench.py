@@ -25,6 +25,7 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--shape", default=SHAPE)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--no-tune", action="store_true", help="do not let the library pick its fastest kernel per product shape")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -34,6 +35,10 @@ def main():
 
     from tq_kv_amd import Engine, GenerationParams, Model, generate
     from tq_kv_amd.config import catalog
+    from tq_kv_amd.parts.linear import tune_library
+
+    if not args.no_tune:
+        tune_library(True)          # products of more than 16 rows are the library's: let it try its kernels once per shape
 
     raw = dict(catalog.find(args.shape))
     full_layers = raw["num_hidden_layers"]
@@ -55,7 +60,7 @@ def main():
     # -- prefill of one prompt --------------------------------------------------------------
     p = prompts(1)[0]
     times = []
-    for i in range(4):
+    for i in range(5):
         slot = engine.open()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -63,7 +68,7 @@ def main():
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
         engine.close(slot)
-    prefill_s = min(times[1:])
+    prefill_s = min(times[2:])
     T = args.prompt_len
     linear_params = layers * (H * (nh + 2 * nkv) * d + nh * d * H + 3 * H * I)
     prefill_flops = 2.0 * T * linear_params + layers * 4.0 * nh * d * (T * (T + 1) / 2) + 2.0 * H * V
@@ -102,7 +107,8 @@ def main():
         "config": {"model": args.shape, "global_batch": args.batch, "seq_len": ctx_len, "parallelism": "single-gpu",
                    "layers": layers, "layers_of_shape": full_layers, "hidden": H, "heads": nh, "kv_heads": nkv,
                    "head_dim": d, "intermediate": I, "vocab": V, "prompt_len": args.prompt_len,
-                   "new_tokens": args.warmup + args.steps + 1, "weights": "random N(0,0.02)", "sampling": "greedy"},
+                   "new_tokens": args.warmup + args.steps + 1, "weights": "random N(0,0.02)", "sampling": "greedy",
+                   "library_tuning": not args.no_tune},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK["hbm_gbs"], "unit": "GB/s",
                      "frac": round(achieved / PEAK["hbm_gbs"], 4)},

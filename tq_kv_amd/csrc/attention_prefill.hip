@@ -6,7 +6,10 @@
 // start at any position (the reference's is only for position 0, :1937-1956), with an
 // optional window.
 //
-// A block of 4 waves owns the tile; wave w owns queries 16w..16w+15.  The pages of keys
+// A block of 4 waves owns the tile; wave w owns queries 16w..16w+15.  Tiles late in a
+// sequence see more keys than early ones: the host lists the tiles longest first, and
+// blocks are numbered heads-fastest, so that the blocks that share a compute unit have
+// different lengths and the long ones start first.  The pages of keys
 // (64 positions x head_dim) and of values (head_dim x 64 positions, stored transposed)
 // are staged in LDS once per block and read by all four waves; the next page is on
 // its way from global memory into registers while the current one is computed on.
@@ -26,6 +29,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
 union pf_pack8 {
     bf16x8_t v;
     bf16x4_t h[2];
+    __bf16 b[8];
     uint16_t u[8];
     uint4 q;
 };
@@ -53,7 +57,7 @@ void attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __rest
     const int tid = threadIdx.x;
     const int wave = tid / TQK_WAVE, lane = tid % TQK_WAVE;
     const int col = lane % 16, g = lane / 16;
-    const int tile = blockIdx.x, head = blockIdx.y;
+    const int tile = blockIdx.y, head = blockIdx.x;      // heads fastest: neighbouring blocks do equal work
     const int kvh = head / (n_heads / n_kv_heads);
     const int seq = tile_seq[tile], tok0 = tile_tok0[tile], count = tile_count[tile];
     const int pos0 = tok_pos[tok0];
@@ -67,7 +71,10 @@ void attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __rest
     // the wave's and the tile's ranges of positions
     const bool wave_live = wave * 16 < count;
     const int wave_last = min(pos0 + wave * 16 + 15, pos0 + count - 1);
-    const int wave_lo = window > 0 ? max(0, pos0 + wave * 16 - window + 1) : 0;
+    const int wave_first = pos0 + wave * 16;                  // the wave's first query: it sees the fewest late keys
+    const int wave_lo = window > 0 ? max(0, wave_first - window + 1) : 0;
+    const int wave_lo_last = window > 0 ? max(0, wave_last - window + 1) : 0;   // the wave's last query sees the fewest early keys
+    const float c2 = scale * 1.44269504088896340736f;
     const int tile_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
     const int first_page = tile_lo / TQK_PAGE, last_page = (pos0 + count - 1) / TQK_PAGE;
 
@@ -132,54 +139,68 @@ void attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __rest
         const int key0 = pg * TQK_PAGE;
         if (!wave_live || key0 > wave_last || key0 + TQK_PAGE - 1 < wave_lo) continue;
 
+        // four independent chains of products (one per group of 16 keys), interleaved
         floatx4_t s[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < 4; ++t) s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb) {
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
                 const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(&k_lds[(t * 16 + col) * KSTRIDE + kb * 32 + g * 8]);
                 s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq[kb], s[t], 0, 0, 0);
             }
+        // Softmax in base 2: with c = scale * log2(e), p = 2^(s*c - m) where m is the running
+        // maximum of s*c.  Only pages that cross a query's causal or window edge need the mask.
+        const bool need_mask = key0 + TQK_PAGE - 1 > wave_first || key0 < wave_lo_last;
+        float mx = -INFINITY;
+        if (need_mask) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int j = key0 + t * 16 + g * 4 + r;
+                    if (j < my_lo || j > my_pos) s[t][r] = -INFINITY;
+                    mx = fmaxf(mx, s[t][r]);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[t][r]);
         }
-        float mx = m;
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int j = key0 + t * 16 + g * 4 + r;
-                const float v = (j >= my_lo && j <= my_pos) ? s[t][r] * scale : -INFINITY;
-                s[t][r] = v;
-                mx = fmaxf(mx, v);
-            }
         mx = fmaxf(mx, __shfl_xor(mx, 16, TQK_WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));
+        const float m_new = fmaxf(m, mx * c2);           // c2 > 0, so the maximum of s*c2 is c2 times the maximum of s
         // a query may have no key in this page yet (window, or a lane without a query)
-        const float alpha = mx == -INFINITY ? 1.f : expf(m - mx);
-        m = mx;
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m - m_use);     // 2^(-inf) = 0 on a query's first keys
+        m = m_new;
         float psum = 0.f;
         pf_pack8 pb[2];
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float p = s[t][r] == -INFINITY ? 0.f : expf(s[t][r] - mx);
-                const uint16_t pbits = float_to_bf16_bits(p);
-                psum += __uint_as_float(((uint32_t)pbits) << 16);
-                pb[t / 2].u[(t % 2) * 4 + r] = pbits;
+                const float p = __builtin_amdgcn_exp2f(fmaf(s[t][r], c2, -m_use));
+                // the probability enters the product as bfloat16; the sum uses the same rounded value
+                const __bf16 pr16 = (__bf16)p;
+                psum += (float)pr16;
+                pb[t / 2].b[(t % 2) * 4 + r] = pr16;
             }
         l = l * alpha + psum;
+        if (__any(alpha != 1.f)) {
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            o[db][0] *= alpha; o[db][1] *= alpha; o[db][2] *= alpha; o[db][3] *= alpha;
-            // the lane's 8 keys of each half page lie together (value_place)
-            const uint16_t* vrow = &v_lds[(db * 16 + col) * VSTRIDE + g * 8];
+            for (int db = 0; db < DB; ++db) { o[db][0] *= alpha; o[db][1] *= alpha; o[db][2] *= alpha; o[db][3] *= alpha; }
+        }
+        // the lane's 8 keys of each half page lie together (value_place); DB independent chains
 #pragma unroll
-            for (int pr = 0; pr < 2; ++pr) {
-                const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(vrow + pr * 32);
+        for (int pr = 0; pr < 2; ++pr)
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(&v_lds[(db * 16 + col) * VSTRIDE + g * 8 + pr * 32]);
                 o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pb[pr].v, o[db], 0, 0, 0);
             }
-        }
     }
     l += __shfl_xor(l, 16, TQK_WAVE);
     l += __shfl_xor(l, 32, TQK_WAVE);
@@ -211,10 +232,10 @@ extern "C" int tqk_attention_prefill(const void* q, const void* keys, const void
     TQK_REQUIRE(tqk_attention_prefill_supported(head_dim), "tqk_attention_prefill: head_dim %d is not one of 32, 64, 96, 128", head_dim);
     TQK_REQUIRE(table_width > 0 && n_pages > 0 && n_seqs > 0, "tqk_attention_prefill: empty page table");
     TQK_REQUIRE(window >= 0, "tqk_attention_prefill: negative window");
-    TQK_REQUIRE(n_heads <= 65535, "tqk_attention_prefill: too many heads for the grid");
+    TQK_REQUIRE(n_tiles <= 65535, "tqk_attention_prefill: %d tiles are more than the grid takes", n_tiles);
     if (n_tiles == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    dim3 grid(n_tiles, n_heads);
+    dim3 grid(n_heads, n_tiles);
 #define LAUNCH(DD) attention_prefill_kernel<DD><<<grid, PF_THREADS, 0, s>>>( \
         (const bf16_t*)q, (const bf16_t*)keys, (const bf16_t*)values, tok_pos, page_table, table_width, tile_seq, tile_tok0, \
         tile_count, seq_start, seq_new, window, scale, (bf16_t*)out, n_heads, n_kv_heads)

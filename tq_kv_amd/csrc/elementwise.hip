@@ -169,7 +169,7 @@ extern "C" int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const
 // ---- bias + rotation + cache write ------------------------------------------------
 // Rotation as src/models/turbo_generic.rs:417-427 (halves) and :430-443 (pairs), angle
 // tables as :1654-1670, applied after the bias (:805-813, :832-833); the cache holds
-// rotated keys.  A block handles one head of one token; a thread computes one element
+// rotated keys.  A wave handles one head of one token; a thread computes one element
 // and reads the partner it rotates with.
 template <typename TA, typename TB>
 __global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restrict__ bias,
@@ -181,7 +181,10 @@ __global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restri
                                   TA* __restrict__ q_out, int n_heads, int n_kv_heads, int head_dim,
                                   int write_kv) {
     const int t = blockIdx.x;
-    const int head = blockIdx.y;                       // 0..nh-1 q, then nkv k heads, then nkv v heads
+    // a wave per head, four heads per block: 0..nh-1 q, then nkv k heads, then nkv v heads
+    const int head = blockIdx.y * 4 + threadIdx.x / TQK_WAVE;
+    const int lane = threadIdx.x % TQK_WAVE;
+    if (head >= n_heads + 2 * n_kv_heads) return;
     const int total = (n_heads + 2 * n_kv_heads) * head_dim;
     const int pos = tok_pos[t];
     const int kind = head < n_heads ? 0 : (head < n_heads + n_kv_heads ? 1 : 2);
@@ -211,7 +214,7 @@ __global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restri
 
     const int half_rot = rot_dim / 2;
     const bool rotate = style != 0 && kind != 2 && pos < max_positions;
-    for (int i = threadIdx.x; i < head_dim; i += blockDim.x) {
+    for (int i = lane; i < head_dim; i += TQK_WAVE) {
         float x = to_float(src[i]) + (b ? to_float(b[i]) : 0.f);
         if (rotate && i < rot_dim) {
             // `first`: this element is x0 of its pair, else x1; p is the pair's table column
@@ -249,8 +252,8 @@ extern "C" int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, 
     }
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    dim3 grid(n_tokens, n_heads + 2 * n_kv_heads);
-    const int threads = 64;
+    dim3 grid(n_tokens, (n_heads + 2 * n_kv_heads + 3) / 4);
+    const int threads = 4 * TQK_WAVE;
 #define LAUNCH(TA, TB) rope_store_kernel<TA, TB><<<grid, threads, 0, s>>>( \
         (const TA*)qkv, (const TB*)bias, cos_table, sin_table, rot_dim, style, max_positions, tok_seq, tok_pos, \
         page_table, table_width, (TA*)keys, (TA*)values, (TA*)q_out, n_heads, n_kv_heads, head_dim, write_kv)
@@ -275,13 +278,36 @@ __global__ void swiglu_kernel(const TA* __restrict__ gate_up, TA* __restrict__ o
     out[i] = from_float<TA>((g / (1.f + expf(-g))) * u);
 }
 
+// The same, 8 bfloat16 values (16 bytes) per thread; inter must be a multiple of 8.
+__global__ void swiglu_bf16x8_kernel(const uint4* __restrict__ gate_up, uint4* __restrict__ out, int inter8, size_t total8) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total8) return;
+    const size_t t = i / inter8, c = i % inter8;
+    const uint4 g4 = gate_up[t * 2 * inter8 + c], u4 = gate_up[t * 2 * inter8 + inter8 + c];
+    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
+        const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
+        const float r0 = (g0 / (1.f + expf(-g0))) * u0, r1 = (g1 / (1.f + expf(-g1))) * u1;
+        ow[k] = (uint32_t)float_to_bf16_bits(r0) | ((uint32_t)float_to_bf16_bits(r1) << 16);
+    }
+    out[i] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 extern "C" int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, void* stream) {
     TQK_REQUIRE(gate_up && out, "tqk_swiglu: null pointer");
     TQK_REQUIRE(n_tokens >= 0 && inter > 0, "tqk_swiglu: bad sizes");
     if (n_tokens == 0) return 0;
     const size_t total = (size_t)n_tokens * inter;
-    const unsigned blocks = (unsigned)((total + 255) / 256);
     hipStream_t s = (hipStream_t)stream;
+    if (act_dtype == TQK_BF16 && inter % 8 == 0 && ((((uintptr_t)gate_up) | ((uintptr_t)out)) & 15) == 0) {
+        const size_t total8 = total / 8;
+        swiglu_bf16x8_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, s>>>((const uint4*)gate_up, (uint4*)out, inter / 8, total8);
+        return tqk_check_launch("tqk_swiglu");
+    }
+    const unsigned blocks = (unsigned)((total + 255) / 256);
     if (act_dtype == TQK_F32) swiglu_kernel<float><<<blocks, 256, 0, s>>>((const float*)gate_up, (float*)out, inter, total);
     else if (act_dtype == TQK_BF16) swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, total);
     else return tqk_fail("tqk_swiglu: unknown dtype %d", act_dtype);

@@ -77,9 +77,11 @@ class StepContext:
                 t_seq.append(i)
                 t_tok0.append(int(host.cu[i]) + a)
                 t_count.append(min(TILE, n - a))
-        host.tile_seq = np.asarray(t_seq, dtype=np.int32)
-        host.tile_tok0 = np.asarray(t_tok0, dtype=np.int32)
-        host.tile_count = np.asarray(t_count, dtype=np.int32)
+        # longest first (a tile's work grows with the position of its last query)
+        order = sorted(range(len(t_seq)), key=lambda k: -(int(host.tok_pos[t_tok0[k]]) + t_count[k]))
+        host.tile_seq = np.asarray([t_seq[k] for k in order], dtype=np.int32)
+        host.tile_tok0 = np.asarray([t_tok0[k] for k in order], dtype=np.int32)
+        host.tile_count = np.asarray([t_count[k] for k in order], dtype=np.int32)
         self.host = host
         self.all_decode = all(n == 1 for n in lens)
         self.max_new = max(lens)

@@ -22,6 +22,18 @@ from .. import kernels as K
 POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16}
 
 
+def tune_library(on=True, seconds=30):
+    """Let the library try its kernels for each new product shape once and keep the fastest
+    (PyTorch's TunableOp over hipBLASLt and rocBLAS).  The first call with a new shape then
+    takes up to `seconds`; it pays for prompts, whose products are the library's."""
+    import torch.cuda.tunable as tunable
+    tunable.enable(bool(on))
+    tunable.tuning_enable(bool(on))
+    if on:
+        tunable.set_max_tuning_duration(int(seconds * 1000))
+        tunable.record_untuned_enable(False)
+
+
 def _skinny_ok(x, weight):
     return (POLICY["skinny"] and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
             and x.shape[1] % 32 == 0 and x.shape[0] <= POLICY["skinny_max_rows"] and K.has_skinny())
