@@ -40,6 +40,11 @@ def main():
     if not args.no_tune:
         tune_library(True)          # products of more than 16 rows are the library's: let it try its kernels once per shape
 
+    t_start = time.perf_counter()
+
+    def note(msg):
+        print("[bench %.0fs] %s" % (time.perf_counter() - t_start, msg), file=sys.stderr, flush=True)
+
     raw = dict(catalog.find(args.shape))
     full_layers = raw["num_hidden_layers"]
     if args.layers:
@@ -48,6 +53,7 @@ def main():
     H, I, V = raw["hidden_size"], raw["intermediate_size"], raw["vocab_size"]
     nh, nkv, d = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"]
     ctx_len = raw["max_position_embeddings"]
+    note("making random weights for %s (%d layers)" % (args.shape, layers))
     model = Model.random(raw, seed=0, dtype="bfloat16", device="cuda:0")
     max_batch = 64 if not args.no_points else args.batch
     total_new = args.steps + args.warmup + 2
@@ -60,6 +66,7 @@ def main():
     # -- prefill of one prompt --------------------------------------------------------------
     p = prompts(1)[0]
     times = []
+    note("prefill of %d tokens" % args.prompt_len)
     for i in range(5):
         slot = engine.open()
         torch.cuda.synchronize()
@@ -69,6 +76,10 @@ def main():
         times.append(time.perf_counter() - t0)
         engine.close(slot)
     prefill_s = min(times[2:])
+    if not args.no_tune:
+        # keep what was found for the prompt's product shapes, try nothing new from here on
+        import torch.cuda.tunable as tunable
+        tunable.tuning_enable(False)
     T = args.prompt_len
     linear_params = layers * (H * (nh + 2 * nkv) * d + nh * d * H + 3 * H * I)
     prefill_flops = 2.0 * T * linear_params + layers * 4.0 * nh * d * (T * (T + 1) / 2) + 2.0 * H * V
@@ -90,11 +101,15 @@ def main():
         seconds = marks[warmup + steps] - marks[warmup]
         return batch * steps / seconds, seconds / steps
 
+    note("decode at batch %d" % args.batch)
     tps, sec_per_step = decode(args.batch, args.steps, args.warmup)
     points = {}
     if not args.no_points:
+        note("decode at batch 1")
         points["decode_b1"] = round(decode(1, min(args.steps, 64), 8)[0], 1)
+        note("decode at batch 64")
         points["decode_b64"] = round(decode(64, min(args.steps, 32), 4)[0], 1)
+    note("done")
 
     weight_bytes = 2.0 * (linear_params + H * V)                      # every weight the step uses, once
     mean_ctx = args.prompt_len + args.warmup + args.steps / 2.0

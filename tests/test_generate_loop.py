@@ -34,8 +34,9 @@ class FakeEngine:
         out = []
         for s, toks, want in items:
             self.seen[s].extend(toks)
-            assert want == [len(toks) - 1]
-            out.append(list(self.seen[s]))
+            assert want in ([len(toks) - 1], [])
+            if want:
+                out.append(list(self.seen[s]))
         return out
 
 
@@ -102,6 +103,17 @@ def test_batches_follow_one_another_and_reuse_slots():
     assert [len(s) for s in firsts] == [2, 2, 1]
     assert {slot for s in eng.steps for slot, _ in s} == {0, 1}       # the same two slots serve all five
     assert eng.seen == {}
+
+
+def test_long_prompts_are_fed_in_several_steps():
+    from tq_kv_amd.engine.generate import _prompt_steps
+    assert _prompt_steps([3, 4, 2], 100) == [[(0, 0, 3), (1, 0, 4), (2, 0, 2)]]
+    assert _prompt_steps([3, 4, 2], 5) == [[(0, 0, 3), (1, 0, 2)], [(1, 2, 4), (2, 0, 2)]]
+    assert _prompt_steps([7], 3) == [[(0, 0, 3)], [(0, 3, 6)], [(0, 6, 7)]]
+    out, eng, _ = run([[1, 2, 3], [4, 5, 6, 7], [8, 9]], [[10, 11], [20, 21], [30, 31]], 2, max_step_tokens=5)
+    assert out == [[10, 11], [20, 21], [30, 31]]
+    assert eng.steps[0] == [(0, [1, 2, 3]), (1, [4, 5])] and eng.steps[1] == [(1, [6, 7]), (2, [8, 9])]
+    assert eng.steps[2] == [(0, [10]), (1, [20]), (2, [30])] and len(eng.steps) == 3
 
 
 def test_plan_batches_by_cache_room():

@@ -45,12 +45,15 @@ def plan_batches(prompt_lens, max_new, max_tokens, max_batch):
     return batches
 
 
-def generate(engine, prompts, params=None, eos_ids=(), on_tokens=None, max_batch=64, make_sampler=None):
+def generate(engine, prompts, params=None, eos_ids=(), on_tokens=None, max_batch=64, make_sampler=None,
+             max_step_tokens=8192):
     """prompts: token-id lists.  Returns for each prompt the emitted token ids.
 
     eos_ids: stop tokens.  on_tokens(pairs): called after every step with the
     (request index, token) pairs emitted by it.  make_sampler(params, request_ids): the
-    sampler of a batch (default: the device sampler)."""
+    sampler of a batch (default: the device sampler).  max_step_tokens: most tokens one step
+    runs; a batch's prompts are fed in as many steps as that takes (whole prompts together
+    while they fit, a longer prompt in pieces), which bounds the step's working memory."""
     params = params or GenerationParams()
     eos = set(int(t) for t in eos_ids)
     prompts = [list(p) for p in prompts]
@@ -68,19 +71,49 @@ def generate(engine, prompts, params=None, eos_ids=(), on_tokens=None, max_batch
 
     emitted = [[] for _ in prompts]
     for batch in plan_batches([len(p) for p in prompts], params.max_tokens, engine.max_tokens, max_batch):
-        _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, make_sampler(params, batch))
+        _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, make_sampler(params, batch),
+                   max(1, int(max_step_tokens)))
     return emitted
 
 
-def _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, sampler):
+def _prompt_steps(lens, max_step_tokens):
+    """Cut prompts of the given lengths into steps of at most max_step_tokens tokens.
+    Returns steps, each a list of (index, begin, end); a prompt's pieces come in order."""
+    steps, cur, room = [], [], max_step_tokens
+    for i, n in enumerate(lens):
+        begin = 0
+        while begin < n:
+            take = min(n - begin, room)
+            cur.append((i, begin, begin + take))
+            begin += take
+            room -= take
+            if room == 0:
+                steps.append(cur)
+                cur, room = [], max_step_tokens
+    if cur:
+        steps.append(cur)
+    return steps
+
+
+def _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, sampler, max_step_tokens):
     slots = {}
     borrow = {"borrow": True} if getattr(engine, "use_graphs", False) else {}
     try:
         for r in batch:
             slots[r] = engine.open()
-        logits = engine.step([(slots[r], prompts[r], [len(prompts[r]) - 1]) for r in batch])
         live = list(range(len(batch)))                 # indices into `batch`
-        drawn = dict(zip(live, sampler.sample(logits, live)))
+        drawn = {}
+        for step in _prompt_steps([len(prompts[r]) for r in batch], max_step_tokens):
+            items, ends = [], []
+            for b, begin, end in step:
+                r = batch[b]
+                last = end == len(prompts[r])
+                items.append((slots[r], prompts[r][begin:end], [end - begin - 1] if last else []))
+                if last:
+                    ends.append(b)
+            logits = engine.step(items)
+            if ends:
+                drawn.update(zip(ends, sampler.sample(logits, ends)))
         while live:
             feed, pairs = [], []
             for b in live:
