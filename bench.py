@@ -35,10 +35,6 @@ def main():
 
     from tq_kv_amd import Engine, GenerationParams, Model, generate
     from tq_kv_amd.config import catalog
-    from tq_kv_amd.parts.linear import tune_library
-
-    if not args.no_tune:
-        tune_library(True)          # products of more than 16 rows are the library's: let it try its kernels once per shape
 
     t_start = time.perf_counter()
 
@@ -64,6 +60,13 @@ def main():
         return torch.randint(0, V, (n, args.prompt_len), generator=gen).tolist()
 
     # -- prefill of one prompt --------------------------------------------------------------
+    if not args.no_tune:
+        # products of more than 16 rows are the library's: let it try its kernels once for the
+        # shapes of the measured steps (a prompt of prompt_len tokens, decoding at batch 64)
+        note("library tuning for %d and 64 rows" % args.prompt_len)
+        model.tune_library(args.prompt_len)
+        if not args.no_points:
+            model.tune_library(64)
     p = prompts(1)[0]
     times = []
     note("prefill of %d tokens" % args.prompt_len)
@@ -76,10 +79,7 @@ def main():
         times.append(time.perf_counter() - t0)
         engine.close(slot)
     prefill_s = min(times[2:])
-    if not args.no_tune:
-        # keep what was found for the prompt's product shapes, try nothing new from here on
-        import torch.cuda.tunable as tunable
-        tunable.tuning_enable(False)
+
     T = args.prompt_len
     linear_params = layers * (H * (nh + 2 * nkv) * d + nh * d * H + 3 * H * I)
     prefill_flops = 2.0 * T * linear_params + layers * 4.0 * nh * d * (T * (T + 1) / 2) + 2.0 * H * V

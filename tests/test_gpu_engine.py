@@ -240,3 +240,31 @@ def test_sampled_generation_float32_equals_plain(name):
     together = generate(eng, ps, GenerationParams(max_tokens=10, seed=5, temperature=0.8, top_k=0, top_p=1.0,
                                                   repeat_penalty=1.0), max_batch=4)
     assert alone == together
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_many_sequences_decode_through_replayed_graphs(dtype):
+    # 40 sequences: more rows than the skinny products take, so the captured step holds library
+    # calls too; every replay is checked (with other work between the replays)
+    eng = G.engine("B", dtype, True)
+    reqs = G.prompts("B", [3 + (7 * i) % 50 for i in range(40)], seed=1000)
+    slots = [eng.open() for _ in reqs]
+    heads = [len(r) - 6 for r in reqs]
+    heads = [max(1, h) for h in heads]
+    eng.step([(s, r[:h], []) for s, r, h in zip(slots, reqs, heads)])
+    pos = list(heads)
+    refs = [G.plain_logits("B", r, True) for r in reqs]
+    n_graphs = len(eng.graphs)
+    for step in range(6):
+        live = [i for i in range(len(reqs)) if pos[i] < len(reqs[i])]
+        if not live:
+            break
+        out = eng.step([(slots[i], [reqs[i][pos[i]]], [0]) for i in live])
+        torch.zeros(1000, device=out.device).add_(1.0)           # unrelated work between replays
+        for j, i in enumerate(live):
+            G.close(out[j], refs[i][pos[i]], dtype, "seq %d at %d (step %d)" % (i, pos[i], step))
+            pos[i] += 1
+    assert len(eng.graphs) > n_graphs
+    for s in slots:
+        eng.close(s)
+    eng.cache.check()

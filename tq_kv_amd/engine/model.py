@@ -44,10 +44,10 @@ class Model:
         self.head = None
         self.loaded = False
         # a step can be captured as a graph if every part's forward launches the same kernels
-        # whatever the step's data are; steps of more rows than the skinny products take
-        # would bring library calls into the graph and are run directly
+        # whatever the step's data are; up to 64 rows (beyond 16 the products are library calls,
+        # which capture as they are)
         self.graph_safe = all(getattr(b, "graph_safe", False) for b in self.blocks) and getattr(self.final_norm, "graph_safe", False)
-        self.graph_max_rows = 16
+        self.graph_max_rows = 64
 
     # -- tensors ----------------------------------------------------------
     def tensor_specs(self):
@@ -107,6 +107,26 @@ class Model:
                               % (shape, ", ".join("%s:%s" % e for e in catalog.entries())))
         model = Model.from_config_dict(raw, "float32", "cpu")
         return write_model_folder(folder, raw, model.tensor_specs(), seed, store_dtype)
+
+    def tune_library(self, rows):
+        """Let the library try its kernels once for every product of the model at `rows`
+        rows (more than 16: fewer never reach the library) and keep the fastest for later
+        calls.  Takes seconds per distinct weight shape."""
+        from ..parts import linear as L
+        if self.dtype != torch.bfloat16 or rows <= L.POLICY["skinny_max_rows"]:
+            return
+        L.tune_library(True)
+        seen = set()
+        products = [w for b in self.blocks for w in b.product_weights()] + [(self.head, torch.float32)]
+        for weight, out_dtype in products:
+            key = (tuple(weight.shape), out_dtype)
+            if weight.dtype != torch.bfloat16 or key in seen:
+                continue
+            seen.add(key)
+            x = torch.zeros((rows, weight.shape[1]), dtype=torch.bfloat16, device=self.device)
+            L.linear(x, weight, out_dtype=out_dtype)
+        torch.cuda.synchronize()
+        L.freeze_library_tuning()
 
     # -- one step ---------------------------------------------------------
     def forward(self, ctx, cache):

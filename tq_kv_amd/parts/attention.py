@@ -70,6 +70,9 @@ class Attention(Part):
     def cache_need(self):
         return KVNeed(self.n_kv_heads, self.head_dim, self.window)
 
+    def product_weights(self):
+        return [(self.w_qkv, None), (self.w_o, None)]
+
     def forward(self, x, ctx, entry):
         n = x.shape[0]
         qkv = linear(x, self.w_qkv)

@@ -55,6 +55,9 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def product_weights(self):
+        return [w for part in self.parts.values() for w in part.product_weights()]
+
     def forward(self, h, delta, ctx, entry):
         x = self.mixer_norm.add_norm(h, delta)
         a = self.mixer.forward(x, ctx, entry)

@@ -29,5 +29,8 @@ class GatedSiLU(Part):
         self.w_gate_up = torch.cat([w.to(dtype) for w in ws], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"]
 
+    def product_weights(self):
+        return [(self.w_gate_up, None), (self.w_down, None)]
+
     def forward(self, x, ctx):
         return linear(gated_silu_linear(x, self.w_gate_up), self.w_down)

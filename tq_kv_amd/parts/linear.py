@@ -34,6 +34,13 @@ def tune_library(on=True, seconds=30):
         tunable.record_untuned_enable(False)
 
 
+def freeze_library_tuning():
+    """Keep using what tuning has found so far, try nothing new."""
+    import torch.cuda.tunable as tunable
+    tunable.enable(True)
+    tunable.tuning_enable(False)
+
+
 def _skinny_ok(x, weight):
     return (POLICY["skinny"] and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
             and x.shape[1] % 32 == 0 and x.shape[0] <= POLICY["skinny_max_rows"] and K.has_skinny())

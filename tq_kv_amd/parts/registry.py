@@ -76,3 +76,8 @@ class Part:
 
     def cache_need(self):
         return None
+
+    def product_weights(self):
+        """[(weight [N, K], output dtype or None)] of the matrix products the part runs
+        through parts.linear (what the library can be tuned for)."""
+        return []
