@@ -1,0 +1,71 @@
+"""The layer sizes of the three large shapes (Qwen2.5-7B, 1.5B, 32B) with two layers each:
+the float32 path against the plain implementation (7B sizes), and the bfloat16 path against
+the float32 path at spot-checked positions, prompt and decoding, in a batch of unequal
+lengths.  Sizes here are what the small configurations cannot show: 28/40/12 heads in groups
+of 7/5/6, widths and vocabularies that are no power of two, rows of 18944 and 27648."""
+import pytest
+import torch
+
+import helpers
+import plain_qwen2 as plain
+from tq_kv_amd import Engine, Model
+from tq_kv_amd.config import catalog
+from tq_kv_amd.weights import random_tensors
+
+pytestmark = pytest.mark.gpu
+
+
+def two_layer(shape):
+    raw = dict(catalog.find(shape))
+    raw["num_hidden_layers"] = 2
+    return raw
+
+
+def build(raw, dtype, tensors):
+    model = Model.from_config_dict(raw, dtype, "cuda")
+    want = torch.float32 if dtype == "float32" else torch.bfloat16
+    return model.load({k: v.to(want) for k, v in tensors.items()})
+
+
+def tensors_for(raw, seed):
+    specs = Model.from_config_dict(raw, "float32", "cpu").tensor_specs()
+    return random_tensors(specs, seed, torch.bfloat16, "cuda")
+
+
+@pytest.mark.parametrize("shape", ["qwen2.5:7b", "qwen2.5:1.5b", "qwen2.5:32b"])
+def test_bfloat16_tracks_float32_at_large_sizes(shape):
+    raw = two_layer(shape)
+    tensors = tensors_for(raw, 3)
+    lens = [300, 70, 1]
+    prompts = [helpers.random_tokens(n, raw["vocab_size"], 50 + i) for i, n in enumerate(lens)]
+    nxt = [7, 11, 13]
+    outs = {}
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine(build(raw, dtype, tensors), max_tokens=1024)
+        slots = [eng.open() for _ in prompts]
+        a = eng.step([(s, p, [len(p) - 1, 0] if len(p) > 1 else [0]) for s, p in zip(slots, prompts)])
+        b = eng.step([(s, [t], [0]) for s, t in zip(slots, nxt)])
+        outs[dtype] = torch.cat([a, b]).cpu()
+        for s in slots:
+            eng.close(s)
+        del eng
+        torch.cuda.empty_cache()
+    scale = outs["float32"].abs().max().item()
+    assert 0.05 < scale < 50
+    torch.testing.assert_close(outs["bfloat16"], outs["float32"], atol=0.03 * max(1.0, scale), rtol=0.03)
+
+
+def test_float32_path_equals_plain_at_7b_sizes():
+    raw = two_layer("qwen2.5:7b")
+    tensors = tensors_for(raw, 4)
+    prompt = helpers.random_tokens(40, raw["vocab_size"], 60)
+    eng = Engine(build(raw, "float32", tensors), max_tokens=256)
+    s = eng.open()
+    got = [eng.step([(s, prompt[:33], [0, 32])])]
+    for t in range(33, 40):
+        got.append(eng.step([(s, [prompt[t]], [0])]))
+    eng.close(s)
+    got = torch.cat(got).cpu()
+    cfg = dict(raw)
+    want = plain.forward({k: v.float().cpu() for k, v in tensors.items()}, cfg, prompt)[[0] + list(range(32, 40))]
+    torch.testing.assert_close(got, want, atol=2e-5 * max(1.0, want.abs().max().item()), rtol=2e-5)

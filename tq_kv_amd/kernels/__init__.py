@@ -227,7 +227,7 @@ def attention_decode_supported(head_dim):
     return bool(library().tqk_attention_decode_supported(int(head_dim)))
 
 
-def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, target_blocks=512):
+def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, target_blocks=256):
     """Attention of one new token per sequence (q [B, heads, d] bfloat16, row b belongs to
     sequence b at position tok_pos[b]) over the paged cache; out [B, heads*d]."""
     n, n_heads, head_dim = q.shape
