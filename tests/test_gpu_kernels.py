@@ -28,7 +28,7 @@ def ints(values):
 
 
 def test_library_is_built_and_loaded():
-    assert K.library().tqk_abi_version() == 1
+    assert K.library().tqk_abi_version() == 2
     assert K.library_path().endswith(".so")
     with pytest.raises(K.KernelError, match="GPU only"):
         K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
@@ -37,10 +37,11 @@ def test_library_is_built_and_loaded():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_embed(dtype):
-    table = rand(301, 72, seed=1, dtype=DT[dtype])
+@pytest.mark.parametrize("hidden", [70, 72, 3584, 9000])
+def test_embed(dtype, hidden):
+    table = rand(301, hidden, seed=1, dtype=DT[dtype])
     ids = ints([0, 300, 17, 17, 5])
-    out = torch.full((5, 72), float("nan"), device=DEV)
+    out = torch.full((5, hidden), float("nan"), device=DEV)
     K.embed(table, ids, out)
     assert torch.equal(out, table.float()[ids.long()])
 
@@ -473,3 +474,140 @@ def test_attention_prefill(nh, nkv, d, window):
     if window != 70:
         other = attention_reference(qs[0][-1:].float(), ks[0], vs[0], torch.tensor([299]), 70, scale)
         assert (other - out[149:150].float().cpu()).abs().max() > 0.1
+
+
+# ---- skinny products with norm, residual sum, gate and rotation folded in ----------------------
+def bf(x):
+    return x.to(torch.bfloat16).float()
+
+
+def prepared(h, nw):
+    """What a kernel that adds to the stream leaves for the next norm: the stream times the
+    norm's weight in bfloat16, and the rows' sums of squares in pieces of 16 columns."""
+    m, k = h.shape
+    xw = (h * nw.float()).to(torch.bfloat16)
+    parts = (k + 15) // 16
+    ss = torch.zeros(parts, 16, device=DEV)
+    pad = torch.zeros(m, parts * 16, device=DEV)
+    pad[:, :k] = h * h
+    ss[:, :m] = pad.reshape(m, parts, 16).sum(-1).t()
+    return xw, (ss, parts)
+
+
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("n,k", [(100, 96), (3584, 3584), (1000, 1536)])
+def test_fused_store_with_and_without_norm(m, n, k):
+    h = rand(16, k, seed=100, scale=2.0)
+    w = rand(n, k, seed=101, scale=1.0 / math.sqrt(k), dtype=torch.bfloat16)
+    nw = (1 + rand(k, seed=102, scale=0.1)).to(torch.bfloat16)
+    rows = ints(list(range(15, 15 - m, -1)))                     # m rows of x, backwards
+    out = torch.full((m, n), float("nan"), device=DEV)
+    xb = h.to(torch.bfloat16)
+    K.fused_store(xb, w, out, rows=rows)
+    torch.testing.assert_close(out.double(), xb.double()[rows.long()] @ w.double().t(), atol=2e-3, rtol=1e-3)
+    eps = 1e-5
+    xw, (ss, parts) = prepared(h, nw)
+    K.fused_store(xw, w, out, (ss, parts, eps), rows=rows)
+    want = plain.rms_norm(h[rows.long()], nw.float(), eps).double() @ w.double().t()
+    torch.testing.assert_close(out.double(), want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("m", [1, 8, 16])
+@pytest.mark.parametrize("inter,k", [(112, 64), (18944, 3584)])
+def test_fused_gated(m, inter, k):
+    h = rand(m, k, seed=103, scale=1.5)
+    w = rand(2 * inter, k, seed=104, scale=0.4 / math.sqrt(k), dtype=torch.bfloat16)      # gate and up of size about 1
+    nw = (1 + rand(k, seed=105, scale=0.1)).to(torch.bfloat16)
+    out = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    xw, (ss, parts) = prepared(h, nw)
+    K.fused_gated(xw, w, out, (ss, parts, 1e-6))
+    gu = bf(plain.rms_norm(h, nw.float(), 1e-6).double() @ w.double().t())
+    torch.testing.assert_close(out.float(), F.silu(gu[:, :inter]) * gu[:, inter:], atol=3e-2, rtol=3e-2)
+    xb = h.to(torch.bfloat16)
+    K.fused_gated(xb, w, out)
+    gu = bf(xb.double() @ w.double().t())
+    torch.testing.assert_close(out.float(), F.silu(gu[:, :inter]) * gu[:, inter:], atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("n,k", [(96, 64), (3584, 18944), (100, 32)])
+def test_fused_residual_prepares_the_next_norm(m, n, k):
+    x = rand(m, k, seed=106, dtype=torch.bfloat16)
+    w = rand(n, k, seed=107, scale=0.02, dtype=torch.bfloat16)
+    nw = (1 + rand(n, seed=113, scale=0.1)).to(torch.bfloat16)
+    h = rand(m, n, seed=108, scale=3.0)
+    want = h + bf((x.double() @ w.double().t()).float())
+    xw = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ss = torch.full((K.fused_residual_parts(n), 16), float("nan"), device=DEV)
+    parts = K.fused_residual(x, w, h, xw, nw, ss)
+    torch.testing.assert_close(h, want, atol=4e-2, rtol=0)          # one bfloat16 step of the product at most
+    assert torch.equal(xw, (h * nw.float()).to(torch.bfloat16))
+    assert parts == (n + 15) // 16
+    torch.testing.assert_close(ss[:, :m].sum(0), (h * h).sum(-1), rtol=1e-5, atol=1e-5)
+    # and what the next product makes of it is the norm of the new stream
+    w2 = rand(48, n, seed=114, scale=1.0 / math.sqrt(n), dtype=torch.bfloat16)
+    if n % 32 == 0:
+        out = torch.empty(m, 48, device=DEV)
+        K.fused_store(xw, w2, out, (ss, parts, 1e-6))
+        torch.testing.assert_close(out.double(), plain.rms_norm(h, nw.float(), 1e-6).double() @ w2.double().t(), atol=2e-2, rtol=2e-2)
+    # without a next norm: the plain copy, no sums
+    h2 = h.clone()
+    K.fused_residual(x, w, h2, xw)
+    assert torch.equal(xw, h2.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("hidden", [96, 100, 3584, 8200])
+def test_embed_prepares_the_first_norm(hidden):
+    table = rand(301, hidden, seed=115, dtype=torch.bfloat16)
+    nw = (1 + rand(hidden, seed=116, scale=0.1)).to(torch.bfloat16)
+    ids = ints([5, 300, 0])
+    h, xw, ss = torch.empty(3, hidden, device=DEV), torch.empty(3, hidden, dtype=torch.bfloat16, device=DEV), torch.zeros(1, 16, device=DEV)
+    K.embed(table, ids, h, copy=xw, copy_weight=nw, ss_out=ss)
+    assert torch.equal(h, table.float()[ids.long()]) and torch.equal(xw, (h * nw.float()).to(torch.bfloat16))
+    torch.testing.assert_close(ss[0, :3], (h * h).sum(-1), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("nh,nkv,d,k", [(28, 4, 128, 3584), (3, 1, 32, 96), (6, 2, 64, 160)])
+def test_fused_qkv_equals_product_then_rotation_kernel(nh, nkv, d, k):
+    m, n_pages = 5, 9
+    total = (nh + 2 * nkv) * d
+    h = rand(m, k, seed=109, scale=1.5)
+    w = rand(total, k, seed=110, scale=1.0 / math.sqrt(k), dtype=torch.bfloat16)
+    bias = rand(total, seed=111, scale=0.3, dtype=torch.bfloat16)
+    nw = (1 + rand(k, seed=112, scale=0.1)).to(torch.bfloat16)
+    c, s = plain.rope_tables(d, 1e4, 400)
+    cos, sin = c.to(DEV), s.to(DEV)
+    pos = ints([0, 63, 64, 200, 399])
+    table = ints([[3, -1, -1, -1, -1, -1, -1], [8, -1, -1, -1, -1, -1, -1], [0, 5, -1, -1, -1, -1, -1],
+                  [1, 1, 1, 2, -1, -1, -1], [4, 4, 4, 4, 4, 4, 7]])
+    keys, values = make_cache(n_pages, nkv, d, torch.bfloat16)
+    q = torch.empty(m, nh, d, dtype=torch.bfloat16, device=DEV)
+    xw, (ss, parts) = prepared(h, nw)
+    K.fused_qkv(xw, w, bias, cos, sin, pos, table, keys, values, q, nh, nkv, d, norm=(ss, parts, 1e-6))
+    # the same with separate kernels: norm, product, rotation + cache write
+    xn = torch.empty(m, k, dtype=torch.bfloat16, device=DEV)
+    K.add_rmsnorm(h, None, nw, 1e-6, xn)
+    qkv = torch.empty(m, total, dtype=torch.bfloat16, device=DEV)
+    K.skinny_bf16(xn, w, qkv)
+    keys2, values2 = make_cache(n_pages, nkv, d, torch.bfloat16)
+    q2 = torch.empty_like(q)
+    K.rope_store(qkv, bias, cos, sin, d, K.STYLE_HALVES, ints([0, 1, 2, 3, 4]), pos, table, keys2, values2, q2, nh, nkv, d)
+    torch.testing.assert_close(q.float(), q2.float(), atol=4e-2, rtol=3e-2)
+    for a, b in ((keys, keys2), (values, values2)):
+        assert torch.equal(torch.isnan(a.float()), torch.isnan(b.float()))          # the same places written
+        ok = ~torch.isnan(a.float())
+        torch.testing.assert_close(a.float()[ok], b.float()[ok], atol=4e-2, rtol=3e-2)
+    # and without norm and bias
+    K.fused_qkv(xn, w, None, cos, sin, pos, table, keys, values, q, nh, nkv, d)
+    K.rope_store(qkv, None, cos, sin, d, K.STYLE_HALVES, ints([0, 1, 2, 3, 4]), pos, table, keys2, values2, q2, nh, nkv, d)
+    torch.testing.assert_close(q.float(), q2.float(), atol=2e-2, rtol=2e-2)
+    ok = ~torch.isnan(keys.float())
+    torch.testing.assert_close(keys.float()[ok], keys2.float()[ok], atol=2e-2, rtol=2e-2)
+
+
+def test_fused_kernels_refuse_what_they_do_not_take():
+    w = rand(16, 64, dtype=torch.bfloat16)
+    with pytest.raises(K.KernelError, match="at most 16"):
+        K.fused_store(rand(17, 64, dtype=torch.bfloat16), w, torch.empty(17, 16, device=DEV))
+    with pytest.raises(K.KernelError, match="multiple of 32"):
+        K.fused_store(rand(2, 48, dtype=torch.bfloat16), rand(16, 48, dtype=torch.bfloat16), torch.empty(2, 16, device=DEV))

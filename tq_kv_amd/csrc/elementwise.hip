@@ -7,28 +7,93 @@
 // The reference looks rows up with candle's embedding op (src/models/turbo_generic.rs:1958).
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
-                             int hidden, int vocab, float* __restrict__ out) {
+                             int hidden, int vocab, float* __restrict__ out, bf16_t* __restrict__ copy,
+                             const bf16_t* __restrict__ copy_weight, float* __restrict__ ss_out) {
+    __shared__ float scratch[16];
     const int t = blockIdx.x;
     const int id = ids[t];
     float* o = out + (size_t)t * hidden;
-    if (id < 0 || id >= vocab) {
-        for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = 0.f;
-        return;
+    bf16_t* c = copy ? copy + (size_t)t * hidden : nullptr;
+    const bool ok = id >= 0 && id < vocab;
+    const T* row = table + (size_t)(ok ? id : 0) * hidden;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float v = ok ? to_float(row[i]) : 0.f;
+        o[i] = v;
+        ss = fmaf(v, v, ss);
+        if (c) c[i] = from_float<bf16_t>(copy_weight ? v * to_float(copy_weight[i]) : v);
     }
-    const T* row = table + (size_t)id * hidden;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_float(row[i]);
+    if (ss_out) {
+        const float total = block_sum(ss, scratch);
+        if (threadIdx.x == 0) ss_out[t] = total;
+    }
+}
+
+// bfloat16 table, hidden a multiple of 8: 16 bytes per thread and load, one pass.
+__global__ void embed_bf16x8_kernel(const bf16_t* __restrict__ table, const int32_t* __restrict__ ids,
+                                    int hidden, int vocab, float* __restrict__ out, bf16_t* __restrict__ copy,
+                                    const bf16_t* __restrict__ copy_weight, float* __restrict__ ss_out) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    const bool ok = id >= 0 && id < vocab;
+    const uint4* row = reinterpret_cast<const uint4*>(table + (size_t)(ok ? id : 0) * hidden);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden / 8; i += blockDim.x) {
+        const uint4 raw = ok ? row[i] : make_uint4(0, 0, 0, 0);
+        const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[2 * j] = __uint_as_float(words[j] << 16);
+            v[2 * j + 1] = __uint_as_float(words[j] & 0xffff0000u);
+        }
+        float4* o = reinterpret_cast<float4*>(out + (size_t)t * hidden + (size_t)i * 8);
+        o[0] = make_float4(v[0], v[1], v[2], v[3]);
+        o[1] = make_float4(v[4], v[5], v[6], v[7]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss = fmaf(v[j], v[j], ss);
+        if (copy) {
+            uint4 packed = raw;
+            if (copy_weight) {
+                const uint4 wraw = reinterpret_cast<const uint4*>(copy_weight)[i];
+                const uint32_t ww[4] = {wraw.x, wraw.y, wraw.z, wraw.w};
+                uint32_t pw[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t lo = float_to_bf16_bits(v[2 * j] * __uint_as_float(ww[j] << 16));
+                    const uint32_t hi = float_to_bf16_bits(v[2 * j + 1] * __uint_as_float(ww[j] & 0xffff0000u));
+                    pw[j] = lo | (hi << 16);
+                }
+                packed = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+            }
+            reinterpret_cast<uint4*>(copy + (size_t)t * hidden)[i] = packed;
+        }
+    }
+    if (ss_out) {
+        const float total = block_sum(ss, scratch);
+        if (threadIdx.x == 0) ss_out[t] = total;
+    }
 }
 
 extern "C" int tqk_embed(const void* table, int table_dtype, const int32_t* ids, int n_tokens,
-                         int hidden, int vocab, float* out, void* stream) {
+                         int hidden, int vocab, float* out, void* copy_bf16, const void* copy_weight,
+                         float* ss_out, void* stream) {
     TQK_REQUIRE(table && ids && out, "tqk_embed: null pointer");
     TQK_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "tqk_embed: bad sizes tokens=%d hidden=%d vocab=%d", n_tokens, hidden, vocab);
+    TQK_REQUIRE(!ss_out || n_tokens <= 16, "tqk_embed: sums of squares are kept for at most 16 tokens, got %d", n_tokens);
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (table_dtype == TQK_F32)
-        embed_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)table, ids, hidden, vocab, out);
-    else if (table_dtype == TQK_BF16)
-        embed_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)table, ids, hidden, vocab, out);
+        embed_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)table, ids, hidden, vocab, out, (bf16_t*)copy_bf16,
+                                                     (const bf16_t*)copy_weight, ss_out);
+    else if (table_dtype == TQK_BF16 && hidden % 8 == 0 && (((uintptr_t)table | (uintptr_t)out | (uintptr_t)copy_bf16 | (uintptr_t)copy_weight) & 15) == 0) {
+        const int threads = ((hidden / 8 + TQK_WAVE - 1) / TQK_WAVE) * TQK_WAVE;
+        embed_bf16x8_kernel<<<n_tokens, threads > 1024 ? 1024 : threads, 0, s>>>((const bf16_t*)table, ids, hidden, vocab, out, (bf16_t*)copy_bf16,
+                                                                               (const bf16_t*)copy_weight, ss_out);
+    } else if (table_dtype == TQK_BF16)
+        embed_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)table, ids, hidden, vocab, out, (bf16_t*)copy_bf16,
+                                                      (const bf16_t*)copy_weight, ss_out);
     else
         return tqk_fail("tqk_embed: unknown dtype %d", table_dtype);
     return tqk_check_launch("tqk_embed");

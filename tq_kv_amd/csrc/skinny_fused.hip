@@ -1,0 +1,371 @@
+// The skinny product (up to 16 rows of x, bfloat16, MFMA, weights streamed once; see
+// skinny_gemm.hip for the mapping) with the neighbouring small operations of a decoding
+// step folded into its two ends, so that a layer takes six kernel launches instead of
+// nine.  At these sizes a launch costs as much as the work of a norm or a rotation.
+//
+// The norm between two products is split over them.  RMSNorm is x / rms(x) * weight
+// (src/models/turbo_generic.rs:41-51), and the division by the row's rms commutes with
+// the product that follows.  So the kernel that adds to the residual stream h (back end
+// "residual") also writes xw = bfloat16(h * weight of the next norm) and, per block, the
+// sum of h^2 over its 16 columns; the product that consumes the norm (front end "norm")
+// takes xw as it is, adds the blocks' sums up in their order, and divides its finished
+// sums by sqrt(mean + eps).  The statistics are those of the float32 stream.
+//
+// Back ends:
+//   store     y = result (bfloat16 or float32)
+//   gated     rows n and n_out + n of w are gate and up: y = silu(gate) * up
+//             (src/models/turbo_generic.rs:105-111)
+//   residual  h += bfloat16(result) in float32: the residual sum of
+//             src/models/turbo_generic.rs:1969, :1980; xw and the sums of squares as above
+//   qkv       rows are q heads, k heads, v heads of head_dim each; bias, rotation in the
+//             halves layout at the row's position (src/models/turbo_generic.rs:805-833,
+//             :417-427), q to q_out, k and v into the row's cache page
+//
+// Rounding points are those of the separate kernels (products rounded to bfloat16
+// before bias, rotation, gate or residual sum), so a decoded token and a prompt token
+// go through the same roundings except for the place of the norm's division.
+#include "common.h"
+#include "tq_kernels.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
+
+__device__ __forceinline__ bf16x8_t load8f(const bf16_t* p) {
+    return *reinterpret_cast<const bf16x8_t*>(p);
+}
+
+enum { EPI_STORE = 0, EPI_GATED = 1, EPI_RESIDUAL = 2, EPI_QKV = 3 };
+
+struct FusedArgs {
+    const bf16_t* x;            // [rows of x, K]
+    const int32_t* x_rows;      // row m of the product reads x row x_rows[m] (null: m)
+    const float* ss_parts;      // [n_ss_parts, 16] sums of squares of x's rows, in pieces (front end "norm")
+    int n_ss_parts;
+    float eps;
+    const bf16_t* w;            // [N, K]
+    int M, N, K;
+    // store / gated
+    void* y;
+    // residual
+    float* h;                   // [M, N]
+    const bf16_t* next_norm_w;  // [N] weight of the norm that follows, or null
+    bf16_t* xw_out;             // [M, N] bfloat16(h * next_norm_w), or bfloat16(h) without a weight
+    float* ss_out;              // [blocks, 16] this block's sum of h^2 per row, or null
+    // qkv
+    const bf16_t* bias;         // [N] or null
+    const float* cos_table;     // [max_positions, head_dim/2]
+    const float* sin_table;
+    const int32_t* tok_pos;     // [M]
+    const int32_t* page_table;  // [M, table_width]: row m is sequence m
+    int table_width, n_heads, n_kv_heads, head_dim, max_positions;
+    bf16_t* q_out;              // [M, n_heads, head_dim]
+    bf16_t* keys;               // [pages, kv heads, 64, head_dim]
+    bf16_t* values;             // [pages, kv heads, head_dim, 64 places]
+};
+
+#define SF_UNROLL 4
+
+template <bool NORM, int EPI, typename TY>
+__global__ __launch_bounds__(1024)
+void skinny_fused_kernel(const FusedArgs p) {
+    extern __shared__ float red[];                 // [waves][TILES * 4][64 lanes], then [waves][4 lanes] float4 of squares
+    constexpr int TILES = (EPI == EPI_GATED || EPI == EPI_QKV) ? 2 : 1;
+    constexpr int SLOTS = TILES * 4;
+    const int lane = threadIdx.x % TQK_WAVE, wave = threadIdx.x / TQK_WAVE;
+    const int n_waves = blockDim.x / TQK_WAVE;
+    const int row = lane % 16, kgrp = lane / 16;
+    const int K = p.K;
+
+    // which rows of w: n_lo (and n_hi for the second tile)
+    int n_lo0, n_hi0, n_out;
+    int head = 0, j16 = 0;
+    if (EPI == EPI_QKV) {
+        const int tiles_per_head = p.head_dim / 32;             // pairs of tiles (lo half, hi half)
+        head = blockIdx.x / tiles_per_head;
+        j16 = (blockIdx.x % tiles_per_head) * 16;
+        n_lo0 = head * p.head_dim + j16;
+        n_hi0 = n_lo0 + p.head_dim / 2;
+        n_out = p.N;
+    } else if (EPI == EPI_GATED) {
+        n_out = p.N / 2;
+        n_lo0 = blockIdx.x * 16;
+        n_hi0 = n_out + n_lo0;
+    } else {
+        n_out = p.N;
+        n_lo0 = blockIdx.x * 16;
+        n_hi0 = 0;
+    }
+    const int n_clamp = (EPI == EPI_GATED) ? n_out - 1 : p.N - 1;
+    const bf16_t* wrow[TILES];
+    wrow[0] = p.w + (size_t)min(n_lo0 + row, n_clamp) * K + kgrp * 8;
+    if (TILES == 2) wrow[1] = p.w + (size_t)(EPI == EPI_GATED ? n_out + min(n_lo0 + row, n_clamp) : n_hi0 + row) * K + kgrp * 8;
+
+    // Column m of the result depends on row m of x alone, so the lanes of rows past M read
+    // row 0 and their results are dropped.
+    const int xr = row < p.M ? (p.x_rows ? p.x_rows[row] : row) : 0;
+    const bf16_t* xrow = p.x + (size_t)xr * K + kgrp * 8;
+
+    // The sums of squares [n_ss_parts, 16 rows] as float4s: thread t takes the float4s t, t + threads, ...,
+    // which all hold rows 4*(t%4) .. +3.  The first is asked for here and used after the product.
+    const int n_ss4 = NORM ? p.n_ss_parts * 4 : 0;
+    const float4* ss4 = reinterpret_cast<const float4*>(p.ss_parts);
+    float4 ssq = make_float4(0.f, 0.f, 0.f, 0.f);
+    __builtin_amdgcn_sched_barrier(0);              // after the row's address is known: no wait covers this load
+    if (NORM && (int)threadIdx.x < n_ss4) ssq = ss4[threadIdx.x];
+
+    floatx4_t acc[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) acc[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    const int chunk = SF_UNROLL * 32;
+    const int n_chunks = K / chunk;
+    for (int c = wave; c < n_chunks; c += n_waves) {
+        const int k0 = c * chunk;
+        bf16x8_t a[TILES][SF_UNROLL], bx[SF_UNROLL];
+#pragma unroll
+        for (int u = 0; u < SF_UNROLL; ++u) {
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) a[t][u] = load8f(wrow[t] + k0 + u * 32);
+            bx[u] = load8f(xrow + k0 + u * 32);
+        }
+        __builtin_amdgcn_sched_barrier(0);          // every load of the chunk is on its way before the first product waits
+#pragma unroll
+        for (int u = 0; u < SF_UNROLL; ++u)
+#pragma unroll
+            for (int t = 0; t < TILES; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bx[u], acc[t], 0, 0, 0);
+    }
+    for (int s = n_chunks * SF_UNROLL + wave; s < K / 32; s += n_waves) {
+        const int k0 = s * 32;
+        const bf16x8_t bxs = load8f(xrow + k0);
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load8f(wrow[t] + k0), bxs, acc[t], 0, 0, 0);
+    }
+
+    if (NORM) {
+        for (int i = threadIdx.x + blockDim.x; i < n_ss4; i += blockDim.x) {
+            const float4 v = ss4[i];
+            ssq.x += v.x; ssq.y += v.y; ssq.z += v.z; ssq.w += v.w;
+        }
+        // lanes with equal lane%4 hold the same rows: add them up, fixed order
+#pragma unroll
+        for (int d = 4; d < TQK_WAVE; d *= 2) {
+            ssq.x += __shfl_xor(ssq.x, d, TQK_WAVE);
+            ssq.y += __shfl_xor(ssq.y, d, TQK_WAVE);
+            ssq.z += __shfl_xor(ssq.z, d, TQK_WAVE);
+            ssq.w += __shfl_xor(ssq.w, d, TQK_WAVE);
+        }
+    }
+
+    // add the waves' partial tiles up in wave order
+    if (n_waves > 1) {
+        float* mine = red + (size_t)wave * SLOTS * TQK_WAVE;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mine[(t * 4 + r) * TQK_WAVE + lane] = acc[t][r];
+        if (NORM && lane < 4) reinterpret_cast<float4*>(red + (size_t)n_waves * SLOTS * TQK_WAVE)[wave * 4 + lane] = ssq;
+        __syncthreads();
+        if (wave != 0) return;
+        for (int ww = 1; ww < n_waves; ++ww) {
+            const float* theirs = red + (size_t)ww * SLOTS * TQK_WAVE;
+#pragma unroll
+            for (int t = 0; t < TILES; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[t][r] += theirs[(t * 4 + r) * TQK_WAVE + lane];
+            if (NORM) {
+                const float4 v = reinterpret_cast<const float4*>(red + (size_t)n_waves * SLOTS * TQK_WAVE)[ww * 4 + lane % 4];
+                ssq.x += v.x; ssq.y += v.y; ssq.z += v.z; ssq.w += v.w;
+            }
+        }
+    }
+
+    // the lane holds column m = row of the result, for features n0 + 4*kgrp + r
+    const int m = row;
+    float inv_rms = 1.f;
+    if (NORM) {
+        // the lanes l with l%4 == xr/4 hold row xr's sum of squares in component xr%4
+        const float s0 = __shfl(ssq.x, xr / 4, TQK_WAVE), s1 = __shfl(ssq.y, xr / 4, TQK_WAVE);
+        const float s2 = __shfl(ssq.z, xr / 4, TQK_WAVE), s3 = __shfl(ssq.w, xr / 4, TQK_WAVE);
+        const float ss = (xr & 2) ? ((xr & 1) ? s3 : s2) : ((xr & 1) ? s1 : s0);
+        inv_rms = 1.f / sqrtf(ss / (float)K + p.eps);
+    }
+    if (m >= p.M && EPI != EPI_RESIDUAL) return;
+    const int nb = 4 * kgrp;
+
+    if constexpr (EPI == EPI_STORE) {
+        TY* y = (TY*)p.y;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int n = n_lo0 + nb + r;
+            if (n < p.N) y[(size_t)m * p.N + n] = from_float<TY>(acc[0][r] * inv_rms);
+        }
+    } else if constexpr (EPI == EPI_GATED) {
+        bf16_t* y = (bf16_t*)p.y;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int n = n_lo0 + nb + r;
+            if (n >= n_out) continue;
+            const float g = to_float(from_float<bf16_t>(acc[0][r] * inv_rms));
+            const float up = to_float(from_float<bf16_t>(acc[1][r] * inv_rms));
+            y[(size_t)m * n_out + n] = from_float<bf16_t>((g / (1.f + expf(-g))) * up);
+        }
+    } else if constexpr (EPI == EPI_RESIDUAL) {
+        float sq = 0.f;
+        if (m < p.M) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int n = n_lo0 + nb + r;
+                if (n >= p.N) continue;
+                const size_t at = (size_t)m * p.N + n;
+                const float v = p.h[at] + to_float(from_float<bf16_t>(acc[0][r]));
+                p.h[at] = v;
+                sq = fmaf(v, v, sq);
+                p.xw_out[at] = from_float<bf16_t>(p.next_norm_w ? v * to_float(p.next_norm_w[n]) : v);
+            }
+        }
+        if (p.ss_out) {
+            // this block's 16 columns of row m: the four lanes of the row, in lane order
+            const float s1 = __shfl_xor(sq, 16, TQK_WAVE);
+            const float s2 = __shfl_xor(sq, 32, TQK_WAVE);
+            const float s3 = __shfl_xor(s1, 32, TQK_WAVE);
+            if (kgrp == 0 && m < p.M) p.ss_out[(size_t)blockIdx.x * 16 + m] = ((sq + s1) + s2) + s3;
+        }
+    } else {    // EPI_QKV
+        const int d = p.head_dim, half = d / 2;
+        const int kind = head < p.n_heads ? 0 : (head < p.n_heads + p.n_kv_heads ? 1 : 2);
+        const int pos = p.tok_pos[m];
+        bf16_t* dst;
+        size_t stride = 1;
+        if (kind == 0) {
+            dst = p.q_out + ((size_t)m * p.n_heads + head) * d;
+        } else {
+            const int kvh = kind == 1 ? head - p.n_heads : head - p.n_heads - p.n_kv_heads;
+            const int page = p.page_table[(size_t)m * p.table_width + pos / TQK_PAGE];
+            if (page < 0) return;                   // the host never lets this happen
+            const size_t base = ((size_t)page * p.n_kv_heads + kvh) * TQK_PAGE * d;
+            if (kind == 1) dst = p.keys + base + (size_t)(pos % TQK_PAGE) * d;
+            else { dst = p.values + base + value_place(pos % TQK_PAGE); stride = TQK_PAGE; }
+        }
+        const bool rotate = kind != 2 && pos < p.max_positions;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int i_lo = j16 + nb + r, i_hi = i_lo + half;          // elements inside the head
+            float lo = to_float(from_float<bf16_t>(acc[0][r] * inv_rms));
+            float hi = to_float(from_float<bf16_t>(acc[1][r] * inv_rms));
+            if (p.bias) {
+                lo += to_float(p.bias[head * d + i_lo]);
+                hi += to_float(p.bias[head * d + i_hi]);
+            }
+            if (rotate) {
+                const float c = p.cos_table[(size_t)pos * half + i_lo], s = p.sin_table[(size_t)pos * half + i_lo];
+                const float r0 = lo * c - hi * s, r1 = lo * s + hi * c;
+                lo = r0; hi = r1;
+            }
+            dst[(size_t)i_lo * stride] = from_float<bf16_t>(lo);
+            dst[(size_t)i_hi * stride] = from_float<bf16_t>(hi);
+        }
+    }
+}
+
+static int pick_waves(int blocks, int K, int tiles) {
+    const int chunks = K / (SF_UNROLL * 32) > 0 ? K / (SF_UNROLL * 32) : 1;
+    const int max_waves = tiles == 2 ? 8 : 16;
+    int waves = 1;
+    while (waves < max_waves && blocks * waves < 1024 && waves * 2 <= chunks) waves *= 2;
+    return waves;
+}
+
+template <bool NORM, int EPI, typename TY>
+static int launch_fused(const FusedArgs& a, int blocks, hipStream_t s) {
+    const int tiles = (EPI == EPI_GATED || EPI == EPI_QKV) ? 2 : 1;
+    const int waves = pick_waves(blocks, a.K, tiles);
+    const size_t lds = waves > 1 ? (size_t)waves * (tiles * 4) * TQK_WAVE * sizeof(float) + (NORM ? (size_t)waves * 16 * sizeof(float) : 0) : 0;
+    skinny_fused_kernel<NORM, EPI, TY><<<blocks, waves * TQK_WAVE, lds, s>>>(a);
+    return tqk_check_launch("tqk_skinny_fused");
+}
+
+static int check_common(const FusedArgs& a, const char* what) {
+    TQK_REQUIRE(a.x && a.w, "%s: null pointer", what);
+    TQK_REQUIRE(a.M >= 0 && a.M <= 16, "%s: M=%d rows, this kernel takes at most 16", what, a.M);
+    TQK_REQUIRE(a.N > 0 && a.K > 0 && a.K % 32 == 0, "%s: K=%d must be a positive multiple of 32 (N=%d)", what, a.K, a.N);
+    TQK_REQUIRE((((uintptr_t)a.x) & 15) == 0 && (((uintptr_t)a.w) & 15) == 0, "%s: x and w must be 16-byte aligned", what);
+    TQK_REQUIRE(!a.ss_parts || a.n_ss_parts > 0, "%s: sums of squares given in %d pieces", what, a.n_ss_parts);
+    TQK_REQUIRE((((uintptr_t)a.ss_parts) & 15) == 0, "%s: the sums of squares must be 16-byte aligned", what);
+    return 0;
+}
+
+/* y[M,N] = x w^T, or with ss_parts (the sums of squares of the stream's rows in n_ss_parts
+ * pieces of 16 rows each; x is then the stream times the norm's weight) that divided by
+ * sqrt(sum / K + eps).  x_rows (optional) picks the rows of x. */
+extern "C" int tqk_fused_store(const void* x, const int32_t* x_rows, const float* ss_parts, int n_ss_parts, float eps,
+                               const void* w, void* y, int y_dtype, int M, int N, int K, void* stream) {
+    FusedArgs a = {};
+    a.x = (const bf16_t*)x; a.x_rows = x_rows; a.ss_parts = ss_parts; a.n_ss_parts = n_ss_parts; a.eps = eps;
+    a.w = (const bf16_t*)w; a.M = M; a.N = N; a.K = K; a.y = y;
+    if (check_common(a, "tqk_fused_store")) return -1;
+    TQK_REQUIRE(y, "tqk_fused_store: null output");
+    TQK_REQUIRE(y_dtype == TQK_F32 || y_dtype == TQK_BF16, "tqk_fused_store: unknown output dtype %d", y_dtype);
+    if (M == 0) return 0;
+    const int blocks = (N + 15) / 16;
+    hipStream_t s = (hipStream_t)stream;
+    if (ss_parts) return y_dtype == TQK_F32 ? launch_fused<true, EPI_STORE, float>(a, blocks, s) : launch_fused<true, EPI_STORE, bf16_t>(a, blocks, s);
+    return y_dtype == TQK_F32 ? launch_fused<false, EPI_STORE, float>(a, blocks, s) : launch_fused<false, EPI_STORE, bf16_t>(a, blocks, s);
+}
+
+/* y[M, N/2] = silu(gate) * up of the (normalised) product, w = gate rows then up rows. */
+extern "C" int tqk_fused_gated(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, void* y,
+                               int M, int N, int K, void* stream) {
+    FusedArgs a = {};
+    a.x = (const bf16_t*)x; a.ss_parts = ss_parts; a.n_ss_parts = n_ss_parts; a.eps = eps; a.w = (const bf16_t*)w;
+    a.M = M; a.N = N; a.K = K; a.y = y;
+    if (check_common(a, "tqk_fused_gated")) return -1;
+    TQK_REQUIRE(y && N % 2 == 0, "tqk_fused_gated: null output or odd N=%d", N);
+    if (M == 0) return 0;
+    const int blocks = (N / 2 + 15) / 16;
+    hipStream_t s = (hipStream_t)stream;
+    return ss_parts ? launch_fused<true, EPI_GATED, bf16_t>(a, blocks, s) : launch_fused<false, EPI_GATED, bf16_t>(a, blocks, s);
+}
+
+extern "C" int tqk_fused_residual_parts(int N) { return (N + 15) / 16; }
+
+/* h[M,N] += bfloat16(x w^T) in float32; xw_out = bfloat16(h * next_norm_w) (bfloat16(h)
+ * without a weight); ss_out (optional) [tqk_fused_residual_parts(N), 16]: piece b, row m =
+ * sum of h[m, 16b..16b+15]^2. */
+extern "C" int tqk_fused_residual(const void* x, const void* w, float* h, const void* next_norm_w, void* xw_out,
+                                  float* ss_out, int M, int N, int K, void* stream) {
+    FusedArgs a = {};
+    a.x = (const bf16_t*)x; a.w = (const bf16_t*)w; a.M = M; a.N = N; a.K = K; a.h = h;
+    a.next_norm_w = (const bf16_t*)next_norm_w; a.xw_out = (bf16_t*)xw_out; a.ss_out = ss_out;
+    if (check_common(a, "tqk_fused_residual")) return -1;
+    TQK_REQUIRE(h && xw_out, "tqk_fused_residual: null output");
+    if (M == 0) return 0;
+    return launch_fused<false, EPI_RESIDUAL, bf16_t>(a, (N + 15) / 16, (hipStream_t)stream);
+}
+
+/* The q, k, v product of a decoding step: the (normalised) product + bias, q and k rotated
+ * (halves layout over the whole head) at tok_pos[m], q to q_out, k and v into the page of
+ * row m's sequence (row m of page_table).  head_dim must be a multiple of 32. */
+extern "C" int tqk_fused_qkv(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, const void* bias,
+                             const float* cos_table, const float* sin_table, int max_positions,
+                             const int32_t* tok_pos, const int32_t* page_table, int table_width,
+                             void* keys, void* values, int n_pages, void* q_out,
+                             int M, int n_heads, int n_kv_heads, int head_dim, int K, void* stream) {
+    FusedArgs a = {};
+    a.x = (const bf16_t*)x; a.ss_parts = ss_parts; a.n_ss_parts = n_ss_parts; a.eps = eps; a.w = (const bf16_t*)w;
+    a.M = M; a.N = (n_heads + 2 * n_kv_heads) * head_dim; a.K = K;
+    a.bias = (const bf16_t*)bias; a.cos_table = cos_table; a.sin_table = sin_table; a.max_positions = max_positions;
+    a.tok_pos = tok_pos; a.page_table = page_table; a.table_width = table_width;
+    a.n_heads = n_heads; a.n_kv_heads = n_kv_heads; a.head_dim = head_dim;
+    a.q_out = (bf16_t*)q_out; a.keys = (bf16_t*)keys; a.values = (bf16_t*)values;
+    TQK_REQUIRE(n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && head_dim % 32 == 0,
+                "tqk_fused_qkv: head_dim %d must be a positive multiple of 32", head_dim);
+    if (check_common(a, "tqk_fused_qkv")) return -1;
+    TQK_REQUIRE(cos_table && sin_table && max_positions > 0 && tok_pos && page_table && keys && values && q_out,
+                "tqk_fused_qkv: null pointer");
+    TQK_REQUIRE(table_width > 0 && n_pages > 0, "tqk_fused_qkv: empty page table");
+    if (M == 0) return 0;
+    const int blocks = (n_heads + 2 * n_kv_heads) * (head_dim / 32);
+    hipStream_t s = (hipStream_t)stream;
+    return ss_parts ? launch_fused<true, EPI_QKV, bf16_t>(a, blocks, s) : launch_fused<false, EPI_QKV, bf16_t>(a, blocks, s);
+}

@@ -18,9 +18,12 @@ extern "C" {
 const char* tqk_last_error(void);
 int tqk_abi_version(void);
 
-/* out[t, :] = float(table[ids[t], :]); ids outside [0, vocab) give zeros. */
+/* out[t, :] = float(table[ids[t], :]); ids outside [0, vocab) give zeros.  copy_bf16
+ * (optional): the same values as bfloat16 [tokens, hidden], times copy_weight [hidden]
+ * (bfloat16) if given.  ss_out (optional, at most 16 tokens): ss_out[t] = sum of out[t]^2. */
 int tqk_embed(const void* table, int table_dtype, const int32_t* ids, int n_tokens,
-              int hidden, int vocab, float* out, void* stream);
+              int hidden, int vocab, float* out, void* copy_bf16, const void* copy_weight,
+              float* ss_out, void* stream);
 
 /* Row r (row index rows[r], or r if rows is NULL):
  *   v = (h ? h[row] : 0) + (delta ? delta[row] : 0);  if write_back: h[row] = v;
@@ -40,6 +43,29 @@ int tqk_gemm(const void* x, int x_dtype, const void* w, int w_dtype, const void*
  * (N = 2*inter), y[M,inter] = silu(gate)*up (bfloat16).  K must be a multiple of 32. */
 int tqk_skinny_bf16(const void* x, const void* w, void* y, int y_dtype, int M, int N, int K,
                     int epilogue, void* stream);
+
+/* Skinny products (up to 16 rows, bfloat16, K a multiple of 32) with the small operations
+ * around them folded in.  A norm between two products is split over them: the one that adds
+ * to the stream h writes xw = bfloat16(h * weight of the next norm) and the sums of h^2 in
+ * pieces (tqk_fused_residual, tqk_embed); the one that consumes the norm takes xw and the
+ * pieces (ss_parts [n_ss_parts, 16]) and divides its result by sqrt(sum / K + eps). */
+int tqk_fused_store(const void* x, const int32_t* x_rows, const float* ss_parts, int n_ss_parts, float eps,
+                    const void* w, void* y, int y_dtype, int M, int N, int K, void* stream);
+/* y[M, N/2] = silu(gate) * up, w = gate rows then up rows */
+int tqk_fused_gated(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, void* y,
+                    int M, int N, int K, void* stream);
+/* h[M,N] += bfloat16(x w^T) in float32; xw_out = bfloat16(h * next_norm_w) or bfloat16(h);
+ * ss_out (optional) [tqk_fused_residual_parts(N), 16] */
+int tqk_fused_residual_parts(int N);
+int tqk_fused_residual(const void* x, const void* w, float* h, const void* next_norm_w, void* xw_out,
+                       float* ss_out, int M, int N, int K, void* stream);
+/* q, k, v of a decoding step: + bias, rotation (halves over the whole head) at tok_pos[m],
+ * q to q_out [M, heads, head_dim], k and v into the cache page of sequence m */
+int tqk_fused_qkv(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, const void* bias,
+                  const float* cos_table, const float* sin_table, int max_positions,
+                  const int32_t* tok_pos, const int32_t* page_table, int table_width,
+                  void* keys, void* values, int n_pages, void* q_out,
+                  int M, int n_heads, int n_kv_heads, int head_dim, int K, void* stream);
 
 /* For each token t and head: add bias, rotate q and k heads by the angle table row
  * tok_pos[t] (style 0: none, 1: halves (j, j+rot/2), 2: pairs (2j, 2j+1)), write q to

@@ -84,6 +84,7 @@ class StepContext:
         host.tile_count = np.asarray([t_count[k] for k in order], dtype=np.int32)
         self.host = host
         self.all_decode = all(n == 1 for n in lens)
+        self.fuse_small = False      # set by the model for small decoding steps in bfloat16
         self.max_new = max(lens)
         self.max_end = int((host.seq_start + host.seq_new).max())
         self.groups = list(cache.kv_groups) if cache is not None else []

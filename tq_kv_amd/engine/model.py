@@ -9,6 +9,7 @@ from .. import kernels as K
 from ..config import catalog
 from ..config.base import ConfigError, read_config_json
 from ..config.registry import config_from_dict, spec_for
+from ..parts import linear as L
 from ..parts.linear import linear
 from ..parts.registry import BuildEnv
 from ..parts.spec import TensorSpec
@@ -40,6 +41,10 @@ class Model:
                 raise ValueError("run %d reads the cache of run %r, which is not an earlier run" % (i, run.cache_of))
         self.needs = [self.blocks[run.layer].cache_need() for run in spec.order]
         self.cache_of = [run.cache_of for run in spec.order]
+        for run in spec.order:
+            mixer = getattr(self.blocks[run.layer], "mixer", None)
+            if run.cache_of is not None and hasattr(mixer, "reads_other_cache"):
+                mixer.reads_other_cache = True
         self.embedding = None
         self.head = None
         self.loaded = False
@@ -136,14 +141,35 @@ class Model:
             raise RuntimeError("the model has no weights yet")
         s = self.spec
         h = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.float32, device=self.device)
-        K.embed(self.embedding, ctx.dev.tokens, h)
-        delta = None
+        # small decoding steps: products fold the norms and the residual sums around them in
+        ctx.fuse_small = (L.POLICY["fused"] and self.dtype == torch.bfloat16 and ctx.all_decode
+                          and ctx.n_tokens <= 16 and s.hidden_size % 32 == 0)
+        firsts = [self.blocks[run.layer].first_norm() if hasattr(self.blocks[run.layer], "first_norm") else None
+                  for run in s.order] + [self.final_norm]
+        if ctx.fuse_small:
+            xw = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.bfloat16, device=self.device)
+            ss = torch.empty((max(1, K.fused_residual_parts(s.hidden_size)), 16), dtype=torch.float32, device=self.device)
+            stream = L.Stream(h, xw, ss)
+            norm = firsts[0] if getattr(firsts[0], "foldable", False) else None
+            K.embed(self.embedding, ctx.dev.tokens, h, copy=xw, copy_weight=norm.weight if norm is not None else None, ss_out=ss)
+            stream.xw_for, stream.n_ss = norm, 1
+        else:
+            stream = L.Stream(h)
+            K.embed(self.embedding, ctx.dev.tokens, h)
         for i, run in enumerate(s.order):
-            delta = self.blocks[run.layer].forward(h, delta, ctx, cache.entry(i))
+            block = self.blocks[run.layer]
+            if hasattr(block, "first_norm"):
+                block.forward(stream, ctx, cache.entry(i), next_norm=firsts[i + 1])
+            else:
+                block.forward(stream, ctx, cache.entry(i))
         n_rows = ctx.dev.want_rows.shape[0]
         if n_rows == 0:
             return torch.empty((0, s.vocab_size), dtype=torch.float32, device=self.device)
-        x = self.final_norm.gather_add_norm(h, delta, ctx.dev.want_rows)
+        lazy = self.final_norm.lazy(stream) if ctx.fuse_small and hasattr(self.final_norm, "lazy") else None
+        if lazy is not None and n_rows <= 16 and L.fusable(n_rows, self.head):
+            logits = torch.empty((n_rows, s.vocab_size), dtype=torch.float32, device=self.device)
+            return K.fused_store(lazy.xw, self.head, logits, lazy.norm, rows=ctx.dev.want_rows)
+        x = self.final_norm.gather_add_norm(stream.h, stream.pending, ctx.dev.want_rows)
         return linear(x, self.head, out_dtype=torch.float32)
 
     def __repr__(self):

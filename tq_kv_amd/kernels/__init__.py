@@ -76,12 +76,19 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def embed(table, ids, out):
-    """out[t] = float32(table[ids[t]]);  table [V,H], ids [T] int32, out [T,H] float32."""
+def embed(table, ids, out, copy=None, copy_weight=None, ss_out=None):
+    """out[t] = float32(table[ids[t]]);  table [V,H], ids [T] int32, out [T,H] float32.
+    copy (optional): the same as bfloat16 [T,H], times copy_weight [H] if given; ss_out
+    (optional, float32, at least T values, T <= 16): sums of squares of the rows."""
     vocab, hidden = table.shape
     n = ids.shape[0]
+    if ss_out is not None and ss_out.numel() < max(n, 1):
+        raise KernelError("embed: ss_out holds %d values for %d tokens" % (ss_out.numel(), n))
     _check(library().tqk_embed(_dev(table, "table"), _code(table.dtype), _dev(ids, "ids", torch.int32, (n,)),
-                               n, hidden, vocab, _dev(out, "out", torch.float32, (n, hidden)), _stream()),
+                               n, hidden, vocab, _dev(out, "out", torch.float32, (n, hidden)),
+                               _opt(copy, "copy", torch.bfloat16, (n, hidden)),
+                               _opt(copy_weight, "copy_weight", torch.bfloat16, (hidden,)),
+                               _opt(ss_out, "ss_out", torch.float32), _stream()),
            "embed")
     return out
 
@@ -276,3 +283,84 @@ def attention_prefill(q, keys, values, tok_pos, page_table, tile_seq, tile_tok0,
         int(window or 0), ctypes.c_float(scale), _dev(out, "out", torch.bfloat16, (n, n_heads * head_dim)),
         n, n_heads, n_kv_heads, head_dim, _stream()), "attention_prefill")
     return out
+
+
+# ---- skinny products with the neighbouring small operations folded in (decoding) ---------------
+# A norm between two products is split over them: `fused_residual` (or `embed`) writes the
+# stream times the next norm's weight and the rows' sums of squares in pieces; the consuming
+# product gets both as `norm=(ss_parts, n_parts, eps)` and divides its result by the rows' rms.
+def _norm_args(norm, m):
+    if norm is None:
+        return ctypes.c_void_p(0), 0, ctypes.c_float(0.0)
+    ss_parts, n_parts, eps = norm
+    if ss_parts.dtype != torch.float32 or ss_parts.numel() < 16 * n_parts or n_parts < 1:
+        raise KernelError("sums of squares: %d float32 values for %d pieces of 16 rows" % (ss_parts.numel(), n_parts))
+    return _dev(ss_parts, "ss_parts", torch.float32), int(n_parts), ctypes.c_float(eps)
+
+
+def fused_store(x, weight, out, norm=None, rows=None):
+    """out[M,N] = x weight^T (divided by the rows' rms with `norm`); x bfloat16 [*, K]
+    (rows: int32 indices of the M rows used)."""
+    m, n = out.shape
+    k = weight.shape[1]
+    if x.shape[1] != k or (rows is None and x.shape[0] != m) or x.shape[0] > 16:
+        raise KernelError("fused_store: x is %s for %d rows of %d (at most 16 rows)" % (tuple(x.shape), m, k))
+    ss, n_parts, eps = _norm_args(norm, m)
+    _check(library().tqk_fused_store(
+        _dev(x, "x", torch.bfloat16), _opt(rows, "rows", torch.int32, (m,)), ss, n_parts, eps,
+        _dev(weight, "weight", torch.bfloat16, (n, k)), _dev(out, "out"), _code(out.dtype), m, n, k, _stream()), "fused_store")
+    return out
+
+
+def fused_gated(x, weight_gate_up, out, norm=None):
+    """out[M, I] = silu(gate) * up of x [gate; up]^T (normalised with `norm`)."""
+    m, inter = out.shape
+    k = weight_gate_up.shape[1]
+    ss, n_parts, eps = _norm_args(norm, m)
+    _check(library().tqk_fused_gated(
+        _dev(x, "x", torch.bfloat16, (m, k)), ss, n_parts, eps,
+        _dev(weight_gate_up, "weight", torch.bfloat16, (2 * inter, k)), _dev(out, "out", torch.bfloat16), m, 2 * inter, k,
+        _stream()), "fused_gated")
+    return out
+
+
+def fused_residual_parts(n):
+    return int(library().tqk_fused_residual_parts(int(n)))
+
+
+def fused_residual(x, weight, h, xw, next_norm_weight=None, ss_out=None):
+    """h[M,N] += bfloat16(x weight^T) (float32 sum); xw = bfloat16(h * next_norm_weight) (or
+    bfloat16(h)); ss_out (optional, float32 [fused_residual_parts(N), 16]): the rows' sums of
+    squares in pieces.  Returns the number of pieces."""
+    m, k = x.shape
+    n = weight.shape[0]
+    parts = fused_residual_parts(n)
+    if ss_out is not None and ss_out.numel() < parts * 16:
+        raise KernelError("fused_residual: ss_out holds %d values, %d pieces of 16 are written" % (ss_out.numel(), parts))
+    _check(library().tqk_fused_residual(
+        _dev(x, "x", torch.bfloat16), _dev(weight, "weight", torch.bfloat16, (n, k)), _dev(h, "h", torch.float32, (m, n)),
+        _opt(next_norm_weight, "next_norm_weight", torch.bfloat16, (n,)), _dev(xw, "xw", torch.bfloat16, (m, n)),
+        _opt(ss_out, "ss_out", torch.float32), m, n, k, _stream()), "fused_residual")
+    return parts
+
+
+def fused_qkv(x, weight, bias, cos, sin, tok_pos, page_table, keys, values, q_out, n_heads, n_kv_heads, head_dim,
+              norm=None):
+    """q, k, v of a decoding step (row m is sequence m): product (normalised with `norm`),
+    bias, rotation, q out, k and v into the cache pages."""
+    m, k = x.shape
+    total = (n_heads + 2 * n_kv_heads) * head_dim
+    n_pages = keys.shape[0]
+    width = page_table.shape[1]
+    max_pos = cos.shape[0]
+    ss, n_parts, eps = _norm_args(norm, m)
+    _check(library().tqk_fused_qkv(
+        _dev(x, "x", torch.bfloat16), ss, n_parts, eps,
+        _dev(weight, "weight", torch.bfloat16, (total, k)), _opt(bias, "bias", torch.bfloat16, (total,)),
+        _dev(cos, "cos", torch.float32, (max_pos, head_dim // 2)), _dev(sin, "sin", torch.float32, (max_pos, head_dim // 2)), max_pos,
+        _dev(tok_pos, "tok_pos", torch.int32, (m,)), _dev(page_table, "page_table", torch.int32, (m, width)), width,
+        _dev(keys, "keys", torch.bfloat16, (n_pages, n_kv_heads, 64, head_dim)),
+        _dev(values, "values", torch.bfloat16, (n_pages, n_kv_heads, head_dim, 64)), n_pages,
+        _dev(q_out, "q_out", torch.bfloat16, (m, n_heads, head_dim)), m, n_heads, n_kv_heads, head_dim, k, _stream()),
+        "fused_qkv")
+    return q_out

@@ -11,7 +11,7 @@ import math
 import torch
 
 from .. import kernels as K
-from .linear import linear
+from .linear import LazyNorm, fusable, linear
 from .registry import Part, register
 from .spec import KVNeed, TensorSpec
 
@@ -45,6 +45,7 @@ class Attention(Part):
         self.position = env.shared[key]
         self.graph_safe = not hasattr(self.position, "apply") or getattr(self.position, "graph_safe", False)
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+        self.reads_other_cache = False      # set when a run of this layer reads another run's cache
 
     def tensors(self):
         q, kv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
@@ -73,11 +74,49 @@ class Attention(Part):
     def product_weights(self):
         return [(self.w_qkv, None), (self.w_o, None)]
 
-    def forward(self, x, ctx, entry):
-        n = x.shape[0]
-        qkv = linear(x, self.w_qkv)
+    def _fused_qkv_ok(self, ctx):
+        """The folded q/k/v kernel takes decoding steps (row m is sequence m) of rotary
+        positions in the halves layout over the whole head."""
+        if not (ctx.all_decode and fusable(ctx.n_tokens, self.w_qkv) and self.head_dim % 32 == 0):
+            return False
+        if hasattr(self.position, "apply"):
+            return False
+        cos, _, rot_dim, style = self.position.tables()
+        if style != K.STYLE_HALVES or rot_dim != self.head_dim:
+            return False
+        return self.b_qkv is None or self.b_qkv.dtype == torch.bfloat16
+
+    def folds_norm(self, ctx):
+        return self._fused_qkv_ok(ctx) and not self.reads_other_cache
+
+    def adds_to_stream(self, ctx):
+        return fusable(ctx.n_tokens, self.w_o) and self.b_o is None
+
+    def forward(self, x, ctx, entry, stream=None):
+        lazy = isinstance(x, LazyNorm)
+        n = x.xw.shape[0] if lazy else x.shape[0]
+        dtype = torch.bfloat16 if lazy else x.dtype
         table = ctx.page_table(entry.group)
-        q = torch.empty((n, self.n_heads, self.head_dim), dtype=x.dtype, device=x.device)
+        q = torch.empty((n, self.n_heads, self.head_dim), dtype=dtype, device=self.w_qkv.device)
+        if lazy or (ctx.fuse_small and entry.writes and self._fused_qkv_ok(ctx)):
+            if lazy and not entry.writes:
+                raise RuntimeError("a run that reads another run's cache cannot take a folded norm")
+            cos, sin, _, _ = self.position.tables()
+            K.fused_qkv(x.xw if lazy else x, self.w_qkv, self.b_qkv, cos, sin, ctx.dev.tok_pos, table,
+                        entry.keys, entry.values, q, self.n_heads, self.n_kv_heads, self.head_dim,
+                        norm=x.norm if lazy else None)
+        else:
+            self._qkv(x, ctx, entry, table, q)
+        y = torch.empty((n, self.n_heads * self.head_dim), dtype=dtype, device=q.device)
+        attend(q, entry, table, ctx, self.window, self.scale, y)
+        if stream is not None:
+            stream.add_product(y, self.w_o)
+            return None
+        return linear(y, self.w_o, self.b_o)
+
+    def _qkv(self, x, ctx, entry, table, q):
+        """Product, then bias, position encoding and cache write in their own kernel."""
+        qkv = linear(x, self.w_qkv)
         if hasattr(self.position, "apply"):
             # a position encoding of its own: bias first, then it changes q and k in place
             if self.b_qkv is not None:
@@ -93,9 +132,6 @@ class Attention(Part):
         K.rope_store(qkv, bias, cos, sin, rot_dim, style, ctx.dev.tok_seq, ctx.dev.tok_pos, table,
                      entry.keys, entry.values, q, self.n_heads, self.n_kv_heads, self.head_dim,
                      write_kv=entry.writes)
-        y = torch.empty((n, self.n_heads * self.head_dim), dtype=x.dtype, device=x.device)
-        attend(q, entry, table, ctx, self.window, self.scale, y)
-        return linear(y, self.w_o, self.b_o)
 
 
 # The bfloat16 attention kernels can be switched off one by one (tests compare each with

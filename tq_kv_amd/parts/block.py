@@ -4,9 +4,12 @@
 x = x + mixer(norm(x)); x = x + ff(norm(x)), with optional norms on the mixer's and
 the feed-forward's outputs (:1965-1968, :1976-1979).
 
-The residual stream h is float32.  A block receives h and the previous block's
-update that has not been added yet, and returns its own last update the same way, so
-that each addition happens inside the next norm's kernel.
+The residual stream is float32 (parts.linear.Stream).  A part's output is left pending
+on the stream and added inside the next norm's kernel.  In small decoding steps the
+framework's parts go further: a product that consumes a norm computes it itself
+(LazyNorm) and a part's last product adds its result to the stream in its epilogue, so
+that the norm kernels disappear; parts that do not offer this (`folds_norm`,
+`adds_to_stream`) are simply given tensors.
 """
 from .registry import Part, register
 
@@ -58,13 +61,38 @@ class PreNormBlock(Part):
     def product_weights(self):
         return [w for part in self.parts.values() for w in part.product_weights()]
 
-    def forward(self, h, delta, ctx, entry):
-        x = self.mixer_norm.add_norm(h, delta)
-        a = self.mixer.forward(x, ctx, entry)
-        if self.post_mixer_norm is not None:
-            a = self.post_mixer_norm.forward(a)
-        x = self.ff_norm.add_norm(h, a)
-        f = self.feed_forward.forward(x, ctx)
-        if self.post_ff_norm is not None:
-            f = self.post_ff_norm.forward(f)
-        return f
+    def first_norm(self):
+        """The norm that reads the stream first when this block runs."""
+        return self.mixer_norm
+
+    def _normed(self, norm, stream, part, ctx):
+        """The part's input: the norm of the stream, computed now, or left to the part."""
+        if ctx.fuse_small and getattr(part, "folds_norm", None) and part.folds_norm(ctx):
+            lazy = norm.lazy(stream)
+            if lazy is not None:
+                return lazy
+        x = norm.add_norm(stream.h, stream.pending)
+        stream.pending = None
+        stream.invalidate()
+        return x
+
+    def _run(self, part, post_norm, next_norm, x, stream, ctx, *extra):
+        """Run a part; its output is added to the stream by the part itself (it returns None)
+        or is left pending for the next norm's kernel."""
+        if ctx.fuse_small and post_norm is None and getattr(part, "adds_to_stream", None) and part.adds_to_stream(ctx):
+            stream.next_norm = next_norm
+            out = part.forward(x, ctx, *extra, stream=stream)
+        else:
+            out = part.forward(x, ctx, *extra)
+        if out is not None:
+            if post_norm is not None:
+                out = post_norm.forward(out)
+            stream.pending = out
+            stream.invalidate()
+
+    def forward(self, stream, ctx, entry, next_norm=None):
+        """next_norm: the norm that reads the stream after this block."""
+        x = self._normed(self.mixer_norm, stream, self.mixer, ctx)
+        self._run(self.mixer, self.post_mixer_norm, self.ff_norm, x, stream, ctx, entry)
+        x = self._normed(self.ff_norm, stream, self.feed_forward, ctx)
+        self._run(self.feed_forward, self.post_ff_norm, next_norm, x, stream, ctx)

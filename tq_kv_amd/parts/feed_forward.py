@@ -3,7 +3,8 @@
 up are one product with the weights stacked."""
 import torch
 
-from .linear import gated_silu_linear, linear
+from .. import kernels as K
+from .linear import LazyNorm, fusable, gated_silu_linear, linear
 from .registry import Part, register
 from .spec import TensorSpec
 
@@ -32,5 +33,20 @@ class GatedSiLU(Part):
     def product_weights(self):
         return [(self.w_gate_up, None), (self.w_down, None)]
 
-    def forward(self, x, ctx):
+    def folds_norm(self, ctx):
+        return fusable(ctx.n_tokens, self.w_gate_up)
+
+    def adds_to_stream(self, ctx):
+        return fusable(ctx.n_tokens, self.w_down) and fusable(ctx.n_tokens, self.w_gate_up)
+
+    def forward(self, x, ctx, stream=None):
+        lazy = isinstance(x, LazyNorm)
+        if lazy or stream is not None:
+            xin = x.xw if lazy else x
+            act = torch.empty((xin.shape[0], self.inter), dtype=torch.bfloat16, device=self.w_down.device)
+            K.fused_gated(xin, self.w_gate_up, act, x.norm if lazy else None)
+            if stream is None:
+                return linear(act, self.w_down)
+            stream.add_product(act, self.w_down)
+            return None
         return linear(gated_silu_linear(x, self.w_gate_up), self.w_down)

@@ -19,7 +19,49 @@ from .. import kernels as K
 # plain kernel); nothing else reads these.
 # Measured on MI355X at the Qwen2.5-7B sizes: up to 16 rows the skinny kernel is ahead of the
 # library on every product; at 64 rows the library is ahead on every one.
-POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16}
+POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16, "fused": True}
+
+
+class Stream:
+    """The residual stream of a step.  h: float32 [tokens, hidden].  pending: an update (of
+    the activation dtype) that has not been added to h yet, or None.
+
+    In small decoding steps the kernels that add to h also prepare the next norm: xw is
+    bfloat16(h * weight of norm `xw_for`) and ss the rows' sums of squares in n_ss pieces
+    (valid only while nothing is pending).  next_norm is set by whoever runs a part, to the
+    norm that will read the stream after that part."""
+
+    def __init__(self, h, xw_buffer=None, ss_buffer=None):
+        self.h, self.pending = h, None
+        self.xw_buffer, self.ss_buffer = xw_buffer, ss_buffer
+        self.xw_for, self.n_ss = None, 0
+        self.next_norm = None
+
+    def add_product(self, x, weight):
+        """h += bfloat16(x weight^T) in the product's epilogue, preparing next_norm."""
+        norm = self.next_norm if getattr(self.next_norm, "foldable", False) else None
+        self.n_ss = K.fused_residual(x, weight, self.h, self.xw_buffer,
+                                     norm.weight if norm is not None else None, self.ss_buffer)
+        self.xw_for = norm
+        self.pending = None
+
+    def invalidate(self):
+        self.xw_for = None
+
+
+class LazyNorm:
+    """An RMSNorm of the stream that has not been computed: xw is the stream times the norm's
+    weight, norm = (sums of squares in pieces, number of pieces, eps); the product that takes
+    it divides its result by the rows' rms."""
+
+    def __init__(self, xw, ss, n_ss, eps):
+        self.xw, self.norm = xw, (ss, n_ss, eps)
+
+
+def fusable(x_rows, weight):
+    """Whether the folded skinny kernels take a product of x_rows rows with this weight."""
+    return (POLICY["fused"] and POLICY["skinny"] and x_rows <= 16 and weight.dtype == torch.bfloat16
+            and weight.shape[1] % 32 == 0)
 
 
 def tune_library(on=True, seconds=30):

@@ -30,6 +30,19 @@ class RMSNorm(Part):
         out = torch.empty_like(x)
         return K.add_rmsnorm(None, x, self.weight, self.eps, out)
 
+    @property
+    def foldable(self):
+        """Whether the kernels that add to the stream can prepare this norm (bfloat16 weight)."""
+        return self.weight is not None and self.weight.dtype == torch.bfloat16
+
+    def lazy(self, stream):
+        """The norm of the stream, left to the product that consumes it: possible if the
+        kernel that last added to the stream prepared it for this norm."""
+        from .linear import LazyNorm
+        if stream.pending is not None or stream.xw_for is not self:
+            return None
+        return LazyNorm(stream.xw_buffer, stream.ss_buffer, stream.n_ss, self.eps)
+
     def add_norm(self, h, delta):
         """h: [T, size] float32 residual stream, delta: update of the activation dtype or
         None.  h += delta in place; returns norm(h) in the activation dtype."""
