@@ -65,7 +65,7 @@ struct FusedArgs {
 
 #define SF_UNROLL 4
 
-template <bool NORM, int EPI, typename TY>
+template <bool NORM, int EPI, typename TY, bool GATHER>
 __global__ __launch_bounds__(1024)
 void skinny_fused_kernel(const FusedArgs p) {
     extern __shared__ float red[];                 // [waves][TILES * 4][64 lanes], then [waves][4 lanes] float4 of squares
@@ -102,7 +102,7 @@ void skinny_fused_kernel(const FusedArgs p) {
 
     // Column m of the result depends on row m of x alone, so the lanes of rows past M read
     // row 0 and their results are dropped.
-    const int xr = row < p.M ? (p.x_rows ? p.x_rows[row] : row) : 0;
+    const int xr = row < p.M ? (GATHER ? p.x_rows[row] : row) : 0;
     const bf16_t* xrow = p.x + (size_t)xr * K + kgrp * 8;
 
     // The sums of squares [n_ss_parts, 16 rows] as float4s: thread t takes the float4s t, t + threads, ...,
@@ -118,9 +118,63 @@ void skinny_fused_kernel(const FusedArgs p) {
     for (int t = 0; t < TILES; ++t) acc[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
     const int chunk = SF_UNROLL * 32;
     const int n_chunks = K / chunk;
-    for (int c = wave; c < n_chunks; c += n_waves) {
-        const int k0 = c * chunk;
+    auto multiply_chunk = [&](const bf16x8_t (&a)[TILES][SF_UNROLL], const bf16x8_t (&bx)[SF_UNROLL]) {
+#pragma unroll
+        for (int u = 0; u < SF_UNROLL; ++u)
+#pragma unroll
+            for (int t = 0; t < TILES; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bx[u], acc[t], 0, 0, 0);
+    };
+
+    // The first chunk stands apart: what the back end needs beside the product (the stream's
+    // values and the next norm's weight; or the page, the angles and the bias at the row's
+    // position) is asked for right behind its loads and looked at after the product, so it
+    // arrives meanwhile.  Nothing here is under a condition, so that the waits can be counted:
+    // lanes and blocks that need nothing load from a valid place and drop it.  With K below a
+    // chunk (a wave then has no whole chunk) the first chunk's loads stay inside the row and
+    // meet zeros.
+    const int m = row, nb = 4 * kgrp;
+    const int ml = m < p.M ? m : 0;
+    float4 pre_f0 = make_float4(0.f, 0.f, 0.f, 0.f), pre_f1 = pre_f0;
+    uint2 pre_h0 = make_uint2(0, 0), pre_h1 = pre_h0;
+    int pos = 0, page = -1;
+    if (EPI == EPI_QKV) pos = p.tok_pos[ml];
+    {
         bf16x8_t a[TILES][SF_UNROLL], bx[SF_UNROLL];
+        const bool whole = n_chunks > 0;            // then every wave has a first chunk: waves <= chunks
+#pragma unroll
+        for (int u = 0; u < SF_UNROLL; ++u) {
+            const int k0 = min(wave * chunk + u * 32, K - 32);
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) a[t][u] = load8f(wrow[t] + k0);
+            bx[u] = load8f(xrow + k0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (EPI == EPI_RESIDUAL) {
+            const int n = min(n_lo0 + nb, p.N - 4);
+            pre_f0 = *reinterpret_cast<const float4*>(p.h + (size_t)ml * p.N + n);
+            pre_h0 = *reinterpret_cast<const uint2*>(p.next_norm_w ? p.next_norm_w + n : p.w);
+        }
+        if (EPI == EPI_QKV) {
+            const int half = p.head_dim / 2, i_lo = j16 + nb;
+            page = p.page_table[(size_t)ml * p.table_width + pos / TQK_PAGE];
+            const size_t angle = (size_t)min(pos, p.max_positions - 1) * half + i_lo;
+            pre_f0 = *reinterpret_cast<const float4*>(p.cos_table + angle);
+            pre_f1 = *reinterpret_cast<const float4*>(p.sin_table + angle);
+            pre_h0 = *reinterpret_cast<const uint2*>(p.bias ? p.bias + head * p.head_dim + i_lo : p.w);
+            pre_h1 = *reinterpret_cast<const uint2*>(p.bias ? p.bias + head * p.head_dim + i_lo + half : p.w);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (!whole) {
+            const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int u = 0; u < SF_UNROLL; ++u) bx[u] = zero;
+        }
+        multiply_chunk(a, bx);
+    }
+    for (int c = wave + n_waves; c < n_chunks; c += n_waves) {
+        bf16x8_t a[TILES][SF_UNROLL], bx[SF_UNROLL];
+        const int k0 = c * chunk;
 #pragma unroll
         for (int u = 0; u < SF_UNROLL; ++u) {
 #pragma unroll
@@ -128,11 +182,7 @@ void skinny_fused_kernel(const FusedArgs p) {
             bx[u] = load8f(xrow + k0 + u * 32);
         }
         __builtin_amdgcn_sched_barrier(0);          // every load of the chunk is on its way before the first product waits
-#pragma unroll
-        for (int u = 0; u < SF_UNROLL; ++u)
-#pragma unroll
-            for (int t = 0; t < TILES; ++t)
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bx[u], acc[t], 0, 0, 0);
+        multiply_chunk(a, bx);
     }
     for (int s = n_chunks * SF_UNROLL + wave; s < K / 32; s += n_waves) {
         const int k0 = s * 32;
@@ -181,7 +231,6 @@ void skinny_fused_kernel(const FusedArgs p) {
     }
 
     // the lane holds column m = row of the result, for features n0 + 4*kgrp + r
-    const int m = row;
     float inv_rms = 1.f;
     if (NORM) {
         // the lanes l with l%4 == xr/4 hold row xr's sum of squares in component xr%4
@@ -191,7 +240,6 @@ void skinny_fused_kernel(const FusedArgs p) {
         inv_rms = 1.f / sqrtf(ss / (float)K + p.eps);
     }
     if (m >= p.M && EPI != EPI_RESIDUAL) return;
-    const int nb = 4 * kgrp;
 
     if constexpr (EPI == EPI_STORE) {
         TY* y = (TY*)p.y;
@@ -212,16 +260,19 @@ void skinny_fused_kernel(const FusedArgs p) {
         }
     } else if constexpr (EPI == EPI_RESIDUAL) {
         float sq = 0.f;
+        const float pre_h[4] = {pre_f0.x, pre_f0.y, pre_f0.z, pre_f0.w};
+        const float pre_w[4] = {__uint_as_float(pre_h0.x << 16), __uint_as_float(pre_h0.x & 0xffff0000u),
+                                __uint_as_float(pre_h0.y << 16), __uint_as_float(pre_h0.y & 0xffff0000u)};
         if (m < p.M) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int n = n_lo0 + nb + r;
                 if (n >= p.N) continue;
                 const size_t at = (size_t)m * p.N + n;
-                const float v = p.h[at] + to_float(from_float<bf16_t>(acc[0][r]));
+                const float v = pre_h[r] + to_float(from_float<bf16_t>(acc[0][r]));
                 p.h[at] = v;
                 sq = fmaf(v, v, sq);
-                p.xw_out[at] = from_float<bf16_t>(p.next_norm_w ? v * to_float(p.next_norm_w[n]) : v);
+                p.xw_out[at] = from_float<bf16_t>(p.next_norm_w ? v * pre_w[r] : v);
             }
         }
         if (p.ss_out) {
@@ -234,32 +285,35 @@ void skinny_fused_kernel(const FusedArgs p) {
     } else {    // EPI_QKV
         const int d = p.head_dim, half = d / 2;
         const int kind = head < p.n_heads ? 0 : (head < p.n_heads + p.n_kv_heads ? 1 : 2);
-        const int pos = p.tok_pos[m];
         bf16_t* dst;
         size_t stride = 1;
         if (kind == 0) {
             dst = p.q_out + ((size_t)m * p.n_heads + head) * d;
         } else {
             const int kvh = kind == 1 ? head - p.n_heads : head - p.n_heads - p.n_kv_heads;
-            const int page = p.page_table[(size_t)m * p.table_width + pos / TQK_PAGE];
             if (page < 0) return;                   // the host never lets this happen
             const size_t base = ((size_t)page * p.n_kv_heads + kvh) * TQK_PAGE * d;
             if (kind == 1) dst = p.keys + base + (size_t)(pos % TQK_PAGE) * d;
             else { dst = p.values + base + value_place(pos % TQK_PAGE); stride = TQK_PAGE; }
         }
         const bool rotate = kind != 2 && pos < p.max_positions;
+        const float pre_cos[4] = {pre_f0.x, pre_f0.y, pre_f0.z, pre_f0.w}, pre_sin[4] = {pre_f1.x, pre_f1.y, pre_f1.z, pre_f1.w};
+        const float bias_lo[4] = {__uint_as_float(pre_h0.x << 16), __uint_as_float(pre_h0.x & 0xffff0000u),
+                                  __uint_as_float(pre_h0.y << 16), __uint_as_float(pre_h0.y & 0xffff0000u)};
+        const float bias_hi[4] = {__uint_as_float(pre_h1.x << 16), __uint_as_float(pre_h1.x & 0xffff0000u),
+                                  __uint_as_float(pre_h1.y << 16), __uint_as_float(pre_h1.y & 0xffff0000u)};
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int i_lo = j16 + nb + r, i_hi = i_lo + half;          // elements inside the head
             float lo = to_float(from_float<bf16_t>(acc[0][r] * inv_rms));
             float hi = to_float(from_float<bf16_t>(acc[1][r] * inv_rms));
             if (p.bias) {
-                lo += to_float(p.bias[head * d + i_lo]);
-                hi += to_float(p.bias[head * d + i_hi]);
+                lo += bias_lo[r];
+                hi += bias_hi[r];
             }
             if (rotate) {
-                const float c = p.cos_table[(size_t)pos * half + i_lo], s = p.sin_table[(size_t)pos * half + i_lo];
-                const float r0 = lo * c - hi * s, r1 = lo * s + hi * c;
+                const float c = pre_cos[r], sn = pre_sin[r];
+                const float r0 = lo * c - hi * sn, r1 = lo * sn + hi * c;
                 lo = r0; hi = r1;
             }
             dst[(size_t)i_lo * stride] = from_float<bf16_t>(lo);
@@ -276,12 +330,12 @@ static int pick_waves(int blocks, int K, int tiles) {
     return waves;
 }
 
-template <bool NORM, int EPI, typename TY>
+template <bool NORM, int EPI, typename TY, bool GATHER = false>
 static int launch_fused(const FusedArgs& a, int blocks, hipStream_t s) {
     const int tiles = (EPI == EPI_GATED || EPI == EPI_QKV) ? 2 : 1;
     const int waves = pick_waves(blocks, a.K, tiles);
     const size_t lds = waves > 1 ? (size_t)waves * (tiles * 4) * TQK_WAVE * sizeof(float) + (NORM ? (size_t)waves * 16 * sizeof(float) : 0) : 0;
-    skinny_fused_kernel<NORM, EPI, TY><<<blocks, waves * TQK_WAVE, lds, s>>>(a);
+    skinny_fused_kernel<NORM, EPI, TY, GATHER><<<blocks, waves * TQK_WAVE, lds, s>>>(a);
     return tqk_check_launch("tqk_skinny_fused");
 }
 
@@ -309,6 +363,10 @@ extern "C" int tqk_fused_store(const void* x, const int32_t* x_rows, const float
     if (M == 0) return 0;
     const int blocks = (N + 15) / 16;
     hipStream_t s = (hipStream_t)stream;
+    if (x_rows) {
+        if (ss_parts) return y_dtype == TQK_F32 ? launch_fused<true, EPI_STORE, float, true>(a, blocks, s) : launch_fused<true, EPI_STORE, bf16_t, true>(a, blocks, s);
+        return y_dtype == TQK_F32 ? launch_fused<false, EPI_STORE, float, true>(a, blocks, s) : launch_fused<false, EPI_STORE, bf16_t, true>(a, blocks, s);
+    }
     if (ss_parts) return y_dtype == TQK_F32 ? launch_fused<true, EPI_STORE, float>(a, blocks, s) : launch_fused<true, EPI_STORE, bf16_t>(a, blocks, s);
     return y_dtype == TQK_F32 ? launch_fused<false, EPI_STORE, float>(a, blocks, s) : launch_fused<false, EPI_STORE, bf16_t>(a, blocks, s);
 }
@@ -339,6 +397,8 @@ extern "C" int tqk_fused_residual(const void* x, const void* w, float* h, const 
     a.next_norm_w = (const bf16_t*)next_norm_w; a.xw_out = (bf16_t*)xw_out; a.ss_out = ss_out;
     if (check_common(a, "tqk_fused_residual")) return -1;
     TQK_REQUIRE(h && xw_out, "tqk_fused_residual: null output");
+    TQK_REQUIRE(N % 4 == 0, "tqk_fused_residual: N=%d must be a multiple of 4", N);
+    TQK_REQUIRE(((((uintptr_t)h) | ((uintptr_t)next_norm_w)) & 15) == 0, "tqk_fused_residual: h and the norm's weight must be 16-byte aligned");
     if (M == 0) return 0;
     return launch_fused<false, EPI_RESIDUAL, bf16_t>(a, (N + 15) / 16, (hipStream_t)stream);
 }
@@ -364,6 +424,8 @@ extern "C" int tqk_fused_qkv(const void* x, const float* ss_parts, int n_ss_part
     TQK_REQUIRE(cos_table && sin_table && max_positions > 0 && tok_pos && page_table && keys && values && q_out,
                 "tqk_fused_qkv: null pointer");
     TQK_REQUIRE(table_width > 0 && n_pages > 0, "tqk_fused_qkv: empty page table");
+    TQK_REQUIRE(((((uintptr_t)cos_table) | ((uintptr_t)sin_table) | ((uintptr_t)bias)) & 15) == 0,
+                "tqk_fused_qkv: the angle tables and the bias must be 16-byte aligned");
     if (M == 0) return 0;
     const int blocks = (n_heads + 2 * n_kv_heads) * (head_dim / 32);
     hipStream_t s = (hipStream_t)stream;

@@ -90,7 +90,7 @@ class Attention(Part):
         return self._fused_qkv_ok(ctx) and not self.reads_other_cache
 
     def adds_to_stream(self, ctx):
-        return fusable(ctx.n_tokens, self.w_o) and self.b_o is None
+        return fusable(ctx.n_tokens, self.w_o, adds=True) and self.b_o is None
 
     def forward(self, x, ctx, entry, stream=None):
         lazy = isinstance(x, LazyNorm)

@@ -37,7 +37,7 @@ class GatedSiLU(Part):
         return fusable(ctx.n_tokens, self.w_gate_up)
 
     def adds_to_stream(self, ctx):
-        return fusable(ctx.n_tokens, self.w_down) and fusable(ctx.n_tokens, self.w_gate_up)
+        return fusable(ctx.n_tokens, self.w_down, adds=True) and fusable(ctx.n_tokens, self.w_gate_up)
 
     def forward(self, x, ctx, stream=None):
         lazy = isinstance(x, LazyNorm)

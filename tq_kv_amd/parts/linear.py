@@ -58,10 +58,11 @@ class LazyNorm:
         self.xw, self.norm = xw, (ss, n_ss, eps)
 
 
-def fusable(x_rows, weight):
-    """Whether the folded skinny kernels take a product of x_rows rows with this weight."""
+def fusable(x_rows, weight, adds=False):
+    """Whether the folded skinny kernels take a product of x_rows rows with this weight
+    (adds: with the result added to the stream)."""
     return (POLICY["fused"] and POLICY["skinny"] and x_rows <= 16 and weight.dtype == torch.bfloat16
-            and weight.shape[1] % 32 == 0)
+            and weight.shape[1] % 32 == 0 and (not adds or weight.shape[0] % 4 == 0))
 
 
 def tune_library(on=True, seconds=30):

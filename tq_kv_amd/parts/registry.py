@@ -14,8 +14,16 @@ Categories and what each must offer beyond `tensors()` and `load()`:
   mixer         cache_need() -> KVNeed | StateNeed | None;
                 forward(x, ctx, cache_entry) -> y, x and y [tokens, hidden]
   feed_forward  forward(x, ctx) -> y
-  block         the arrangement: forward(h, delta, ctx, cache_entry) -> delta, where h
-                is the float32 residual stream and delta the update not yet added
+  block         the arrangement: forward(stream, ctx, cache_entry, next_norm), where stream
+                (parts.linear.Stream) holds the float32 residual stream h and the update
+                not yet added to it, and next_norm is the norm that reads the stream after
+                this block; first_norm() -> the norm this block reads the stream with
+
+Optional, for small decoding steps (ctx.fuse_small), and never needed for a part to work:
+a norm with `foldable` and `lazy(stream)` lets the product after it do the division; a
+mixer or feed-forward with `folds_norm(ctx)` accepts a parts.linear.LazyNorm as x, and
+with `adds_to_stream(ctx)` accepts `stream=` and adds its output to the stream itself
+(Stream.add_product), returning None.
 """
 from typing import Callable, Dict
 
