@@ -89,15 +89,19 @@ def main():
     # -- decoding ---------------------------------------------------------------------------
     def decode(batch, steps, warmup):
         """Tokens per second over `steps` decode steps of `batch` sequences after their prompts."""
-        marks = []
+        marks, calls = {}, [0]
 
         def on_tokens(pairs):
-            torch.cuda.synchronize()
-            marks.append(time.perf_counter())
-        params = GenerationParams(max_tokens=warmup + steps + 1, temperature=0.0, repeat_penalty=1.0)
+            # call i comes when the tokens of draw i are known; draw i+1 needs decode step i+1.
+            # The loop keeps one step under way while it reads a draw, so the device is waited
+            # for at the two ends of the timed steps only, and each wait ends just after a step.
+            if calls[0] in (warmup, warmup + steps):
+                torch.cuda.synchronize()
+                marks[calls[0]] = time.perf_counter()
+            calls[0] += 1
+        params = GenerationParams(max_tokens=warmup + steps + 2, temperature=0.0, repeat_penalty=1.0)
         out = generate(engine, prompts(batch), params, on_tokens=on_tokens, max_batch=batch)
-        assert all(len(o) == warmup + steps + 1 for o in out)
-        # marks[i] is taken after the tokens of draw i are known; draw i+1 needs decode step i+1
+        assert all(len(o) == warmup + steps + 2 for o in out)
         seconds = marks[warmup + steps] - marks[warmup]
         return batch * steps / seconds, seconds / steps
 
@@ -122,7 +126,7 @@ def main():
         "config": {"model": args.shape, "global_batch": args.batch, "seq_len": ctx_len, "parallelism": "single-gpu",
                    "layers": layers, "layers_of_shape": full_layers, "hidden": H, "heads": nh, "kv_heads": nkv,
                    "head_dim": d, "intermediate": I, "vocab": V, "prompt_len": args.prompt_len,
-                   "new_tokens": args.warmup + args.steps + 1, "weights": "random N(0,0.02)", "sampling": "greedy",
+                   "new_tokens": args.warmup + args.steps + 2, "weights": "random N(0,0.02)", "sampling": "greedy",
                    "library_tuning": not args.no_tune},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK["hbm_gbs"], "unit": "GB/s",

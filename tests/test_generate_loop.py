@@ -153,3 +153,85 @@ def test_params_have_the_reference_defaults():
     with pytest.raises(ValueError):
         GenerationParams(top_p=0.0)
     assert "temperature=0.7" in repr(p)
+
+
+# ---- running ahead: the next step is started before the draw has been read ---------------------
+class AheadEngine(FakeEngine):
+    """Takes a step's tokens "from the device": here a list that is only looked at when the
+    step is recorded, as a device would."""
+    takes_device_tokens = True
+
+    def step(self, items, device_tokens=None, borrow=False):
+        if device_tokens is not None:
+            assert all(t == [0] for _, t, _ in items) and len(device_tokens) == len(items)
+            items = [(s, [tok], w) for (s, _, w), tok in zip(items, device_tokens)]
+        return FakeEngine.step(self, items)
+
+
+class AheadSampler(ScriptSampler):
+    class Draw:
+        def __init__(self, tokens, log):
+            self.tokens, self.log = tokens, log
+
+        def read(self):
+            self.log.append("read")
+            return self.tokens
+
+    def __init__(self, scripts, request_ids, log):
+        ScriptSampler.__init__(self, scripts, request_ids)
+        self.log = log
+
+    def draw(self, logits, rows):
+        self.log.append("draw")
+        return self.Draw(ScriptSampler.sample(self, logits, rows), self.log)
+
+    def pick(self, drawn, places):
+        return [drawn.tokens[i] for i in places]
+
+
+def run_ahead(prompts, scripts, max_tokens, eos=(), **kw):
+    eng, log, events = AheadEngine(), [], []
+    out = generate(eng, prompts, GenerationParams(max_tokens=max_tokens, temperature=0.0), eos_ids=eos,
+                   on_tokens=events.append, make_sampler=lambda p, ids: AheadSampler(scripts, ids, log), **kw)
+    return out, eng, events, log
+
+
+CASES = [
+    ([[5, 6, 7]], [[10, 11, 12, 13, 14, 15]], 3, ()),
+    ([[5, 6, 7]], [[10, 11, 12, 13, 14, 15]], 1, ()),
+    ([[5, 6, 7]], [[10, 11, 12, 13, 14, 15]], 0, ()),
+    ([[1, 2]], [[10, 11, 99, 12, 13, 14]], 8, (99,)),
+    ([[1, 2]], [[99, 1, 2, 3]], 8, (99,)),
+    ([[1], [2, 2], [3, 3, 3]], [[10, 99, 7, 7], [20, 21, 22, 23, 24, 25], [30, 31, 99, 7, 7]], 4, (99,)),
+    ([[1], [2, 2], [3, 3, 3]], [[10, 11, 12, 13, 99, 5, 5], [20, 99, 5, 5], [99, 5, 5]], 6, (99,)),
+    ([[1] * 10, [2] * 10, [3] * 10, [4] * 10, [5] * 10], [[10 + i] * 9 for i in range(5)], 5, ()),
+]
+
+
+@pytest.mark.parametrize("prompts,scripts,max_tokens,eos", CASES)
+def test_running_ahead_emits_the_same(prompts, scripts, max_tokens, eos):
+    kw = {"max_batch": 2} if len(prompts) == 5 else {}
+    want, plain_eng, want_events = run(prompts, scripts, max_tokens, eos, **kw)
+    out, eng, events, _ = run_ahead(prompts, scripts, max_tokens, eos, **kw)
+    assert out == want and events == want_events
+    assert eng.seen == {} and sorted(eng.closed) == sorted(plain_eng.closed)        # every slot back, once
+    # every step of the plain run is there, for the same slots and tokens; beyond them only rows of
+    # requests whose stop token had not been read yet
+    for plain_step, step in zip(plain_eng.steps, eng.steps):
+        assert [x for x in step if x in plain_step] == plain_step
+
+
+def test_running_ahead_starts_the_next_step_before_reading_the_draw():
+    out, eng, _, log = run_ahead([[1, 2]], [[10, 11, 12, 13, 14]], 4)
+    assert out == [[10, 11, 12, 13]]
+    assert eng.steps == [[(0, [1, 2])], [(0, [10])], [(0, [11])], [(0, [12])]]
+    # after the first decoding step there are always two draws under way when one is read
+    assert log == ["draw", "draw", "read", "draw", "read", "read"]
+
+
+def test_running_ahead_wastes_one_row_on_a_stop_token():
+    out, eng, _, _ = run_ahead([[1], [2]], [[10, 11, 99, 5, 5], [20, 21, 22, 23, 24]], 5, eos=(99,))
+    assert out == [[10, 11], [20, 21, 22, 23, 24]]
+    # request 0's stop token 99 was fed once, because the step was started before it was read
+    assert eng.steps[3] == [(0, [99]), (1, [22])] and eng.steps[4] == [(1, [23])]
+    assert eng.seen == {}

@@ -182,6 +182,40 @@ def test_step_refuses_what_it_cannot_run():
     small.cache.check()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_tokens_given_on_the_device_equal_tokens_given_by_the_host(dtype):
+    from tq_kv_amd import StepError
+    # one-token steps whose tokens the host does not know (chosen by a kernel just before)
+    eng = G.engine("A", dtype, True)
+    reqs = G.prompts("A", [9, 4, 13], seed=1100)
+    for device_side in (False, True, True):           # the second device-side round replays the graph
+        slots = [eng.open() for _ in reqs]
+        eng.step([(s, r[:-3], []) for s, r in zip(slots, reqs)])
+        outs = []
+        for k in range(3, 0, -1):
+            toks = [r[-k] for r in reqs]
+            if device_side:
+                dev = torch.tensor(toks, dtype=torch.int32, device=eng.model.device)
+                outs.append(eng.step([(s, [0], [0]) for s in slots], device_tokens=dev))
+            else:
+                outs.append(eng.step([(s, [t], [0]) for s, t in zip(slots, toks)]))
+        if device_side:
+            for a, b in zip(outs, want):
+                assert torch.equal(a, b)
+        else:
+            want = outs
+        for s in slots:
+            eng.close(s)
+    with pytest.raises(StepError, match="one token per sequence"):
+        s = eng.open()
+        eng.step([(s, [1, 2], [1])], device_tokens=torch.zeros(1, dtype=torch.int32, device=eng.model.device))
+    eng.close(s)
+    with pytest.raises(StepError, match="int32"):
+        s = eng.open()
+        eng.step([(s, [1], [0])], device_tokens=torch.zeros(2, dtype=torch.int32, device=eng.model.device))
+    eng.close(s)
+
+
 # ---- generation through the entry point -------------------------------------------------------
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_greedy_generation_float32_equals_plain(name):

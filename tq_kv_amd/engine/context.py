@@ -19,29 +19,37 @@ class _Arrays:
 
 
 class HostStaging:
-    """A pinned host buffer that is reused from step to step; the copy of the step
-    before must have finished before it is written again."""
+    """Pinned host buffers for small uploads, used in turn; a buffer is written again only
+    after the copy that last read it has finished."""
 
-    def __init__(self, device):
+    def __init__(self, device, depth=2):
         self.device = device
-        self.buf = None
-        self.event = None
+        self.bufs = [None] * depth
+        self.events = [None] * depth
+        self.turn = 0
 
     def upload(self, packed, into=None):
-        """Copy the packed array to the device: into `into` (a device buffer of the same
-        size that a captured graph reads) or into a new tensor."""
+        """Copy a one-dimensional int32 or float32 array to the device without waiting for
+        the device: into `into` (a device buffer of the same size and kind, for instance one
+        that a captured graph reads) or into a new tensor."""
         n = packed.shape[0]
-        if self.event is not None:
-            self.event.synchronize()
-        if self.buf is None or self.buf.shape[0] < n:
-            self.buf = torch.empty(max(4096, 2 * n), dtype=torch.int32, pin_memory=True)
-        self.buf[:n].numpy()[:] = packed
-        dev = into if into is not None else torch.empty(n, dtype=torch.int32, device=self.device)
-        if dev.shape[0] != n:
-            raise ValueError("the step's arrays take %d values, the buffer holds %d" % (n, dev.shape[0]))
-        dev.copy_(self.buf[:n], non_blocking=True)
-        self.event = torch.cuda.Event()
-        self.event.record()
+        kind = torch.float32 if packed.dtype == np.float32 else torch.int32
+        if kind == torch.int32 and packed.dtype != np.int32:
+            raise TypeError("uploads are int32 or float32, got %s" % packed.dtype)
+        i = self.turn
+        self.turn = (i + 1) % len(self.bufs)
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        if self.bufs[i] is None or self.bufs[i].shape[0] < n:
+            self.bufs[i] = torch.empty(max(4096, 2 * n), dtype=torch.int32, pin_memory=True)
+        host = self.bufs[i][:n].view(kind)
+        host.numpy()[:] = packed
+        dev = into if into is not None else torch.empty(n, dtype=kind, device=self.device)
+        if dev.shape[0] != n or dev.dtype != kind:
+            raise ValueError("the upload is %d values of %s, the buffer holds %d of %s" % (n, kind, dev.shape[0], dev.dtype))
+        dev.copy_(host, non_blocking=True)
+        self.events[i] = torch.cuda.Event()
+        self.events[i].record()
         return dev
 
 

@@ -26,6 +26,7 @@ class Engine:
 
     GRAPH_WIDTH_STEP = 8       # page-table widths of graphed steps grow in steps of 8 pages
     MAX_GRAPHS = 32
+    takes_device_tokens = True
 
     def __init__(self, model, max_tokens, max_slots=256, use_graphs=True):
         self.model = model
@@ -53,14 +54,23 @@ class Engine:
         return self.cache.length(slot)
 
     # -- the step ---------------------------------------------------------
-    def step(self, items, borrow=False):
+    def step(self, items, borrow=False, device_tokens=None):
         """items: [(slot, tokens, want)].  tokens: the sequence's next tokens (at least one);
         want: indices among them whose logits are wanted (may be empty).  Returns float32
         logits [sum of len(want), vocab] in the order of items and of want.  borrow: the
         caller is done with the logits before the next step (they may live in a buffer that
-        the next step writes again)."""
+        the next step writes again).  device_tokens: int32 [len(items)] on the device, for a
+        step of one token per sequence whose tokens the host does not know yet (they were
+        chosen on the device and must lie inside the vocabulary); the items' tokens are then
+        placeholders."""
         if not items:
             raise StepError("a step needs at least one sequence")
+        if device_tokens is not None:
+            if any(len(tokens) != 1 for _, tokens, _ in items):
+                raise StepError("tokens on the device stand for one token per sequence")
+            if device_tokens.dtype != torch.int32 or tuple(device_tokens.shape) != (len(items),) \
+                    or device_tokens.device.type != self.model.device.type:
+                raise StepError("device_tokens must be int32 [%d] on %s" % (len(items), self.model.device))
         seen = set()
         for slot, tokens, _ in items:
             if slot in seen:
@@ -79,16 +89,18 @@ class Engine:
         ctx_items = [(slot, self.cache.length(slot), tokens) for slot, tokens, _ in items]
         wants = [want for _, _, want in items]
         if self.use_graphs and all(n == 1 for _, n in sizes) and len(items) <= self.model.graph_max_rows:
-            logits = self._graphed_step(ctx_items, wants)
+            logits = self._graphed_step(ctx_items, wants, device_tokens)
             if not borrow:
                 logits = logits.clone()
         else:
             ctx = StepContext(ctx_items, wants, self.cache, self.model.device, self.staging)
+            if device_tokens is not None:
+                ctx.dev.tokens.copy_(device_tokens)
             logits = self.model.forward(ctx, self.cache)
         self.cache.commit(sizes)
         return logits
 
-    def _graphed_step(self, ctx_items, wants):
+    def _graphed_step(self, ctx_items, wants, device_tokens=None):
         """A step of one token per sequence through a captured graph.  The graph reads the
         step's arrays (tokens, positions, page tables) from one device buffer that is
         overwritten before every replay; its kernels take every size from those arrays or
@@ -98,6 +110,8 @@ class Engine:
         entry = self.graphs.get(key)
         if entry is None:
             ctx = StepContext(ctx_items, wants, self.cache, self.model.device, self.staging, self.GRAPH_WIDTH_STEP)
+            if device_tokens is not None:
+                ctx.dev.tokens.copy_(device_tokens)
             logits = self.model.forward(ctx, self.cache)          # this step's work, and the warm-up
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
@@ -110,5 +124,7 @@ class Engine:
         graph, ctx, static_logits = entry
         self.graphs[key] = self.graphs.pop(key)                     # most recently used last
         self.staging.upload(probe.packed, into=ctx.flat)
+        if device_tokens is not None:
+            ctx.dev.tokens.copy_(device_tokens)
         graph.replay()
         return static_logits

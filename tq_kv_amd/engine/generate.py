@@ -95,13 +95,31 @@ def _prompt_steps(lens, max_step_tokens):
     return steps
 
 
+class _Known:
+    """A draw whose tokens the host already has."""
+
+    def __init__(self, tokens):
+        self.tokens = list(tokens)
+
+    def read(self):
+        return self.tokens
+
+
 def _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, sampler, max_step_tokens):
+    """One batch from its prompts to its last token.
+
+    Running ahead: if the engine takes a step's tokens from the device and the sampler can
+    start a draw without waiting for it (`draw`, `pick`), the step after a draw is started
+    before the draw has been read, for every request that goes on unless its unread token
+    is a stop token; the host then reads the draw while the device works.  A request that
+    did stop has run one step for nothing: its row of the next draw is dropped, and its
+    slot goes back as it would have.  What is emitted is the same either way."""
     slots = {}
     borrow = {"borrow": True} if getattr(engine, "use_graphs", False) else {}
+    ahead = bool(getattr(engine, "takes_device_tokens", False)) and hasattr(sampler, "draw") and hasattr(sampler, "pick")
     try:
         for r in batch:
             slots[r] = engine.open()
-        live = list(range(len(batch)))                 # indices into `batch`
         drawn = {}
         for step in _prompt_steps([len(prompts[r]) for r in batch], max_step_tokens):
             items, ends = [], []
@@ -114,27 +132,44 @@ def _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, sampler,
             logits = engine.step(items)
             if ends:
                 drawn.update(zip(ends, sampler.sample(logits, ends)))
-        while live:
+        rows = list(range(len(batch)))                 # indices into `batch` whose token is in `draw`
+        draw = _Known([drawn[b] for b in rows])
+        stopped = set()                                # requests that ended while a step with them was under way
+        while rows:
+            # the step after this draw, for those that go on if their unread token is no stop token
+            next_rows, next_draw = [], None
+            if ahead and not isinstance(draw, _Known):
+                next_rows = [b for b in rows if b not in stopped and len(emitted[batch[b]]) + 1 < params.max_tokens]
+                if next_rows:
+                    tokens = sampler.pick(draw, [rows.index(b) for b in next_rows])
+                    logits = engine.step([(slots[batch[b]], [0], [0]) for b in next_rows], device_tokens=tokens, **borrow)
+                    next_draw = sampler.draw(logits, next_rows)
             feed, pairs = [], []
-            for b in live:
+            for b, tok in zip(rows, draw.read()):
+                if b in stopped:
+                    continue
                 r = batch[b]
-                tok = drawn[b]
                 if len(emitted[r]) >= params.max_tokens or tok in eos:
                     engine.close(slots.pop(r))          # stop tokens are not emitted (src/engine.rs:381)
+                    stopped.add(b)
                     continue
                 emitted[r].append(tok)
                 pairs.append((r, tok))
                 if len(emitted[r]) >= params.max_tokens:
                     engine.close(slots.pop(r))          # nothing more to draw for it
+                    stopped.add(b)
                     continue
-                feed.append(b)
+                feed.append((b, tok))
             if on_tokens is not None and pairs:
                 on_tokens(pairs)
-            live = feed
-            if not live:
+            if next_draw is not None:
+                rows, draw = next_rows, next_draw
+                continue
+            rows = [b for b, _ in feed]
+            if not rows:
                 break
-            logits = engine.step([(slots[batch[b]], [drawn[b]], [0]) for b in live], **borrow)
-            drawn = dict(zip(live, sampler.sample(logits, live)))
+            logits = engine.step([(slots[batch[b]], [tok], [0]) for b, tok in feed], **borrow)
+            draw = sampler.draw(logits, rows) if ahead else _Known(sampler.sample(logits, rows))
     finally:
         for slot in slots.values():
             engine.close(slot)
