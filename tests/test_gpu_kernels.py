@@ -495,7 +495,7 @@ def prepared(h, nw):
 
 
 @pytest.mark.parametrize("m", [1, 5, 16])
-@pytest.mark.parametrize("n,k", [(100, 96), (3584, 3584), (1000, 1536)])
+@pytest.mark.parametrize("n,k", [(100, 96), (3584, 3584), (1000, 1536), (65610, 64)])       # the last: blocks of two tiles
 def test_fused_store_with_and_without_norm(m, n, k):
     h = rand(16, k, seed=100, scale=2.0)
     w = rand(n, k, seed=101, scale=1.0 / math.sqrt(k), dtype=torch.bfloat16)
@@ -538,11 +538,11 @@ def test_fused_residual_prepares_the_next_norm(m, n, k):
     h = rand(m, n, seed=108, scale=3.0)
     want = h + bf((x.double() @ w.double().t()).float())
     xw = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
-    ss = torch.full((K.fused_residual_parts(n), 16), float("nan"), device=DEV)
+    ss = torch.full((K.fused_residual_parts(n, k), 16), float("nan"), device=DEV)
     parts = K.fused_residual(x, w, h, xw, nw, ss)
     torch.testing.assert_close(h, want, atol=4e-2, rtol=0)          # one bfloat16 step of the product at most
     assert torch.equal(xw, (h * nw.float()).to(torch.bfloat16))
-    assert parts == (n + 15) // 16
+    assert parts == K.fused_residual_parts(n, k) <= (n + 15) // 16
     torch.testing.assert_close(ss[:, :m].sum(0), (h * h).sum(-1), rtol=1e-5, atol=1e-5)
     # and what the next product makes of it is the norm of the new stream
     w2 = rand(48, n, seed=114, scale=1.0 / math.sqrt(n), dtype=torch.bfloat16)

@@ -213,20 +213,26 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 }
 
 // out[seq, head, :] = sum_p exp(m_p - M) o_p / sum_p exp(m_p - M) l_p, partitions in order.
+// No branch in the loops, so that the loads of several partitions are under way together; a
+// partition without keys (m = -inf) has weight 0 and its (unwritten) output is not looked at.
 __global__ void attention_merge_kernel(const float* __restrict__ part_out, const float* __restrict__ part_ml,
                                        int n_parts, int head_dim, bf16_t* __restrict__ out) {
     const size_t row = blockIdx.x;                     // seq * n_heads + head
-    const float* ml = part_ml + row * n_parts * 2;
+    const float2* ml = reinterpret_cast<const float2*>(part_ml) + row * n_parts;
     float M = -INFINITY;
-    for (int p = 0; p < n_parts; ++p) M = fmaxf(M, ml[p * 2]);
+#pragma unroll 8
+    for (int p = 0; p < n_parts; ++p) M = fmaxf(M, ml[p].x);
     for (int c = threadIdx.x; c < head_dim; c += blockDim.x) {
         float acc = 0.f, denom = 0.f;
+        const float* po = part_out + row * n_parts * head_dim + c;
+#pragma unroll 8
         for (int p = 0; p < n_parts; ++p) {
-            const float mp = ml[p * 2];
-            if (mp == -INFINITY) continue;
-            const float wgt = expf(mp - M);
-            denom += wgt * ml[p * 2 + 1];
-            acc += wgt * part_out[(row * n_parts + p) * head_dim + c];
+            const float2 s = ml[p];
+            const float v = po[(size_t)p * head_dim];
+            const bool live = s.x != -INFINITY;
+            const float wgt = live ? expf(s.x - M) : 0.f;
+            denom += wgt * s.y;
+            acc += live ? wgt * v : 0.f;
         }
         out[row * head_dim + c] = from_float<bf16_t>(acc / denom);
     }

@@ -63,14 +63,19 @@ struct FusedArgs {
     bf16_t* values;             // [pages, kv heads, head_dim, 64 places]
 };
 
-#define SF_UNROLL 4
 
-template <bool NORM, int EPI, typename TY, bool GATHER>
+// RT: tiles of 16 output features next to each other per block, for the back ends "store" and
+// "residual" (gated and qkv blocks always hold a pair of tiles).  All tiles of a block meet
+// the same values of x, so x is read RT times less often.
+template <bool NORM, int EPI, typename TY, bool GATHER, int RT>
 __global__ __launch_bounds__(1024)
 void skinny_fused_kernel(const FusedArgs p) {
     extern __shared__ float red[];                 // [waves][TILES * 4][64 lanes], then [waves][4 lanes] float4 of squares
-    constexpr int TILES = (EPI == EPI_GATED || EPI == EPI_QKV) ? 2 : 1;
+    constexpr bool PAIR = EPI == EPI_GATED || EPI == EPI_QKV;
+    static_assert(!PAIR || RT == 1, "gated and qkv blocks hold one pair of tiles");
+    constexpr int TILES = PAIR ? 2 : RT;
     constexpr int SLOTS = TILES * 4;
+    constexpr int SF_UNROLL = 4;                   // k steps of 32 whose loads are under way together
     const int lane = threadIdx.x % TQK_WAVE, wave = threadIdx.x / TQK_WAVE;
     const int n_waves = blockDim.x / TQK_WAVE;
     const int row = lane % 16, kgrp = lane / 16;
@@ -92,13 +97,18 @@ void skinny_fused_kernel(const FusedArgs p) {
         n_hi0 = n_out + n_lo0;
     } else {
         n_out = p.N;
-        n_lo0 = blockIdx.x * 16;
+        n_lo0 = blockIdx.x * 16 * RT;
         n_hi0 = 0;
     }
     const int n_clamp = (EPI == EPI_GATED) ? n_out - 1 : p.N - 1;
     const bf16_t* wrow[TILES];
-    wrow[0] = p.w + (size_t)min(n_lo0 + row, n_clamp) * K + kgrp * 8;
-    if (TILES == 2) wrow[1] = p.w + (size_t)(EPI == EPI_GATED ? n_out + min(n_lo0 + row, n_clamp) : n_hi0 + row) * K + kgrp * 8;
+    if (PAIR) {
+        wrow[0] = p.w + (size_t)min(n_lo0 + row, n_clamp) * K + kgrp * 8;
+        wrow[TILES - 1] = p.w + (size_t)(EPI == EPI_GATED ? n_out + min(n_lo0 + row, n_clamp) : n_hi0 + row) * K + kgrp * 8;
+    } else {
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) wrow[t] = p.w + (size_t)min(n_lo0 + 16 * t + row, n_clamp) * K + kgrp * 8;
+    }
 
     // Column m of the result depends on row m of x alone, so the lanes of rows past M read
     // row 0 and their results are dropped.
@@ -135,8 +145,10 @@ void skinny_fused_kernel(const FusedArgs p) {
     // meet zeros.
     const int m = row, nb = 4 * kgrp;
     const int ml = m < p.M ? m : 0;
-    float4 pre_f0 = make_float4(0.f, 0.f, 0.f, 0.f), pre_f1 = pre_f0;
-    uint2 pre_h0 = make_uint2(0, 0), pre_h1 = pre_h0;
+    float4 pre_f0[TILES], pre_f1 = make_float4(0.f, 0.f, 0.f, 0.f);
+    uint2 pre_h0[TILES], pre_h1 = make_uint2(0, 0);
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) { pre_f0[t] = pre_f1; pre_h0[t] = pre_h1; }
     int pos = 0, page = -1;
     if (EPI == EPI_QKV) pos = p.tok_pos[ml];
     {
@@ -151,17 +163,20 @@ void skinny_fused_kernel(const FusedArgs p) {
         }
         __builtin_amdgcn_sched_barrier(0);
         if (EPI == EPI_RESIDUAL) {
-            const int n = min(n_lo0 + nb, p.N - 4);
-            pre_f0 = *reinterpret_cast<const float4*>(p.h + (size_t)ml * p.N + n);
-            pre_h0 = *reinterpret_cast<const uint2*>(p.next_norm_w ? p.next_norm_w + n : p.w);
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) {
+                const int n = min(n_lo0 + 16 * t + nb, p.N - 4);
+                pre_f0[t] = *reinterpret_cast<const float4*>(p.h + (size_t)ml * p.N + n);
+                pre_h0[t] = *reinterpret_cast<const uint2*>(p.next_norm_w ? p.next_norm_w + n : p.w);
+            }
         }
         if (EPI == EPI_QKV) {
             const int half = p.head_dim / 2, i_lo = j16 + nb;
             page = p.page_table[(size_t)ml * p.table_width + pos / TQK_PAGE];
             const size_t angle = (size_t)min(pos, p.max_positions - 1) * half + i_lo;
-            pre_f0 = *reinterpret_cast<const float4*>(p.cos_table + angle);
+            pre_f0[0] = *reinterpret_cast<const float4*>(p.cos_table + angle);
             pre_f1 = *reinterpret_cast<const float4*>(p.sin_table + angle);
-            pre_h0 = *reinterpret_cast<const uint2*>(p.bias ? p.bias + head * p.head_dim + i_lo : p.w);
+            pre_h0[0] = *reinterpret_cast<const uint2*>(p.bias ? p.bias + head * p.head_dim + i_lo : p.w);
             pre_h1 = *reinterpret_cast<const uint2*>(p.bias ? p.bias + head * p.head_dim + i_lo + half : p.w);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -244,10 +259,12 @@ void skinny_fused_kernel(const FusedArgs p) {
     if constexpr (EPI == EPI_STORE) {
         TY* y = (TY*)p.y;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int n = n_lo0 + nb + r;
-            if (n < p.N) y[(size_t)m * p.N + n] = from_float<TY>(acc[0][r] * inv_rms);
-        }
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int n = n_lo0 + 16 * t + nb + r;
+                if (n < p.N) y[(size_t)m * p.N + n] = from_float<TY>(acc[t][r] * inv_rms);
+            }
     } else if constexpr (EPI == EPI_GATED) {
         bf16_t* y = (bf16_t*)p.y;
 #pragma unroll
@@ -260,23 +277,26 @@ void skinny_fused_kernel(const FusedArgs p) {
         }
     } else if constexpr (EPI == EPI_RESIDUAL) {
         float sq = 0.f;
-        const float pre_h[4] = {pre_f0.x, pre_f0.y, pre_f0.z, pre_f0.w};
-        const float pre_w[4] = {__uint_as_float(pre_h0.x << 16), __uint_as_float(pre_h0.x & 0xffff0000u),
-                                __uint_as_float(pre_h0.y << 16), __uint_as_float(pre_h0.y & 0xffff0000u)};
         if (m < p.M) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int n = n_lo0 + nb + r;
-                if (n >= p.N) continue;
-                const size_t at = (size_t)m * p.N + n;
-                const float v = pre_h[r] + to_float(from_float<bf16_t>(acc[0][r]));
-                p.h[at] = v;
-                sq = fmaf(v, v, sq);
-                p.xw_out[at] = from_float<bf16_t>(p.next_norm_w ? v * pre_w[r] : v);
+            for (int t = 0; t < TILES; ++t) {
+                const float pre_h[4] = {pre_f0[t].x, pre_f0[t].y, pre_f0[t].z, pre_f0[t].w};
+                const float pre_w[4] = {__uint_as_float(pre_h0[t].x << 16), __uint_as_float(pre_h0[t].x & 0xffff0000u),
+                                        __uint_as_float(pre_h0[t].y << 16), __uint_as_float(pre_h0[t].y & 0xffff0000u)};
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int n = n_lo0 + 16 * t + nb + r;
+                    if (n >= p.N) continue;
+                    const size_t at = (size_t)m * p.N + n;
+                    const float v = pre_h[r] + to_float(from_float<bf16_t>(acc[t][r]));
+                    p.h[at] = v;
+                    sq = fmaf(v, v, sq);
+                    p.xw_out[at] = from_float<bf16_t>(p.next_norm_w ? v * pre_w[r] : v);
+                }
             }
         }
         if (p.ss_out) {
-            // this block's 16 columns of row m: the four lanes of the row, in lane order
+            // this block's columns of row m: the four lanes of the row, in lane order
             const float s1 = __shfl_xor(sq, 16, TQK_WAVE);
             const float s2 = __shfl_xor(sq, 32, TQK_WAVE);
             const float s3 = __shfl_xor(s1, 32, TQK_WAVE);
@@ -297,9 +317,9 @@ void skinny_fused_kernel(const FusedArgs p) {
             else { dst = p.values + base + value_place(pos % TQK_PAGE); stride = TQK_PAGE; }
         }
         const bool rotate = kind != 2 && pos < p.max_positions;
-        const float pre_cos[4] = {pre_f0.x, pre_f0.y, pre_f0.z, pre_f0.w}, pre_sin[4] = {pre_f1.x, pre_f1.y, pre_f1.z, pre_f1.w};
-        const float bias_lo[4] = {__uint_as_float(pre_h0.x << 16), __uint_as_float(pre_h0.x & 0xffff0000u),
-                                  __uint_as_float(pre_h0.y << 16), __uint_as_float(pre_h0.y & 0xffff0000u)};
+        const float pre_cos[4] = {pre_f0[0].x, pre_f0[0].y, pre_f0[0].z, pre_f0[0].w}, pre_sin[4] = {pre_f1.x, pre_f1.y, pre_f1.z, pre_f1.w};
+        const float bias_lo[4] = {__uint_as_float(pre_h0[0].x << 16), __uint_as_float(pre_h0[0].x & 0xffff0000u),
+                                  __uint_as_float(pre_h0[0].y << 16), __uint_as_float(pre_h0[0].y & 0xffff0000u)};
         const float bias_hi[4] = {__uint_as_float(pre_h1.x << 16), __uint_as_float(pre_h1.x & 0xffff0000u),
                                   __uint_as_float(pre_h1.y << 16), __uint_as_float(pre_h1.y & 0xffff0000u)};
 #pragma unroll
@@ -322,21 +342,41 @@ void skinny_fused_kernel(const FusedArgs p) {
     }
 }
 
+// Tiles per block for the back ends "store" and "residual", from the product's shape alone
+// (never from M: a row's sums then have one order in every batch).  Two tiles halve the
+// reads of x, but also the number of blocks, and a block keeps one compute unit busy:
+// measured, a pair pays only where there are thousands of blocks left (the vocabulary's product).
+static int pick_tiles(int N, int K) {
+    (void)K;
+    return N / 32 >= 2048 ? 2 : 1;
+}
+
+// Waves per block, which split K between them: about a thousand waves on the chip keep HBM
+// busy; no more than there are chunks of K to share out; a power of two.
 static int pick_waves(int blocks, int K, int tiles) {
-    const int chunks = K / (SF_UNROLL * 32) > 0 ? K / (SF_UNROLL * 32) : 1;
-    const int max_waves = tiles == 2 ? 8 : 16;
+    const int chunks = K / (4 * 32) > 0 ? K / (4 * 32) : 1;
+    const int max_waves = tiles >= 2 ? 8 : 16;
     int waves = 1;
     while (waves < max_waves && blocks * waves < 1024 && waves * 2 <= chunks) waves *= 2;
     return waves;
 }
 
-template <bool NORM, int EPI, typename TY, bool GATHER = false>
+template <bool NORM, int EPI, typename TY, bool GATHER = false, int RT = 1>
 static int launch_fused(const FusedArgs& a, int blocks, hipStream_t s) {
-    const int tiles = (EPI == EPI_GATED || EPI == EPI_QKV) ? 2 : 1;
+    const int tiles = (EPI == EPI_GATED || EPI == EPI_QKV) ? 2 : RT;
     const int waves = pick_waves(blocks, a.K, tiles);
     const size_t lds = waves > 1 ? (size_t)waves * (tiles * 4) * TQK_WAVE * sizeof(float) + (NORM ? (size_t)waves * 16 * sizeof(float) : 0) : 0;
-    skinny_fused_kernel<NORM, EPI, TY, GATHER><<<blocks, waves * TQK_WAVE, lds, s>>>(a);
+    skinny_fused_kernel<NORM, EPI, TY, GATHER, RT><<<blocks, waves * TQK_WAVE, lds, s>>>(a);
     return tqk_check_launch("tqk_skinny_fused");
+}
+
+// the same for 1 or 2 tiles per block
+template <bool NORM, int EPI, typename TY, bool GATHER = false>
+static int launch_tiled(const FusedArgs& a, hipStream_t s) {
+    const int rt = pick_tiles(a.N, a.K);
+    const int blocks = (a.N + 16 * rt - 1) / (16 * rt);
+    if (rt == 2) return launch_fused<NORM, EPI, TY, GATHER, 2>(a, blocks, s);
+    return launch_fused<NORM, EPI, TY, GATHER, 1>(a, blocks, s);
 }
 
 static int check_common(const FusedArgs& a, const char* what) {
@@ -361,14 +401,13 @@ extern "C" int tqk_fused_store(const void* x, const int32_t* x_rows, const float
     TQK_REQUIRE(y, "tqk_fused_store: null output");
     TQK_REQUIRE(y_dtype == TQK_F32 || y_dtype == TQK_BF16, "tqk_fused_store: unknown output dtype %d", y_dtype);
     if (M == 0) return 0;
-    const int blocks = (N + 15) / 16;
     hipStream_t s = (hipStream_t)stream;
     if (x_rows) {
-        if (ss_parts) return y_dtype == TQK_F32 ? launch_fused<true, EPI_STORE, float, true>(a, blocks, s) : launch_fused<true, EPI_STORE, bf16_t, true>(a, blocks, s);
-        return y_dtype == TQK_F32 ? launch_fused<false, EPI_STORE, float, true>(a, blocks, s) : launch_fused<false, EPI_STORE, bf16_t, true>(a, blocks, s);
+        if (ss_parts) return y_dtype == TQK_F32 ? launch_tiled<true, EPI_STORE, float, true>(a, s) : launch_tiled<true, EPI_STORE, bf16_t, true>(a, s);
+        return y_dtype == TQK_F32 ? launch_tiled<false, EPI_STORE, float, true>(a, s) : launch_tiled<false, EPI_STORE, bf16_t, true>(a, s);
     }
-    if (ss_parts) return y_dtype == TQK_F32 ? launch_fused<true, EPI_STORE, float>(a, blocks, s) : launch_fused<true, EPI_STORE, bf16_t>(a, blocks, s);
-    return y_dtype == TQK_F32 ? launch_fused<false, EPI_STORE, float>(a, blocks, s) : launch_fused<false, EPI_STORE, bf16_t>(a, blocks, s);
+    if (ss_parts) return y_dtype == TQK_F32 ? launch_tiled<true, EPI_STORE, float>(a, s) : launch_tiled<true, EPI_STORE, bf16_t>(a, s);
+    return y_dtype == TQK_F32 ? launch_tiled<false, EPI_STORE, float>(a, s) : launch_tiled<false, EPI_STORE, bf16_t>(a, s);
 }
 
 /* y[M, N/2] = silu(gate) * up of the (normalised) product, w = gate rows then up rows. */
@@ -385,11 +424,14 @@ extern "C" int tqk_fused_gated(const void* x, const float* ss_parts, int n_ss_pa
     return ss_parts ? launch_fused<true, EPI_GATED, bf16_t>(a, blocks, s) : launch_fused<false, EPI_GATED, bf16_t>(a, blocks, s);
 }
 
-extern "C" int tqk_fused_residual_parts(int N) { return (N + 15) / 16; }
+extern "C" int tqk_fused_residual_parts(int N, int K) {
+    const int rt = pick_tiles(N, K);
+    return (N + 16 * rt - 1) / (16 * rt);
+}
 
 /* h[M,N] += bfloat16(x w^T) in float32; xw_out = bfloat16(h * next_norm_w) (bfloat16(h)
- * without a weight); ss_out (optional) [tqk_fused_residual_parts(N), 16]: piece b, row m =
- * sum of h[m, 16b..16b+15]^2. */
+ * without a weight); ss_out (optional) [tqk_fused_residual_parts(N, K), 16]: piece b, row m =
+ * the sum of h[m, n]^2 over the columns n of block b. */
 extern "C" int tqk_fused_residual(const void* x, const void* w, float* h, const void* next_norm_w, void* xw_out,
                                   float* ss_out, int M, int N, int K, void* stream) {
     FusedArgs a = {};
@@ -400,7 +442,7 @@ extern "C" int tqk_fused_residual(const void* x, const void* w, float* h, const 
     TQK_REQUIRE(N % 4 == 0, "tqk_fused_residual: N=%d must be a multiple of 4", N);
     TQK_REQUIRE(((((uintptr_t)h) | ((uintptr_t)next_norm_w)) & 15) == 0, "tqk_fused_residual: h and the norm's weight must be 16-byte aligned");
     if (M == 0) return 0;
-    return launch_fused<false, EPI_RESIDUAL, bf16_t>(a, (N + 15) / 16, (hipStream_t)stream);
+    return launch_tiled<false, EPI_RESIDUAL, bf16_t>(a, (hipStream_t)stream);
 }
 
 /* The q, k, v product of a decoding step: the (normalised) product + bias, q and k rotated

@@ -55,8 +55,8 @@ int tqk_fused_store(const void* x, const int32_t* x_rows, const float* ss_parts,
 int tqk_fused_gated(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, void* y,
                     int M, int N, int K, void* stream);
 /* h[M,N] += bfloat16(x w^T) in float32; xw_out = bfloat16(h * next_norm_w) or bfloat16(h);
- * ss_out (optional) [tqk_fused_residual_parts(N), 16] */
-int tqk_fused_residual_parts(int N);
+ * ss_out (optional) [tqk_fused_residual_parts(N, K), 16] */
+int tqk_fused_residual_parts(int N, int K);
 int tqk_fused_residual(const void* x, const void* w, float* h, const void* next_norm_w, void* xw_out,
                        float* ss_out, int M, int N, int K, void* stream);
 /* q, k, v of a decoding step: + bias, rotation (halves over the whole head) at tok_pos[m],

@@ -148,7 +148,7 @@ class Model:
                   for run in s.order] + [self.final_norm]
         if ctx.fuse_small:
             xw = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.bfloat16, device=self.device)
-            ss = torch.empty((max(1, K.fused_residual_parts(s.hidden_size)), 16), dtype=torch.float32, device=self.device)
+            ss = torch.empty(((s.hidden_size + 15) // 16, 16), dtype=torch.float32, device=self.device)      # the most pieces a product gives
             stream = L.Stream(h, xw, ss)
             norm = firsts[0] if getattr(firsts[0], "foldable", False) else None
             K.embed(self.embedding, ctx.dev.tokens, h, copy=xw, copy_weight=norm.weight if norm is not None else None, ss_out=ss)

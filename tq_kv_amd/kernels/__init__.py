@@ -324,17 +324,19 @@ def fused_gated(x, weight_gate_up, out, norm=None):
     return out
 
 
-def fused_residual_parts(n):
-    return int(library().tqk_fused_residual_parts(int(n)))
+def fused_residual_parts(n, k):
+    """In how many pieces fused_residual gives the sums of squares for a weight [n, k]
+    (never more than ceil(n / 16))."""
+    return int(library().tqk_fused_residual_parts(int(n), int(k)))
 
 
 def fused_residual(x, weight, h, xw, next_norm_weight=None, ss_out=None):
     """h[M,N] += bfloat16(x weight^T) (float32 sum); xw = bfloat16(h * next_norm_weight) (or
-    bfloat16(h)); ss_out (optional, float32 [fused_residual_parts(N), 16]): the rows' sums of
+    bfloat16(h)); ss_out (optional, float32 [fused_residual_parts(N, K), 16]): the rows' sums of
     squares in pieces.  Returns the number of pieces."""
     m, k = x.shape
     n = weight.shape[0]
-    parts = fused_residual_parts(n)
+    parts = fused_residual_parts(n, k)
     if ss_out is not None and ss_out.numel() < parts * 16:
         raise KernelError("fused_residual: ss_out holds %d values, %d pieces of 16 are written" % (ss_out.numel(), parts))
     _check(library().tqk_fused_residual(
