@@ -433,7 +433,8 @@ def test_attention_decode_refuses_other_head_sizes():
 
 @pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (3, 1, 96)])
 @pytest.mark.parametrize("window", [0, 70, 12])
-def test_attention_prefill(nh, nkv, d, window):
+@pytest.mark.parametrize("tile", [64, 128])
+def test_attention_prefill(nh, nkv, d, window, tile):
     # sequence 0: 150 new queries at positions 150..299 behind 150 cached ones; sequence 1: a
     # whole prompt of 70; sequence 2: one token at position 0.  Pages scrambled, unread places NaN.
     spans = [(150, 300), (0, 70), (0, 1)]
@@ -459,13 +460,14 @@ def test_attention_prefill(nh, nkv, d, window):
     pos = torch.cat([torch.arange(a, b) for a, b in spans])
     tile_seq, tile_tok0, tile_count, off = [], [], [], 0
     for i, (a, b) in enumerate(spans):
-        for s0 in range(0, b - a, 64):
-            tile_seq.append(i), tile_tok0.append(off + s0), tile_count.append(min(64, b - a - s0))
+        for s0 in range(0, b - a, tile):
+            tile_seq.append(i), tile_tok0.append(off + s0), tile_count.append(min(tile, b - a - s0))
         off += b - a
     out = torch.empty(q.shape[0], nh * d, dtype=torch.bfloat16, device=DEV)
     scale = 1 / math.sqrt(d)
     K.attention_prefill(q, keys, values, pos.to(torch.int32).to(DEV), ints(tables), ints(tile_seq), ints(tile_tok0),
-                        ints(tile_count), ints([a for a, _ in spans]), ints([b - a for a, b in spans]), window, scale, out)
+                        ints(tile_count), ints([a for a, _ in spans]), ints([b - a for a, b in spans]), window, scale, out,
+                        tile_queries=tile)
     off = 0
     for i, (a, b) in enumerate(spans):
         want = attention_reference(qs[i].float(), ks[i], vs[i], torch.arange(a, b), window, scale)

@@ -107,9 +107,9 @@ int tqk_attention_prefill_supported(int head_dim);
 int tqk_attention_prefill(const void* q, const void* keys, const void* values, const int32_t* tok_pos,
                           const int32_t* page_table, int table_width, int n_seqs, int n_pages,
                           const int32_t* tile_seq, const int32_t* tile_tok0, const int32_t* tile_count,
-                          int n_tiles, const int32_t* seq_start, const int32_t* seq_new, int window,
-                          float scale, void* out, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
-                          void* stream);
+                          int n_tiles, int tile_queries, const int32_t* seq_start, const int32_t* seq_new,
+                          int window, float scale, void* out, int n_tokens, int n_heads, int n_kv_heads,
+                          int head_dim, void* stream);
 
 /* out[t, i] = silu(gate_up[t, i]) * gate_up[t, inter + i] */
 int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int inter, void* stream);

@@ -11,7 +11,10 @@ import numpy as np
 import torch
 
 
-TILE = 64      # queries per tile of the prompt attention kernel
+def tile_queries(n_tokens):
+    """Queries per tile of the prompt attention kernel: 128 where there is work for many
+    blocks anyway (a query then costs less), 64 for small steps (fewer idle lanes)."""
+    return 128 if n_tokens >= 1024 else 64
 
 
 class _Arrays:
@@ -78,13 +81,14 @@ class StepContext:
                     raise IndexError("wanted place %d is outside the %d tokens of sequence %d" % (j, lens[i], i))
                 rows.append(int(host.cu[i]) + int(j))
         host.want_rows = np.asarray(rows, dtype=np.int32)
-        # tiles of up to TILE consecutive queries of one sequence, for the prompt attention kernel
+        # tiles of consecutive queries of one sequence, for the prompt attention kernel
+        self.tile_queries = tile = tile_queries(self.n_tokens)
         t_seq, t_tok0, t_count = [], [], []
         for i, n in enumerate(lens):
-            for a in range(0, n, TILE):
+            for a in range(0, n, tile):
                 t_seq.append(i)
                 t_tok0.append(int(host.cu[i]) + a)
-                t_count.append(min(TILE, n - a))
+                t_count.append(min(tile, n - a))
         # longest first (a tile's work grows with the position of its last query)
         order = sorted(range(len(t_seq)), key=lambda k: -(int(host.tok_pos[t_tok0[k]]) + t_count[k]))
         host.tile_seq = np.asarray([t_seq[k] for k in order], dtype=np.int32)

@@ -266,9 +266,10 @@ def attention_prefill_supported(head_dim):
 
 
 def attention_prefill(q, keys, values, tok_pos, page_table, tile_seq, tile_tok0, tile_count, seq_start, seq_new,
-                      window, scale, out):
-    """Causal attention of tiles of up to 64 consecutive queries (q [T, heads, d] bfloat16)
-    over the paged cache; out [T, heads*d]."""
+                      window, scale, out, tile_queries=64):
+    """Causal attention of tiles of up to tile_queries (64 or 128) consecutive queries
+    (q [T, heads, d] bfloat16) over the paged cache; out [T, heads*d].  tile_count must not
+    exceed tile_queries (the caller built the tiles; the kernel covers no more)."""
     n, n_heads, head_dim = q.shape
     n_pages, n_kv_heads = keys.shape[0], keys.shape[1]
     n_seqs, width = page_table.shape
@@ -278,7 +279,7 @@ def attention_prefill(q, keys, values, tok_pos, page_table, tile_seq, tile_tok0,
         _dev(values, "values", torch.bfloat16, (n_pages, n_kv_heads, head_dim, 64)),
         _dev(tok_pos, "tok_pos", torch.int32, (n,)), _dev(page_table, "page_table", torch.int32), width, n_seqs, n_pages,
         _dev(tile_seq, "tile_seq", torch.int32, (n_tiles,)), _dev(tile_tok0, "tile_tok0", torch.int32, (n_tiles,)),
-        _dev(tile_count, "tile_count", torch.int32, (n_tiles,)), n_tiles,
+        _dev(tile_count, "tile_count", torch.int32, (n_tiles,)), n_tiles, int(tile_queries),
         _dev(seq_start, "seq_start", torch.int32, (n_seqs,)), _dev(seq_new, "seq_new", torch.int32, (n_seqs,)),
         int(window or 0), ctypes.c_float(scale), _dev(out, "out", torch.bfloat16, (n, n_heads * head_dim)),
         n, n_heads, n_kv_heads, head_dim, _stream()), "attention_prefill")

@@ -151,5 +151,5 @@ def attend(q, entry, table, ctx, window, scale, out):
     if q.dtype == torch.bfloat16 and POLICY["prefill_mfma"] and K.attention_prefill_supported(head_dim):
         d = ctx.dev
         return K.attention_prefill(q, entry.keys, entry.values, d.tok_pos, table, d.tile_seq, d.tile_tok0, d.tile_count,
-                                   d.seq_start, d.seq_new, window, scale, out)
+                                   d.seq_start, d.seq_new, window, scale, out, tile_queries=ctx.tile_queries)
     return K.attention(q, entry.keys, entry.values, ctx.dev.tok_seq, ctx.dev.tok_pos, table, window, scale, out)
