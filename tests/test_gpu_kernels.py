@@ -176,6 +176,34 @@ def test_rope_store(dtype, style, rot):
     torch.testing.assert_close(q.float().cpu(), want_q, **TOL[dtype])
 
 
+@pytest.mark.parametrize("with_bias", [True, False])
+@pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (3, 1, 64), (7, 7, 8)])
+def test_rope_store_vector_kernel_equals_the_general_one(nh, nkv, d, with_bias):
+    # bfloat16, halves over the whole head: the kernel with 8-byte accesses.  A float32 bias of
+    # the same values sends the same work through the general kernel.
+    n_pages, n = 9, 6
+    tok_seq, tok_pos = ints([0, 0, 1, 1, 1, 2]), ints([63, 64, 0, 1, 2, 399])
+    table = ints([[3, 8, -1, -1, -1, -1, -1], [0, -1, -1, -1, -1, -1, -1], [4, 4, 4, 4, 4, 4, 7]])
+    qkv = rand(n, (nh + 2 * nkv) * d, seed=12, dtype=torch.bfloat16)
+    bias = rand((nh + 2 * nkv) * d, seed=13, dtype=torch.bfloat16) if with_bias else None
+    c, s = plain.rope_tables(d, 1e4, 300)                # position 399 is beyond the table: not rotated
+    cos, sin = c.to(DEV), s.to(DEV)
+    results = []
+    for general in (False, True):
+        keys, values = make_cache(n_pages, nkv, d, torch.bfloat16)
+        q = torch.empty(n, nh, d, dtype=torch.bfloat16, device=DEV)
+        b = bias
+        if general:
+            b = bias.float() if with_bias else torch.zeros((nh + 2 * nkv) * d, device=DEV)
+        K.rope_store(qkv, b, cos, sin, d, K.STYLE_HALVES, tok_seq, tok_pos, table, keys, values, q, nh, nkv, d)
+        results.append((q, keys, values))
+    for a, b in zip(*results):
+        assert torch.equal(torch.isnan(a.float()), torch.isnan(b.float()))          # the same places written
+        ok = ~torch.isnan(a.float())
+        torch.testing.assert_close(a.float()[ok], b.float()[ok], atol=1e-2, rtol=1e-2)
+        assert ok.any()
+
+
 def paged(k, v, page_ids, n_pages, dtype):
     """Lay k, v [nkv, S, d] out in pages given by page_ids; everything else is NaN."""
     nkv, s, d = k.shape

@@ -295,6 +295,78 @@ __global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restri
     }
 }
 
+// The common case in bfloat16 (halves layout over the whole head, head_dim a multiple of 8): a
+// thread takes 4 neighbouring elements of the first half and the 4 they rotate with, 8 bytes
+// per load and store; 16 heads of a token per block.
+__global__ void rope_store_halves_bf16_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict__ bias,
+                                              const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+                                              int max_positions, const int32_t* __restrict__ tok_seq,
+                                              const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table,
+                                              int table_width, bf16_t* __restrict__ keys, bf16_t* __restrict__ values,
+                                              bf16_t* __restrict__ q_out, int n_heads, int n_kv_heads, int head_dim,
+                                              int write_kv) {
+    const int t = blockIdx.x;
+    const int per_head = head_dim / 8;                  // threads per head
+    const int slot = blockIdx.y * blockDim.x + threadIdx.x;
+    const int head = slot / per_head, i = (slot % per_head) * 4, half = head_dim / 2;
+    if (head >= n_heads + 2 * n_kv_heads) return;
+    const int kind = head < n_heads ? 0 : (head < n_heads + n_kv_heads ? 1 : 2);
+    if (kind != 0 && !write_kv) return;
+    const int pos = tok_pos[t];
+    const size_t total = (size_t)(n_heads + 2 * n_kv_heads) * head_dim;
+    const bf16_t* src = qkv + (size_t)t * total + (size_t)head * head_dim;
+    const uint2 lo_raw = *reinterpret_cast<const uint2*>(src + i), hi_raw = *reinterpret_cast<const uint2*>(src + i + half);
+    float lo[4] = {__uint_as_float(lo_raw.x << 16), __uint_as_float(lo_raw.x & 0xffff0000u),
+                   __uint_as_float(lo_raw.y << 16), __uint_as_float(lo_raw.y & 0xffff0000u)};
+    float hi[4] = {__uint_as_float(hi_raw.x << 16), __uint_as_float(hi_raw.x & 0xffff0000u),
+                   __uint_as_float(hi_raw.y << 16), __uint_as_float(hi_raw.y & 0xffff0000u)};
+    if (bias) {
+        const bf16_t* b = bias + (size_t)head * head_dim;
+        const uint2 bl = *reinterpret_cast<const uint2*>(b + i), bh = *reinterpret_cast<const uint2*>(b + i + half);
+        lo[0] += __uint_as_float(bl.x << 16); lo[1] += __uint_as_float(bl.x & 0xffff0000u);
+        lo[2] += __uint_as_float(bl.y << 16); lo[3] += __uint_as_float(bl.y & 0xffff0000u);
+        hi[0] += __uint_as_float(bh.x << 16); hi[1] += __uint_as_float(bh.x & 0xffff0000u);
+        hi[2] += __uint_as_float(bh.y << 16); hi[3] += __uint_as_float(bh.y & 0xffff0000u);
+    }
+    if (kind != 2 && pos < max_positions) {
+        const float4 c4 = *reinterpret_cast<const float4*>(cos_table + (size_t)pos * half + i);
+        const float4 s4 = *reinterpret_cast<const float4*>(sin_table + (size_t)pos * half + i);
+        const float c[4] = {c4.x, c4.y, c4.z, c4.w}, sn[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float x0 = lo[k], x1 = hi[k];
+            lo[k] = x0 * c[k] - x1 * sn[k];
+            hi[k] = x0 * sn[k] + x1 * c[k];
+        }
+    }
+    uint32_t lo_bits[4], hi_bits[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { lo_bits[k] = float_to_bf16_bits(lo[k]); hi_bits[k] = float_to_bf16_bits(hi[k]); }
+    if (kind == 2) {
+        // values are kept transposed inside a page: [kv head][head_dim][place of the position]
+        const int kvh = head - n_heads - n_kv_heads;
+        const int page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+        if (page < 0) return;                          // the host never lets this happen
+        bf16_t* dst = values + ((size_t)page * n_kv_heads + kvh) * TQK_PAGE * head_dim + value_place(pos % TQK_PAGE);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            dst[(size_t)(i + k) * TQK_PAGE].bits = (uint16_t)lo_bits[k];
+            dst[(size_t)(i + half + k) * TQK_PAGE].bits = (uint16_t)hi_bits[k];
+        }
+        return;
+    }
+    bf16_t* dst;
+    if (kind == 0) {
+        dst = q_out + ((size_t)t * n_heads + head) * head_dim;
+    } else {
+        const int page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+        if (page < 0) return;
+        dst = keys + (((size_t)page * n_kv_heads + head - n_heads) * TQK_PAGE + pos % TQK_PAGE) * head_dim;
+    }
+    *reinterpret_cast<uint2*>(dst + i) = make_uint2(lo_bits[0] | (lo_bits[1] << 16), lo_bits[2] | (lo_bits[3] << 16));
+    *reinterpret_cast<uint2*>(dst + i + half) = make_uint2(hi_bits[0] | (hi_bits[1] << 16), hi_bits[2] | (hi_bits[3] << 16));
+}
+
 extern "C" int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, int bias_dtype,
                               const float* cos_table, const float* sin_table, int rot_dim, int style,
                               int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
@@ -317,6 +389,16 @@ extern "C" int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, 
     }
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    if (act_dtype == TQK_BF16 && (!bias || bias_dtype == TQK_BF16) && style == 1 && rot_dim == head_dim && head_dim % 8 == 0 &&
+        ((((uintptr_t)qkv) | ((uintptr_t)bias) | ((uintptr_t)cos_table) | ((uintptr_t)sin_table) | ((uintptr_t)keys) |
+          ((uintptr_t)q_out)) & 15) == 0) {
+        const int slots = (n_heads + 2 * n_kv_heads) * (head_dim / 8);
+        dim3 vgrid(n_tokens, (slots + 255) / 256);
+        rope_store_halves_bf16_kernel<<<vgrid, 256, 0, s>>>(
+            (const bf16_t*)qkv, (const bf16_t*)bias, cos_table, sin_table, max_positions, tok_seq, tok_pos, page_table,
+            table_width, (bf16_t*)keys, (bf16_t*)values, (bf16_t*)q_out, n_heads, n_kv_heads, head_dim, write_kv);
+        return tqk_check_launch("tqk_rope_store");
+    }
     dim3 grid(n_tokens, (n_heads + 2 * n_kv_heads + 3) / 4);
     const int threads = 4 * TQK_WAVE;
 #define LAUNCH(TA, TB) rope_store_kernel<TA, TB><<<grid, threads, 0, s>>>( \
