@@ -28,7 +28,7 @@ def ints(values):
 
 
 def test_library_is_built_and_loaded():
-    assert K.library().tqk_abi_version() == 2
+    assert K.library().tqk_abi_version() == 3
     assert K.library_path().endswith(".so")
     with pytest.raises(K.KernelError, match="GPU only"):
         K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
@@ -307,19 +307,34 @@ def test_argmax_and_ties():
 def test_repeat_penalty():
     logits = rand(3, 1001, seed=22)
     base = logits.clone().cpu()
-    hist = ints([[5, 9, 5, 1000, 5, 0, 0, 0], [0] * 8, [7, 7, 7, 7, 7, 7, 7, 7]])
-    hist_len = ints([5, 0, 8])
-    K.repeat_penalty(logits, ints([0, 1, 2]), hist, hist_len, 1.3)
+    histories = [[5, 9, 5, 1000, 5], [], [7, 7, 7, 7, 7, 7, 7, 7]]
+    hist = torch.zeros(3, 8, dtype=torch.int32, device=DEV)
+    times, hist_len = torch.zeros_like(hist), ints([0, 0, 0])
+    for step in range(8):                            # the histories grow token by token, as in generation
+        reqs = [r for r in range(3) if step < len(histories[r])]
+        K.append_history(ints([histories[r][step] for r in reqs]), ints(reqs), hist, times, hist_len)
+    assert hist_len.tolist() == [5, 0, 8] and hist[0, :5].tolist() == histories[0]
+    assert times[0, :5].tolist() == [0, 1, 0, 1, 3] and times[2].tolist() == [0] * 7 + [8]
+    K.repeat_penalty(logits, ints([0, 1, 2]), hist, times, hist_len, 1.3)
     for r in range(3):
-        want = plain.apply_repeat_penalty(base[r], hist[r, :hist_len[r]].tolist(), 1.3)
+        want = plain.apply_repeat_penalty(base[r], histories[r], 1.3)
         torch.testing.assert_close(logits[r].cpu(), want, atol=0, rtol=1e-6)
     # rows may point at any request
     logits2 = base.clone().to(DEV)
-    K.repeat_penalty(logits2, ints([2, 2, 0]), hist, hist_len, 2.0)
+    K.repeat_penalty(logits2, ints([2, 2, 0]), hist, times, hist_len, 2.0)
     torch.testing.assert_close(logits2[1].cpu(), plain.apply_repeat_penalty(base[1], [7] * 8, 2.0), atol=0, rtol=1e-6)
-    tokens = ints([11, 12, 13])
-    K.append_history(tokens, ints([0, 1, 2]), hist, hist_len)
+    K.append_history(ints([11, 12, 13]), ints([0, 1, 2]), hist, times, hist_len)
     assert hist_len.tolist() == [6, 1, 8] and hist[0, 5].item() == 11 and hist[1, 0].item() == 12   # request 2 is full
+    # a long history with many repeats: one pass each
+    n = 3000
+    long_hist = torch.randint(0, 50, (n,)).tolist()
+    h2, t2, l2 = torch.zeros(1, n, dtype=torch.int32, device=DEV), torch.zeros(1, n, dtype=torch.int32, device=DEV), ints([0])
+    for tok in long_hist:
+        K.append_history(ints([tok]), ints([0]), h2, t2, l2)
+    z = rand(1, 1001, seed=25)
+    want = plain.apply_repeat_penalty(z[0].cpu(), long_hist, 1.01)
+    K.repeat_penalty(z, ints([0]), h2, t2, l2, 1.01)
+    torch.testing.assert_close(z[0].cpu(), want, atol=0, rtol=1e-5)
 
 
 def draw(logits, temperature, top_k, top_p, us):
@@ -351,13 +366,32 @@ def test_sample_inverse_cdf_and_cuts():
 
 
 @pytest.mark.parametrize("vocab,top_k,top_p,temperature", [(5003, 0, 1.0, 0.8), (5003, 40, 0.9, 0.7), (1000, 0, 0.5, 1.3),
-                                                           (151936, 40, 0.9, 0.7), (151936, 0, 0.95, 1.0), (300, 1000, 1.0, 1.0)])
+                                                           (151936, 40, 0.9, 0.7), (151936, 0, 0.95, 1.0), (300, 1000, 1.0, 1.0),
+                                                           (151936, 256, 0.8, 1.0), (151936, 300, 0.8, 1.0), (20000, 200, 1.0, 1.2),
+                                                           (4865, 1, 0.5, 1.0), (9000, 40, 0.3, 0.7)])
 def test_sample_agrees_with_the_plain_rule(vocab, top_k, top_p, temperature):
     logits = rand(1, vocab, seed=23, scale=3.0)
     us = [0.001, 0.13, 0.37, 0.5, 0.77, 0.93, 0.9999]
     got = draw(logits, temperature, top_k, top_p, us)
     want = [plain.sample_token(logits[0].cpu(), [], temperature, top_k, top_p, 1.0, u) for u in us]
     assert got == want
+
+
+def test_sample_top_k_over_chunks_of_the_row():
+    # top-k first reduces every chunk of a few thousand logits to its own k best: equal logits all
+    # over the row (the k lowest ids are kept), the best ones in far-apart chunks, NaN in between
+    flat = torch.zeros(1, 12000, device=DEV)
+    assert draw(flat, 1.0, 50, 1.0, [0.0, 0.011, 0.5, 0.985, 0.999]) == [0, 0, 25, 49, 49]
+    z = rand(1, 30000, seed=24, scale=1.0)
+    z[0, ::7] = float("nan")
+    best = [29999, 5, 14001, 9000]
+    for rank, i in enumerate(best):
+        z[0, i] = 20.0 - rank
+    # in order of id the weights are e^-1, e^-3, e^-2, e^0 of the total 1.5530: cuts at 0.2369, 0.2690, 0.3561
+    assert draw(z, 1.0, 4, 1.0, [0.0, 0.23, 0.24, 0.265, 0.275, 0.35, 0.36, 0.999]) == [5, 5, 9000, 9000, 14001, 14001, 29999, 29999]
+    assert draw(z, 1.0, 2, 1.0, [0.0, 0.26, 0.27, 0.99]) == [5, 5, 29999, 29999]       # e^-1 / (1 + e^-1) = 0.2689 first, by id
+    assert draw(z, 1.0, 4, 0.7, [0.0, 0.26, 0.27, 0.99]) == [5, 5, 29999, 29999]       # from the largest down 0.6439 < 0.7 <= 0.8808: two kept
+    assert draw(torch.full((1, 6000), float("nan"), device=DEV), 1.0, 10, 1.0, [0.5]) == [0]
 
 
 def test_sample_frequencies_follow_the_softmax():

@@ -141,25 +141,51 @@ __device__ __forceinline__ float block_max_f(float v, float* scratch) {
     return m;
 }
 
+// The radix-select step over a histogram of 256 bins in LDS, by the block's first wave: the
+// highest bin b such that the bins above it hold fewer than `remaining` entries and with it
+// at least that many; `remaining` is lowered by what the bins above hold.  Lane 0 gets the result.
+__device__ __forceinline__ void pick_bin(const int* hist, int remaining, int* bin, int* left) {
+    const int lane = threadIdx.x;                      // 0..63: bins 255-4*lane down to 252-4*lane
+    int h[4], sum = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { h[i] = hist[255 - (4 * lane + i)]; sum += h[i]; }
+    int incl = sum;
+#pragma unroll
+    for (int o = 1; o < TQK_WAVE; o <<= 1) {
+        const int up = __shfl_up(incl, o, TQK_WAVE);
+        if (lane >= o) incl += up;
+    }
+    int before = incl - sum, found = -1, found_before = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (found < 0 && before + h[i] >= remaining) { found = 255 - (4 * lane + i); found_before = before; }
+        before += h[i];
+    }
+    // the first lane that found one
+    const unsigned long long who = __ballot(found >= 0);
+    const int first = who ? __ffsll((long long)who) - 1 : TQK_WAVE - 1;
+    const int b = __shfl(found, first, TQK_WAVE), fb = __shfl(found_before, first, TQK_WAVE);
+    *bin = who ? b : 0;
+    *left = who ? remaining - fb : remaining - (__shfl(incl, TQK_WAVE - 1, TQK_WAVE) - hist[0]);
+}
+
 // ---- repeat penalty ----------------------------------------------------------------
 // src/engine.rs:403-419: for every generated token, once per occurrence,
-// l > 0 ? l / penalty : l * penalty.  The thread that holds a token's first occurrence
-// applies the penalty as often as the token occurs.
+// l > 0 ? l / penalty : l * penalty.  The history of a request is kept as its tokens and, for
+// each entry, how often the penalty is to be applied on its behalf: for the last occurrence
+// of a token the number of its occurrences, for the earlier ones 0.  Appending a token keeps
+// that up (one pass over the request's history), so applying the penalty is one pass too.
 __global__ void repeat_penalty_kernel(float* __restrict__ logits, int vocab, const int32_t* __restrict__ row_req,
-                                      const int32_t* __restrict__ hist, int hist_cap,
+                                      const int32_t* __restrict__ hist, const int32_t* __restrict__ times, int hist_cap,
                                       const int32_t* __restrict__ hist_len, float penalty) {
     float* row = logits + (size_t)blockIdx.x * vocab;
     const int req = row_req[blockIdx.x];
     const int32_t* h = hist + (size_t)req * hist_cap;
+    const int32_t* tm = times + (size_t)req * hist_cap;
     const int n = min(hist_len[req], hist_cap);
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
-        const int tok = h[i];
-        if (tok < 0 || tok >= vocab) continue;
-        bool first = true;
-        for (int j = 0; j < i; ++j) if (h[j] == tok) { first = false; break; }
-        if (!first) continue;
-        int count = 1;
-        for (int j = i + 1; j < n; ++j) count += (h[j] == tok);
+        const int count = tm[i], tok = h[i];
+        if (count <= 0 || tok < 0 || tok >= vocab) continue;
         float z = row[tok];
         for (int c = 0; c < count; ++c) z = z > 0.f ? z / penalty : z * penalty;
         row[tok] = z;
@@ -167,31 +193,41 @@ __global__ void repeat_penalty_kernel(float* __restrict__ logits, int vocab, con
 }
 
 extern "C" int tqk_repeat_penalty(float* logits, int n_rows, int vocab, const int32_t* row_req,
-                                  const int32_t* hist, int hist_cap, const int32_t* hist_len, int n_req,
-                                  float penalty, void* stream) {
-    TQK_REQUIRE(logits && row_req && hist && hist_len, "tqk_repeat_penalty: null pointer");
+                                  const int32_t* hist, const int32_t* times, int hist_cap, const int32_t* hist_len,
+                                  int n_req, float penalty, void* stream) {
+    TQK_REQUIRE(logits && row_req && hist && times && hist_len, "tqk_repeat_penalty: null pointer");
     TQK_REQUIRE(n_rows >= 0 && vocab > 0 && hist_cap > 0 && n_req > 0, "tqk_repeat_penalty: bad sizes");
     TQK_REQUIRE(penalty > 0.f, "tqk_repeat_penalty: penalty must be positive, got %g", (double)penalty);
     if (n_rows == 0) return 0;
-    repeat_penalty_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(logits, vocab, row_req, hist, hist_cap, hist_len, penalty);
+    repeat_penalty_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(logits, vocab, row_req, hist, times, hist_cap, hist_len, penalty);
     return tqk_check_launch("tqk_repeat_penalty");
 }
 
+// One block per row: the row's token goes to the end of its request's history; the earlier
+// occurrences of the token hand their count over to it.  Rows of one call name different requests.
 __global__ void append_history_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ row_req,
-                                      int32_t* __restrict__ hist, int hist_cap, int32_t* __restrict__ hist_len, int n_rows) {
-    const int r = blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= n_rows) return;
-    const int req = row_req[r];
+                                      int32_t* __restrict__ hist, int32_t* __restrict__ times, int hist_cap,
+                                      int32_t* __restrict__ hist_len) {
+    __shared__ int scratch[256 / TQK_WAVE];
+    const int r = blockIdx.x;
+    const int req = row_req[r], tok = tokens[r];
+    int32_t* h = hist + (size_t)req * hist_cap;
+    int32_t* tm = times + (size_t)req * hist_cap;
     const int n = hist_len[req];
-    if (n < hist_cap) { hist[(size_t)req * hist_cap + n] = tokens[r]; hist_len[req] = n + 1; }
+    if (n >= hist_cap) return;                         // full: the token is dropped
+    int seen = 0;
+    for (int i = threadIdx.x; i < n; i += blockDim.x)
+        if (h[i] == tok) { ++seen; tm[i] = 0; }
+    const int total = block_sum_any<int>(seen, scratch);
+    if (threadIdx.x == 0) { h[n] = tok; tm[n] = total + 1; hist_len[req] = n + 1; }
 }
 
-extern "C" int tqk_append_history(const int32_t* tokens, const int32_t* row_req, int32_t* hist, int hist_cap,
-                                  int32_t* hist_len, int n_rows, void* stream) {
-    TQK_REQUIRE(tokens && row_req && hist && hist_len, "tqk_append_history: null pointer");
+extern "C" int tqk_append_history(const int32_t* tokens, const int32_t* row_req, int32_t* hist, int32_t* times,
+                                  int hist_cap, int32_t* hist_len, int n_rows, void* stream) {
+    TQK_REQUIRE(tokens && row_req && hist && times && hist_len, "tqk_append_history: null pointer");
     TQK_REQUIRE(n_rows >= 0 && hist_cap > 0, "tqk_append_history: bad sizes");
     if (n_rows == 0) return 0;
-    append_history_kernel<<<(n_rows + 255) / 256, 256, 0, (hipStream_t)stream>>>(tokens, row_req, hist, hist_cap, hist_len, n_rows);
+    append_history_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(tokens, row_req, hist, times, hist_cap, hist_len);
     return tqk_check_launch("tqk_append_history");
 }
 
@@ -234,11 +270,10 @@ void sample_kernel(const float* __restrict__ logits, int vocab, float temperatur
                 if (z == z && (key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 0xff], 1);
             }
             __syncthreads();
-            if (tid == 0) {
-                int remaining = sh_remaining, b = 255;
-                for (; b > 0; --b) { if (hist[b] >= remaining) break; remaining -= hist[b]; }
-                sh_prefix = prefix | ((uint32_t)b << shift);
-                sh_remaining = remaining;
+            if (tid < TQK_WAVE) {
+                int b, left;
+                pick_bin(hist, sh_remaining, &b, &left);
+                if (tid == 0) { sh_prefix = prefix | ((uint32_t)b << shift); sh_remaining = left; }
             }
             __syncthreads();
         }
@@ -353,14 +388,215 @@ void sample_kernel(const float* __restrict__ logits, int vocab, float temperatur
 #undef WEIGHT
 }
 
+// ---- the usual case, 0 < top_k <= 256: candidates first ---------------------------------
+// Only the top_k largest logits of a row can be drawn, so the row is read once, by many
+// blocks: each block takes a chunk of the row into LDS and finds the chunk's top_k there
+// (the row's top_k are among the chunks' top_k); then one block per row picks the top_k of
+// the candidates and does top-p and the draw on those few, with the rules stated above.
+#define CAND_THREADS 256
+#define CAND_CHUNK 4864            // most logits per chunk (19 per thread; keys in LDS)
+#define CAND_MAX_K 256
+#define CAND_MAX_CHUNKS 64
+#define CAND_MAX_TOTAL 6144        // most candidates per row in the second kernel's LDS (48 KB)
+
+// key of a logit for selection: 0 for NaN (never taken), else float_key > 0
+__device__ __forceinline__ uint32_t select_key(float z) { return z == z ? float_key(z) : 0u; }
+__device__ __forceinline__ float key_value(uint32_t key) {
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
+// Among keys[0..n) in LDS (n > want > 0): the key of the want-th largest, and how many of the
+// entries with exactly that key belong to the want largest (lower indices first).  hist: 256
+// ints in LDS; box: 2 uint32 in LDS.  Every thread of the block calls it.
+__device__ void radix_select_lds(const uint32_t* keys, int n, int want, int* hist, uint32_t* box,
+                                 uint32_t* tkey, int* ties) {
+    if (threadIdx.x == 0) { box[0] = 0; box[1] = (uint32_t)want; }
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        for (int b = threadIdx.x; b < 256; b += blockDim.x) hist[b] = 0;
+        __syncthreads();
+        const uint32_t prefix = box[0];
+        const uint32_t mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
+        for (int i = threadIdx.x; i < n; i += blockDim.x) {
+            const uint32_t key = keys[i];
+            if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 0xff], 1);
+        }
+        __syncthreads();
+        if (threadIdx.x < TQK_WAVE) {
+            int b, left;
+            pick_bin(hist, (int)box[1], &b, &left);
+            if (threadIdx.x == 0) { box[0] = prefix | ((uint32_t)b << shift); box[1] = (uint32_t)left; }
+        }
+        __syncthreads();
+    }
+    *tkey = box[0];
+    *ties = (int)box[1];
+}
+
+// The entries of keys[0..n) that belong to the `want` largest (all of them if n <= want; key 0
+// never), copied in order of index to out_key / out_id (ids: first_id + index, or ids[index]).
+// Returns how many.  scan: one int per wave in LDS.
+__device__ int take_largest(const uint32_t* keys, const int32_t* ids, int first_id, int n, int want,
+                            int* hist, uint32_t* box, int* scan, uint32_t* out_key, int32_t* out_id) {
+    uint32_t tkey = 0;
+    int ties = 0x7fffffff;
+    if (n > want) radix_select_lds(keys, n, want, hist, box, &tkey, &ties);
+    const int seg = (n + blockDim.x - 1) / blockDim.x;
+    const int begin = min(n, (int)threadIdx.x * seg), end = min(n, begin + seg);
+    int my_ties = 0, my_above = 0;
+    for (int i = begin; i < end; ++i) {
+        const uint32_t key = keys[i];
+        my_ties += (key == tkey && key != 0);
+        my_above += (key > tkey);
+    }
+    int all_ties, all_above;
+    const int ties_before = block_exclusive_scan<int>(my_ties, scan, &all_ties);
+    // of this thread's ties, those with rank below `ties` are taken
+    const int my_taken_ties = max(0, min(my_ties, ties - ties_before));
+    int total;
+    int at = block_exclusive_scan<int>(my_above + my_taken_ties, scan, &total);
+    (void)all_above;
+    int rank = ties_before;
+    for (int i = begin; i < end; ++i) {
+        const uint32_t key = keys[i];
+        bool take = key > tkey;
+        if (key == tkey && key != 0) { take = rank < ties; ++rank; }
+        if (take) { out_key[at] = key; out_id[at] = ids ? ids[i] : first_id + i; ++at; }
+    }
+    return total;
+}
+
+__global__ __launch_bounds__(CAND_THREADS)
+void sample_candidates_kernel(const float* __restrict__ logits, int vocab, int chunk, int n_chunks, int top_k,
+                              uint32_t* __restrict__ cand_key, int32_t* __restrict__ cand_id, int32_t* __restrict__ cand_n) {
+    __shared__ uint32_t keys[CAND_CHUNK];
+    __shared__ int hist[256];
+    __shared__ uint32_t box[2];
+    __shared__ int scan[CAND_THREADS / TQK_WAVE];
+    const int row = blockIdx.y, blk = blockIdx.x;
+    const int first = blk * chunk, n = max(0, min(vocab - first, chunk));
+    const float* src = logits + (size_t)row * vocab + first;
+    for (int i = threadIdx.x; i < n; i += CAND_THREADS) keys[i] = select_key(src[i]);
+    __syncthreads();
+    const size_t slot = (size_t)row * n_chunks + blk;
+    const int taken = take_largest(keys, nullptr, first, n, top_k, hist, box, scan,
+                                   cand_key + slot * top_k, cand_id + slot * top_k);
+    if (threadIdx.x == 0) cand_n[slot] = taken;
+}
+
+__global__ __launch_bounds__(CAND_THREADS)
+void sample_draw_kernel(const uint32_t* __restrict__ cand_key, const int32_t* __restrict__ cand_id,
+                        const int32_t* __restrict__ cand_n, int n_chunks, int top_k, float temperature, float top_p,
+                        const float* __restrict__ uniforms, int32_t* __restrict__ out) {
+    extern __shared__ uint32_t pool[];                 // keys [n_chunks * top_k], then ids
+    __shared__ int hist[256];
+    __shared__ uint32_t box[2];
+    __shared__ int scan[CAND_THREADS / TQK_WAVE];
+    __shared__ float fscan[CAND_THREADS / TQK_WAVE];
+    __shared__ uint32_t fkey[CAND_MAX_K];              // the top_k, in order of id
+    __shared__ int32_t fid[CAND_MAX_K];
+    __shared__ float sorted_w[CAND_MAX_K];             // weights from the largest down
+    __shared__ uint32_t sorted_key[CAND_MAX_K];
+    __shared__ int sh_first;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    uint32_t* keys = pool;
+    int32_t* ids = reinterpret_cast<int32_t*>(pool + (size_t)n_chunks * top_k);
+
+    // the chunks' candidates, chunk after chunk: in order of id
+    int n = 0;
+    for (int c = 0; c < n_chunks; ++c) {
+        const size_t slot = (size_t)row * n_chunks + c;
+        const int cn = cand_n[slot];
+        for (int i = tid; i < cn; i += CAND_THREADS) { keys[n + i] = cand_key[slot * top_k + i]; ids[n + i] = cand_id[slot * top_k + i]; }
+        n += cn;
+    }
+    __syncthreads();
+    const int m = take_largest(keys, ids, 0, n, top_k, hist, box, scan, fkey, fid);
+    __syncthreads();
+    if (m == 0) {                                      // a row of NaN
+        if (tid == 0) out[row] = 0;
+        return;
+    }
+    // rank from the largest down, lower ids first among equals (the list is in order of id)
+    const uint32_t my_key = tid < m ? fkey[tid] : 0u;
+    int rank = 0;
+    uint32_t kmax = 0;
+    for (int j = 0; j < m; ++j) {
+        const uint32_t kj = fkey[j];
+        kmax = max(kmax, kj);
+        rank += (kj > my_key) || (kj == my_key && j < tid);
+    }
+    const float inv_t = 1.f / temperature;
+    const float zmax = key_value(kmax);
+    const float my_w = tid < m ? expf((key_value(my_key) - zmax) * inv_t) : 0.f;
+    if (tid < m) { sorted_w[rank] = my_w; sorted_key[rank] = my_key; }
+    __syncthreads();
+    // top-p: the place, from the largest down, where the cumulative weight first reaches top_p of the total
+    uint32_t cut_key = 0;                              // keep keys >= cut_key
+    if (top_p < 1.f) {
+        const float w = tid < m ? sorted_w[tid] : 0.f;
+        float total;
+        const float before = block_exclusive_scan<float>(w, fscan, &total);
+        if (tid == 0) sh_first = m - 1;
+        __syncthreads();
+        if (tid < m && before + w >= top_p * total) atomicMin(&sh_first, tid);
+        __syncthreads();
+        cut_key = sorted_key[sh_first];
+    }
+    // the draw, in order of id
+    const bool kept = tid < m && my_key >= cut_key;
+    const float kw = kept ? my_w : 0.f;
+    float total_kept;
+    const float before = block_exclusive_scan<float>(kw, fscan, &total_kept);
+    const float target = uniforms[row] * total_kept;
+    __syncthreads();
+    if (tid == 0) { box[0] = 0x7fffffffu; box[1] = 0; }
+    __syncthreads();
+    if (kept) {
+        if (before + kw > target) atomicMin(&box[0], (uint32_t)tid);
+        atomicMax(&box[1], (uint32_t)tid);
+    }
+    __syncthreads();
+    if (tid == 0) out[row] = fid[box[0] != 0x7fffffffu ? box[0] : box[1]];
+}
+
+static int sample_chunks(int vocab) { return (vocab + CAND_CHUNK - 1) / CAND_CHUNK; }
+
+static bool sample_by_candidates(int vocab, int top_k) {
+    const int chunks = sample_chunks(vocab);
+    return top_k > 0 && top_k <= CAND_MAX_K && top_k < vocab && chunks <= CAND_MAX_CHUNKS &&
+           (long long)chunks * top_k <= CAND_MAX_TOTAL;
+}
+
+/* Bytes of device scratch that tqk_sample wants for these sizes (0: none). */
+extern "C" size_t tqk_sample_scratch_bytes(int n_rows, int vocab, int top_k) {
+    if (n_rows <= 0 || vocab <= 0 || !sample_by_candidates(vocab, top_k)) return 0;
+    const size_t slots = (size_t)n_rows * sample_chunks(vocab);
+    return slots * top_k * 8 + slots * 4;
+}
+
 extern "C" int tqk_sample(const float* logits, int n_rows, int vocab, float temperature, int top_k, float top_p,
-                          const float* uniforms, int32_t* out, void* stream) {
+                          const float* uniforms, int32_t* out, void* scratch, void* stream) {
     TQK_REQUIRE(logits && uniforms && out, "tqk_sample: null pointer");
     TQK_REQUIRE(n_rows >= 0 && vocab > 0, "tqk_sample: bad sizes rows=%d vocab=%d", n_rows, vocab);
     TQK_REQUIRE(temperature > 0.f, "tqk_sample: temperature must be positive (use argmax for greedy), got %g", (double)temperature);
     TQK_REQUIRE(top_k >= 0, "tqk_sample: top_k must not be negative");
     TQK_REQUIRE(top_p > 0.f, "tqk_sample: top_p must be positive, got %g", (double)top_p);
+    TQK_REQUIRE(n_rows <= 65535, "tqk_sample: too many rows for the grid");
     if (n_rows == 0) return 0;
-    sample_kernel<<<n_rows, SAMP_THREADS, 0, (hipStream_t)stream>>>(logits, vocab, temperature, top_k, top_p, uniforms, out);
+    hipStream_t s = (hipStream_t)stream;
+    if (sample_by_candidates(vocab, top_k)) {
+        TQK_REQUIRE(scratch, "tqk_sample: these sizes need scratch memory (tqk_sample_scratch_bytes)");
+        const int chunks = sample_chunks(vocab), chunk = (vocab + chunks - 1) / chunks;
+        const size_t slots = (size_t)n_rows * chunks;
+        uint32_t* cand_key = (uint32_t*)scratch;
+        int32_t* cand_id = (int32_t*)(cand_key + slots * top_k);
+        int32_t* cand_n = cand_id + slots * top_k;
+        sample_candidates_kernel<<<dim3(chunks, n_rows), CAND_THREADS, 0, s>>>(logits, vocab, chunk, chunks, top_k, cand_key, cand_id, cand_n);
+        if (tqk_check_launch("tqk_sample candidates")) return -1;
+        const size_t lds = (size_t)chunks * top_k * 8;
+        sample_draw_kernel<<<n_rows, CAND_THREADS, lds, s>>>(cand_key, cand_id, cand_n, chunks, top_k, temperature, top_p, uniforms, out);
+        return tqk_check_launch("tqk_sample draw");
+    }
+    sample_kernel<<<n_rows, SAMP_THREADS, 0, s>>>(logits, vocab, temperature, top_k, top_p, uniforms, out);
     return tqk_check_launch("tqk_sample");
 }

@@ -119,20 +119,26 @@ int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int 
 int tqk_argmax_scratch_floats(int n_rows, int vocab);
 int tqk_argmax(const float* logits, int n_rows, int vocab, int32_t* out, float* scratch, void* stream);
 
-/* For every generated token of the row's request, once per occurrence:
- * l > 0 ? l / penalty : l * penalty.  hist [n_req, hist_cap], hist_len [n_req]. */
+/* In place: for every token in the history of the row's request, once per occurrence,
+ * l > 0 ? l / penalty : l * penalty.  hist, times [n_req, hist_cap], hist_len [n_req]: the
+ * history as tqk_append_history keeps it (times: for each entry how often the penalty is
+ * applied on its behalf; zeros with hist_len 0 to start with). */
 int tqk_repeat_penalty(float* logits, int n_rows, int vocab, const int32_t* row_req,
-                       const int32_t* hist, int hist_cap, const int32_t* hist_len, int n_req,
-                       float penalty, void* stream);
+                       const int32_t* hist, const int32_t* times, int hist_cap, const int32_t* hist_len,
+                       int n_req, float penalty, void* stream);
 
-/* hist[row_req[r], hist_len[..]++] = tokens[r] */
-int tqk_append_history(const int32_t* tokens, const int32_t* row_req, int32_t* hist, int hist_cap,
-                       int32_t* hist_len, int n_rows, void* stream);
+/* tokens[r] goes to the end of the history of request row_req[r] (dropped when that is full);
+ * rows of one call name different requests. */
+int tqk_append_history(const int32_t* tokens, const int32_t* row_req, int32_t* hist, int32_t* times,
+                       int hist_cap, int32_t* hist_len, int n_rows, void* stream);
 
 /* One draw per row from softmax(logits / temperature) cut to top_k (0: off) and top_p
- * (>= 1: off), by inverse CDF over the kept tokens in order of id with uniforms[r]. */
+ * (>= 1: off), by inverse CDF over the kept tokens in order of id with uniforms[r].
+ * scratch: tqk_sample_scratch_bytes(n_rows, vocab, top_k) bytes of device memory (may be
+ * null where that is 0). */
+size_t tqk_sample_scratch_bytes(int n_rows, int vocab, int top_k);
 int tqk_sample(const float* logits, int n_rows, int vocab, float temperature, int top_k, float top_p,
-               const float* uniforms, int32_t* out, void* stream);
+               const float* uniforms, int32_t* out, void* scratch, void* stream);
 
 #ifdef __cplusplus
 }

@@ -32,6 +32,7 @@ def library():
             raise KernelError("cannot load the HIP kernel library %s: %s" % (path, e))
         lib.tqk_last_error.restype = ctypes.c_char_p
         lib.tqk_abi_version.restype = ctypes.c_int
+        lib.tqk_sample_scratch_bytes.restype = ctypes.c_size_t
         _LIB = lib
     return _LIB
 
@@ -199,34 +200,39 @@ def skinny_bf16(x, w, out, swiglu=False):
     return out
 
 
-def repeat_penalty(logits, row_req, hist, hist_len, penalty):
+def repeat_penalty(logits, row_req, hist, times, hist_len, penalty):
     """In place: for every token in the history of the row's request, once per occurrence,
-    l > 0 ? l / penalty : l * penalty."""
+    l > 0 ? l / penalty : l * penalty.  hist, times, hist_len: as append_history keeps them."""
     rows, vocab = logits.shape
     n_req, cap = hist.shape
     _check(library().tqk_repeat_penalty(
         _dev(logits, "logits", torch.float32), rows, vocab, _dev(row_req, "row_req", torch.int32, (rows,)),
-        _dev(hist, "hist", torch.int32), cap, _dev(hist_len, "hist_len", torch.int32, (n_req,)), n_req,
-        ctypes.c_float(penalty), _stream()), "repeat_penalty")
+        _dev(hist, "hist", torch.int32), _dev(times, "times", torch.int32, (n_req, cap)), cap,
+        _dev(hist_len, "hist_len", torch.int32, (n_req,)), n_req, ctypes.c_float(penalty), _stream()), "repeat_penalty")
     return logits
 
 
-def append_history(tokens, row_req, hist, hist_len):
+def append_history(tokens, row_req, hist, times, hist_len):
+    """tokens[r] joins the history of request row_req[r] (hist, times int32 [requests, cap], zeros
+    and hist_len 0 at the start; different requests in one call)."""
     rows = tokens.shape[0]
     n_req, cap = hist.shape
     _check(library().tqk_append_history(
         _dev(tokens, "tokens", torch.int32, (rows,)), _dev(row_req, "row_req", torch.int32, (rows,)),
-        _dev(hist, "hist", torch.int32), cap, _dev(hist_len, "hist_len", torch.int32, (n_req,)), rows, _stream()),
-        "append_history")
+        _dev(hist, "hist", torch.int32), _dev(times, "times", torch.int32, (n_req, cap)), cap,
+        _dev(hist_len, "hist_len", torch.int32, (n_req,)), rows, _stream()), "append_history")
 
 
 def sample(logits, temperature, top_k, top_p, uniforms, out):
     """One draw per row of logits [R,V] float32 with the uniforms [R] float32; out [R] int32."""
     rows, vocab = logits.shape
-    _check(library().tqk_sample(
+    lib = library()
+    need = int(lib.tqk_sample_scratch_bytes(rows, vocab, int(top_k)))
+    scratch = torch.empty((need,), dtype=torch.uint8, device=logits.device) if need else None
+    _check(lib.tqk_sample(
         _dev(logits, "logits", torch.float32), rows, vocab, ctypes.c_float(temperature), int(top_k),
         ctypes.c_float(top_p), _dev(uniforms, "uniforms", torch.float32, (rows,)),
-        _dev(out, "out", torch.int32, (rows,)), _stream()), "sample")
+        _dev(out, "out", torch.int32, (rows,)), _opt(scratch, "scratch"), _stream()), "sample")
     return out
 
 

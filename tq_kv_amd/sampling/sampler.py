@@ -41,6 +41,7 @@ class Sampler:
         self.use_penalty = params.repeat_penalty != 1.0
         if self.use_penalty:
             self.hist = torch.zeros((n, max(1, params.max_tokens + 1)), dtype=torch.int32, device=device)
+            self.hist_times = torch.zeros_like(self.hist)
             self.hist_len = torch.zeros((n,), dtype=torch.int32, device=device)
         self.steps = [0] * n
         self.staging = HostStaging(device, depth=2 * self.READ_AHEAD)
@@ -57,7 +58,7 @@ class Sampler:
         row_req = None
         if self.use_penalty:
             row_req = self.staging.upload(np.asarray(rows, dtype=np.int32))
-            K.repeat_penalty(logits, row_req, self.hist, self.hist_len, p.repeat_penalty)
+            K.repeat_penalty(logits, row_req, self.hist, self.hist_times, self.hist_len, p.repeat_penalty)
         if p.greedy:
             K.argmax(logits, out)
         else:
@@ -66,7 +67,7 @@ class Sampler:
         for r in rows:
             self.steps[r] += 1
         if self.use_penalty:
-            K.append_history(out, row_req, self.hist, self.hist_len)
+            K.append_history(out, row_req, self.hist, self.hist_times, self.hist_len)
         host = self.landing[self.turn, :n]
         self.turn = (self.turn + 1) % self.READ_AHEAD
         host.copy_(out, non_blocking=True)
