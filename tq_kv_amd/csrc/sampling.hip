@@ -1,5 +1,7 @@
 // Choosing the next token on the device: argmax, and temperature / top-k / top-p /
-// repeat-penalty sampling by inverse CDF.  One block per row of logits.
+// repeat-penalty sampling by inverse CDF.  The rows of logits are read by many blocks each
+// (argmax; top-k up to 256: the chunks' best first, then one block per row on those few);
+// other settings of top-k take one block per row.
 //
 // The reference samples on the host from a copy of the logits
 // (src/engine.rs:353-373, 403-423): argmax if temperature <= 0, else top-k then
