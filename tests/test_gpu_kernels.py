@@ -394,6 +394,22 @@ def test_sample_top_k_over_chunks_of_the_row():
     assert draw(torch.full((1, 6000), float("nan"), device=DEV), 1.0, 10, 1.0, [0.5]) == [0]
 
 
+@pytest.mark.parametrize("vocab", [151936, 5003])
+def test_sample_top_p_alone_peaked_and_flat_rows_together(vocab):
+    # without top-k a row is first tried on its few hundred best tokens; a flat row, whose top-p set
+    # is larger than that, is left to the kernel that reads the whole row.  Both kinds in one call.
+    rows = torch.stack([rand(vocab, seed=26, scale=9.0), rand(vocab, seed=27, scale=0.5),
+                        torch.zeros(vocab, device=DEV), rand(vocab, seed=28, scale=4.0)])
+    rows[3, 100:400] = 15.0                              # 300 equal best tokens: the cut falls among ties
+    us = [0.003, 0.4, 0.77, 0.9999]
+    for top_p, temperature in ((0.9, 1.0), (0.5, 0.7), (0.999, 1.0)):
+        out = torch.empty(4, dtype=torch.int32, device=DEV)
+        for u in us:
+            K.sample(rows.clone(), temperature, 0, top_p, torch.full((4,), u, device=DEV), out)
+            want = [plain.sample_token(rows[r].cpu(), [], temperature, 0, top_p, 1.0, u) for r in range(4)]
+            assert out.tolist() == want, (top_p, temperature, u)
+
+
 def test_sample_frequencies_follow_the_softmax():
     logits = torch.tensor([[0.0, 1.0, -1.0, 2.0, 0.5]], device=DEV)
     n = 4000

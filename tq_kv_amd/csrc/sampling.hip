@@ -236,7 +236,8 @@ extern "C" int tqk_append_history(const int32_t* tokens, const int32_t* row_req,
 // ---- temperature / top-k / top-p draw ------------------------------------------------
 __global__ __launch_bounds__(SAMP_THREADS)
 void sample_kernel(const float* __restrict__ logits, int vocab, float temperature, int top_k, float top_p,
-                   const float* __restrict__ uniforms, int32_t* __restrict__ out) {
+                   const float* __restrict__ uniforms, int32_t* __restrict__ out, const int32_t* __restrict__ done) {
+    if (done && done[blockIdx.x]) return;              // the row has been drawn from its candidates
     __shared__ float fscratch[SAMP_THREADS / TQK_WAVE];
     __shared__ int iscratch[SAMP_THREADS / TQK_WAVE];
     __shared__ int hist[256];
@@ -467,19 +468,43 @@ __device__ int take_largest(const uint32_t* keys, const int32_t* ids, int first_
     return total;
 }
 
+// largest of one unsigned value per thread; scratch: two words in LDS
+__device__ __forceinline__ uint32_t block_max_u(uint32_t v, uint32_t* scratch) {
+    __syncthreads();
+    if (threadIdx.x == 0) scratch[0] = 0;
+    __syncthreads();
+    atomicMax(&scratch[0], v);
+    __syncthreads();
+    const uint32_t m = scratch[0];
+    __syncthreads();
+    return m;
+}
+
 __global__ __launch_bounds__(CAND_THREADS)
 void sample_candidates_kernel(const float* __restrict__ logits, int vocab, int chunk, int n_chunks, int top_k,
-                              uint32_t* __restrict__ cand_key, int32_t* __restrict__ cand_id, int32_t* __restrict__ cand_n) {
+                              uint32_t* __restrict__ cand_key, int32_t* __restrict__ cand_id, int32_t* __restrict__ cand_n,
+                              float inv_t, float2* __restrict__ chunk_mass) {
     __shared__ uint32_t keys[CAND_CHUNK];
     __shared__ int hist[256];
     __shared__ uint32_t box[2];
     __shared__ int scan[CAND_THREADS / TQK_WAVE];
+    __shared__ float fscan[CAND_THREADS / TQK_WAVE];
     const int row = blockIdx.y, blk = blockIdx.x;
     const int first = blk * chunk, n = max(0, min(vocab - first, chunk));
     const float* src = logits + (size_t)row * vocab + first;
-    for (int i = threadIdx.x; i < n; i += CAND_THREADS) keys[i] = select_key(src[i]);
+    uint32_t kmax = 0;
+    for (int i = threadIdx.x; i < n; i += CAND_THREADS) { const uint32_t key = select_key(src[i]); keys[i] = key; kmax = max(kmax, key); }
     __syncthreads();
     const size_t slot = (size_t)row * n_chunks + blk;
+    if (chunk_mass) {
+        // the chunk's largest logit and the weight of all its tokens relative to it
+        // (the order of float_key is that of the values, so the largest key is the largest logit)
+        const float cmax = key_value(block_max_u(kmax, box));
+        float w = 0.f;
+        for (int i = threadIdx.x; i < n; i += CAND_THREADS) { const uint32_t key = keys[i]; if (key) w += expf((key_value(key) - cmax) * inv_t); }
+        w = block_sum_any<float>(w, fscan);
+        if (threadIdx.x == 0) chunk_mass[slot] = make_float2(cmax, w);
+    }
     const int taken = take_largest(keys, nullptr, first, n, top_k, hist, box, scan,
                                    cand_key + slot * top_k, cand_id + slot * top_k);
     if (threadIdx.x == 0) cand_n[slot] = taken;
@@ -488,7 +513,11 @@ void sample_candidates_kernel(const float* __restrict__ logits, int vocab, int c
 __global__ __launch_bounds__(CAND_THREADS)
 void sample_draw_kernel(const uint32_t* __restrict__ cand_key, const int32_t* __restrict__ cand_id,
                         const int32_t* __restrict__ cand_n, int n_chunks, int top_k, float temperature, float top_p,
-                        const float* __restrict__ uniforms, int32_t* __restrict__ out) {
+                        const float* __restrict__ uniforms, int32_t* __restrict__ out,
+                        const float2* __restrict__ chunk_mass, int32_t* __restrict__ done) {
+    // With chunk_mass (no top-k asked for: top_k is only the number of candidates) top-p is cut
+    // against the weight of the whole row; the row is drawn here if the cut lies inside the
+    // candidates for certain, else it is left (done[row] = 0) to the kernel that reads the whole row.
     extern __shared__ uint32_t pool[];                 // keys [n_chunks * top_k], then ids
     __shared__ int hist[256];
     __shared__ uint32_t box[2];
@@ -515,7 +544,7 @@ void sample_draw_kernel(const uint32_t* __restrict__ cand_key, const int32_t* __
     const int m = take_largest(keys, ids, 0, n, top_k, hist, box, scan, fkey, fid);
     __syncthreads();
     if (m == 0) {                                      // a row of NaN
-        if (tid == 0) out[row] = 0;
+        if (tid == 0) { out[row] = 0; if (done) done[row] = 1; }
         return;
     }
     // rank from the largest down, lower ids first among equals (the list is in order of id)
@@ -538,11 +567,24 @@ void sample_draw_kernel(const uint32_t* __restrict__ cand_key, const int32_t* __
         const float w = tid < m ? sorted_w[tid] : 0.f;
         float total;
         const float before = block_exclusive_scan<float>(w, fscan, &total);
-        if (tid == 0) sh_first = m - 1;
+        if (chunk_mass) {
+            // the whole row's weight: the chunks' weights, each moved to the row's largest logit, in order
+            float cw = 0.f;
+            if (tid < n_chunks) { const float2 cm = chunk_mass[(size_t)row * n_chunks + tid]; cw = cm.y > 0.f ? cm.y * expf((cm.x - zmax) * inv_t) : 0.f; }
+            total = block_sum_any<float>(cw, fscan);
+        }
+        __syncthreads();
+        if (tid == 0) sh_first = chunk_mass ? 0x7fffffff : m - 1;
         __syncthreads();
         if (tid < m && before + w >= top_p * total) atomicMin(&sh_first, tid);
         __syncthreads();
-        cut_key = sorted_key[sh_first];
+        const int first = sh_first;
+        // for certain inside: reached at all, and above the smallest candidate unless these are all tokens
+        if (chunk_mass && (first == 0x7fffffff || (n >= top_k && !(sorted_key[first] > sorted_key[m - 1])))) {
+            if (tid == 0) done[row] = 0;
+            return;
+        }
+        cut_key = sorted_key[first];
     }
     // the draw, in order of id
     const bool kept = tid < m && my_key >= cut_key;
@@ -558,22 +600,33 @@ void sample_draw_kernel(const uint32_t* __restrict__ cand_key, const int32_t* __
         atomicMax(&box[1], (uint32_t)tid);
     }
     __syncthreads();
-    if (tid == 0) out[row] = fid[box[0] != 0x7fffffffu ? box[0] : box[1]];
+    if (tid == 0) { out[row] = fid[box[0] != 0x7fffffffu ? box[0] : box[1]]; if (done) done[row] = 1; }
 }
 
 static int sample_chunks(int vocab) { return (vocab + CAND_CHUNK - 1) / CAND_CHUNK; }
 
+// top_k asked for and small: its candidates decide the row
 static bool sample_by_candidates(int vocab, int top_k) {
     const int chunks = sample_chunks(vocab);
     return top_k > 0 && top_k <= CAND_MAX_K && top_k < vocab && chunks <= CAND_MAX_CHUNKS &&
            (long long)chunks * top_k <= CAND_MAX_TOTAL;
 }
 
+// no top-k but top-p: how many candidates a chunk gives for a try (0: no try)
+static int sample_open_candidates(int vocab, int top_k, float top_p) {
+    const int chunks = sample_chunks(vocab);
+    if ((top_k > 0 && top_k < vocab) || !(top_p < 1.f) || chunks > CAND_MAX_CHUNKS || chunks > CAND_THREADS) return 0;
+    const int k = CAND_MAX_TOTAL / chunks < CAND_MAX_K ? CAND_MAX_TOTAL / chunks : CAND_MAX_K;
+    return k >= 16 ? k : 0;
+}
+
 /* Bytes of device scratch that tqk_sample wants for these sizes (0: none). */
-extern "C" size_t tqk_sample_scratch_bytes(int n_rows, int vocab, int top_k) {
-    if (n_rows <= 0 || vocab <= 0 || !sample_by_candidates(vocab, top_k)) return 0;
+extern "C" size_t tqk_sample_scratch_bytes(int n_rows, int vocab, int top_k, float top_p) {
+    if (n_rows <= 0 || vocab <= 0) return 0;
+    const int k = sample_by_candidates(vocab, top_k) ? top_k : sample_open_candidates(vocab, top_k, top_p);
+    if (k == 0) return 0;
     const size_t slots = (size_t)n_rows * sample_chunks(vocab);
-    return slots * top_k * 8 + slots * 4;
+    return slots * k * 8 + slots * 4 + slots * 8 + (size_t)n_rows * 4;
 }
 
 extern "C" int tqk_sample(const float* logits, int n_rows, int vocab, float temperature, int top_k, float top_p,
@@ -586,19 +639,28 @@ extern "C" int tqk_sample(const float* logits, int n_rows, int vocab, float temp
     TQK_REQUIRE(n_rows <= 65535, "tqk_sample: too many rows for the grid");
     if (n_rows == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    if (sample_by_candidates(vocab, top_k)) {
+    const bool closed = sample_by_candidates(vocab, top_k);
+    const int k = closed ? top_k : sample_open_candidates(vocab, top_k, top_p);
+    int32_t* done = nullptr;
+    if (k > 0) {
         TQK_REQUIRE(scratch, "tqk_sample: these sizes need scratch memory (tqk_sample_scratch_bytes)");
         const int chunks = sample_chunks(vocab), chunk = (vocab + chunks - 1) / chunks;
         const size_t slots = (size_t)n_rows * chunks;
-        uint32_t* cand_key = (uint32_t*)scratch;
-        int32_t* cand_id = (int32_t*)(cand_key + slots * top_k);
-        int32_t* cand_n = cand_id + slots * top_k;
-        sample_candidates_kernel<<<dim3(chunks, n_rows), CAND_THREADS, 0, s>>>(logits, vocab, chunk, chunks, top_k, cand_key, cand_id, cand_n);
+        float2* chunk_mass = (float2*)scratch;                        // 8-byte values first
+        uint32_t* cand_key = (uint32_t*)(chunk_mass + slots);
+        int32_t* cand_id = (int32_t*)(cand_key + slots * k);
+        int32_t* cand_n = cand_id + slots * k;
+        done = cand_n + slots;
+        sample_candidates_kernel<<<dim3(chunks, n_rows), CAND_THREADS, 0, s>>>(logits, vocab, chunk, chunks, k, cand_key, cand_id, cand_n,
+                                                                             1.f / temperature, closed ? nullptr : chunk_mass);
         if (tqk_check_launch("tqk_sample candidates")) return -1;
-        const size_t lds = (size_t)chunks * top_k * 8;
-        sample_draw_kernel<<<n_rows, CAND_THREADS, lds, s>>>(cand_key, cand_id, cand_n, chunks, top_k, temperature, top_p, uniforms, out);
-        return tqk_check_launch("tqk_sample draw");
+        const size_t lds = (size_t)chunks * k * 8;
+        sample_draw_kernel<<<n_rows, CAND_THREADS, lds, s>>>(cand_key, cand_id, cand_n, chunks, k, temperature, top_p, uniforms, out,
+                                                             closed ? nullptr : chunk_mass, closed ? nullptr : done);
+        if (tqk_check_launch("tqk_sample draw")) return -1;
+        if (closed) return 0;
     }
-    sample_kernel<<<n_rows, SAMP_THREADS, 0, s>>>(logits, vocab, temperature, top_k, top_p, uniforms, out);
+    // the whole row by one block: every setting; after a try with candidates only the rows that the try left
+    sample_kernel<<<n_rows, SAMP_THREADS, 0, s>>>(logits, vocab, temperature, top_k, top_p, uniforms, out, done);
     return tqk_check_launch("tqk_sample");
 }

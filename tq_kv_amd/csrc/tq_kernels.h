@@ -134,9 +134,9 @@ int tqk_append_history(const int32_t* tokens, const int32_t* row_req, int32_t* h
 
 /* One draw per row from softmax(logits / temperature) cut to top_k (0: off) and top_p
  * (>= 1: off), by inverse CDF over the kept tokens in order of id with uniforms[r].
- * scratch: tqk_sample_scratch_bytes(n_rows, vocab, top_k) bytes of device memory (may be
- * null where that is 0). */
-size_t tqk_sample_scratch_bytes(int n_rows, int vocab, int top_k);
+ * scratch: tqk_sample_scratch_bytes(n_rows, vocab, top_k, top_p) bytes of device memory, 8-byte
+ * aligned (may be null where that is 0). */
+size_t tqk_sample_scratch_bytes(int n_rows, int vocab, int top_k, float top_p);
 int tqk_sample(const float* logits, int n_rows, int vocab, float temperature, int top_k, float top_p,
                const float* uniforms, int32_t* out, void* scratch, void* stream);
 

@@ -227,7 +227,7 @@ def sample(logits, temperature, top_k, top_p, uniforms, out):
     """One draw per row of logits [R,V] float32 with the uniforms [R] float32; out [R] int32."""
     rows, vocab = logits.shape
     lib = library()
-    need = int(lib.tqk_sample_scratch_bytes(rows, vocab, int(top_k)))
+    need = int(lib.tqk_sample_scratch_bytes(rows, vocab, int(top_k), ctypes.c_float(top_p)))
     scratch = torch.empty((need,), dtype=torch.uint8, device=logits.device) if need else None
     _check(lib.tqk_sample(
         _dev(logits, "logits", torch.float32), rows, vocab, ctypes.c_float(temperature), int(top_k),
