@@ -26,6 +26,9 @@ def main():
     ap.add_argument("--shape", default=SHAPE)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--no-tune", action="store_true", help="do not let the library pick its fastest kernel per product shape")
+    ap.add_argument("--mixed", action="store_true",
+                    help="another workload instead: --batch prompts of unequal lengths (uniform in 16..--prompt-len), sampled with "
+                         "the default parameters (temperature 0.7, top-k 40, top-p 0.9, repeat penalty 1.1); prints its own line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -58,6 +61,9 @@ def main():
 
     def prompts(n):
         return torch.randint(0, V, (n, args.prompt_len), generator=gen).tolist()
+
+    if args.mixed:
+        return mixed_workload(args, model, engine, raw, note)
 
     # -- prefill of one prompt --------------------------------------------------------------
     if not args.no_tune:
@@ -134,6 +140,38 @@ def main():
         "points": points,
     }
     print(json.dumps(line))
+    return 0
+
+
+def mixed_workload(args, model, engine, raw, note):
+    """Prompts of unequal lengths in one batch, sampled: tokens per second of the decoding steps."""
+    import torch
+
+    from tq_kv_amd import GenerationParams, generate
+    gen = torch.Generator().manual_seed(1)
+    lens = torch.randint(16, args.prompt_len + 1, (args.batch,), generator=gen).tolist()
+    prompts = [torch.randint(0, raw["vocab_size"], (n,), generator=gen).tolist() for n in lens]
+    if not args.no_tune:
+        model.tune_library(min(args.batch, 64))
+    marks, calls = {}, [0]
+
+    def on_tokens(pairs):
+        if calls[0] in (args.warmup, args.warmup + args.steps):
+            torch.cuda.synchronize()
+            marks[calls[0]] = time.perf_counter()
+        calls[0] += 1
+    note("%d prompts of %d..%d tokens, %d sampled steps" % (args.batch, min(lens), max(lens), args.steps))
+    params = GenerationParams(max_tokens=args.warmup + args.steps + 2)
+    t0 = time.perf_counter()
+    out = generate(engine, prompts, params, on_tokens=on_tokens, max_batch=args.batch)
+    torch.cuda.synchronize()
+    total = time.perf_counter() - t0
+    seconds = marks[args.warmup + args.steps] - marks[args.warmup]
+    print(json.dumps({"metric": "decode tok/s, %d prompts of unequal lengths, %s shape, sampled" % (args.batch, args.shape),
+                      "value": round(args.batch * args.steps / seconds, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+                      "warmup": args.warmup, "ms_per_step": round(seconds / args.steps * 1e3, 4), "dtype": "bf16",
+                      "data": "synthetic", "prompt_tokens": sum(lens), "generated_tokens": sum(len(o) for o in out),
+                      "end_to_end_tok_per_s": round(sum(len(o) for o in out) / total, 1)}))
     return 0
 
 
