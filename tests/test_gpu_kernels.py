@@ -401,7 +401,8 @@ def test_sample_top_p_alone_peaked_and_flat_rows_together(vocab):
     rows = torch.stack([rand(vocab, seed=26, scale=9.0), rand(vocab, seed=27, scale=0.5),
                         torch.zeros(vocab, device=DEV), rand(vocab, seed=28, scale=4.0)])
     rows[3, 100:400] = 15.0                              # 300 equal best tokens: the cut falls among ties
-    us = [0.003, 0.4, 0.77, 0.9999]
+    # (the plain rule sorts the row in Python: at the full vocabulary only a few draws)
+    us = [0.003, 0.4, 0.77, 0.9999] if vocab < 10000 else [0.4]
     for top_p, temperature in ((0.9, 1.0), (0.5, 0.7), (0.999, 1.0)):
         out = torch.empty(4, dtype=torch.int32, device=DEV)
         for u in us:
