@@ -117,7 +117,6 @@ class Model:
         """Let the library try its kernels once for every product of the model at `rows`
         rows (more than 16: fewer never reach the library) and keep the fastest for later
         calls.  Takes seconds per distinct weight shape."""
-        from ..parts import linear as L
         if self.dtype != torch.bfloat16 or rows <= L.POLICY["skinny_max_rows"]:
             return
         L.tune_library(True)
@@ -144,8 +143,8 @@ class Model:
         # small decoding steps: products fold the norms and the residual sums around them in
         ctx.fuse_small = (L.POLICY["fused"] and self.dtype == torch.bfloat16 and ctx.all_decode
                           and ctx.n_tokens <= 16 and s.hidden_size % 32 == 0)
-        firsts = [self.blocks[run.layer].first_norm() if hasattr(self.blocks[run.layer], "first_norm") else None
-                  for run in s.order] + [self.final_norm]
+        # the norm that reads the stream first in every run, and after the last one
+        firsts = [self.blocks[run.layer].first_norm() for run in s.order] + [self.final_norm]
         if ctx.fuse_small:
             xw = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.bfloat16, device=self.device)
             ss = torch.empty(((s.hidden_size + 15) // 16, 16), dtype=torch.float32, device=self.device)      # the most pieces a product gives
@@ -157,11 +156,7 @@ class Model:
             stream = L.Stream(h)
             K.embed(self.embedding, ctx.dev.tokens, h)
         for i, run in enumerate(s.order):
-            block = self.blocks[run.layer]
-            if hasattr(block, "first_norm"):
-                block.forward(stream, ctx, cache.entry(i), next_norm=firsts[i + 1])
-            else:
-                block.forward(stream, ctx, cache.entry(i))
+            self.blocks[run.layer].forward(stream, ctx, cache.entry(i), next_norm=firsts[i + 1])
         n_rows = ctx.dev.want_rows.shape[0]
         if n_rows == 0:
             return torch.empty((0, s.vocab_size), dtype=torch.float32, device=self.device)
