@@ -69,3 +69,26 @@ def test_float32_path_equals_plain_at_7b_sizes():
     cfg = dict(raw)
     want = plain.forward({k: v.float().cpu() for k, v in tensors.items()}, cfg, prompt)[[0] + list(range(32, 40))]
     torch.testing.assert_close(got, want, atol=2e-5 * max(1.0, want.abs().max().item()), rtol=2e-5)
+
+
+def test_generation_through_graphs_and_running_ahead_equals_plain_stepping_at_7b_sizes():
+    # the generation loop (captured graphs, next step started from the device's tokens before the
+    # draw is read) against steps given one by one with the host's tokens and no graphs: the same
+    # kernels either way, so the same tokens; sampled with the default parameters
+    from tq_kv_amd import GenerationParams, generate
+    from tq_kv_amd.sampling.sampler import Sampler
+    raw = two_layer("qwen2.5:7b")
+    model = build(raw, "bfloat16", tensors_for(raw, 5))
+    prompts = [helpers.random_tokens(n, raw["vocab_size"], 70 + i) for i, n in enumerate([90, 17, 40])]
+    params = GenerationParams(max_tokens=20, seed=3)
+    fast = generate(Engine(model, max_tokens=1024), prompts, params)
+    eng = Engine(model, max_tokens=1024, use_graphs=False)
+    sampler = Sampler(params, [0, 1, 2], model.device)
+    slots = [eng.open() for _ in prompts]
+    toks = sampler.sample(eng.step([(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)]), [0, 1, 2])
+    slow = [[t] for t in toks]
+    for _ in range(19):
+        toks = sampler.sample(eng.step([(s, [t], [0]) for s, t in zip(slots, toks)]), [0, 1, 2])
+        for o, t in zip(slow, toks):
+            o.append(t)
+    assert fast == slow
