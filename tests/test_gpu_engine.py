@@ -139,6 +139,36 @@ def test_wanted_places_and_their_order():
     eng.close(sa), eng.close(sb)
 
 
+@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("B", "bfloat16"), ("C", "float32"), ("C", "bfloat16")])
+def test_few_wanted_places_in_any_order_equal_all_places(name, dtype):
+    # where a step wants fewer places than it has tokens, the last layer computes only those
+    # (its keys and values still go to the cache for all tokens): wanted places out of order, twice,
+    # in neighbouring runs, at a window's edge, in several sequences, and none at all; then
+    # decoding goes on from the cache that such steps left
+    eng = G.engine(name, dtype, True)
+    ps = G.prompts(name, [90, 70, 9, 33], seed=1200)
+    wants = [[89, 0, 1, 2, 77, 77, 64, 63], [], [8], [5, 4, 3]]
+    slots = [eng.open() for _ in ps]
+    full = eng.step([(s, p, all_places(p)) for s, p in zip(slots, ps)])
+    for s in slots:
+        eng.close(s)
+    slots = [eng.open() for _ in ps]
+    few = eng.step([(s, p, w) for s, p, w in zip(slots, ps, wants)])
+    offsets = [0, 90, 160, 169]
+    rows = [o + j for o, w in zip(offsets, wants) for j in w]
+    assert few.shape[0] == len(rows)
+    if dtype == "float32":
+        assert torch.equal(few, full[rows])
+    else:
+        G.close(few, full[rows].cpu(), dtype)
+    nxt = eng.step([(s, [7], [0]) for s in slots])
+    for i, p in enumerate(ps):
+        G.close(nxt[i:i + 1], G.plain_logits(name, p + [7], True)[-1:], dtype)
+    for s in slots:
+        eng.close(s)
+    eng.cache.check()
+
+
 def test_float32_results_do_not_depend_on_the_cut_at_all():
     # in float32 every kernel sums in an order that depends on the position only
     eng = G.engine("C", "float32", True)

@@ -81,6 +81,13 @@ class StepContext:
                     raise IndexError("wanted place %d is outside the %d tokens of sequence %d" % (j, lens[i], i))
                 rows.append(int(host.cu[i]) + int(j))
         host.want_rows = np.asarray(rows, dtype=np.int32)
+        # The rows that the last run of the order has to compute: the wanted ones, each once, in
+        # order.  Where these are fewer than the step's tokens (a prompt of which the last place is
+        # wanted, a piece of a prompt of which nothing is), the last run computes its queries,
+        # its output product and its feed-forward for them alone.
+        host.last_rows = np.unique(host.want_rows).astype(np.int32)
+        host.want_in_last = np.searchsorted(host.last_rows, host.want_rows).astype(np.int32)
+        self.n_last = int(host.last_rows.shape[0])
         # tiles of consecutive queries of one sequence, for the prompt attention kernel
         self.tile_queries = tile = tile_queries(self.n_tokens)
         t_seq, t_tok0, t_count = [], [], []
@@ -94,8 +101,25 @@ class StepContext:
         host.tile_seq = np.asarray([t_seq[k] for k in order], dtype=np.int32)
         host.tile_tok0 = np.asarray([t_tok0[k] for k in order], dtype=np.int32)
         host.tile_count = np.asarray([t_count[k] for k in order], dtype=np.int32)
+        # the same for the last run's rows, in their own numbering: runs of neighbouring rows of a sequence
+        host.last_seq = host.tok_seq[host.last_rows] if self.n_last else np.zeros(0, dtype=np.int32)
+        host.last_pos = host.tok_pos[host.last_rows] if self.n_last else np.zeros(0, dtype=np.int32)
+        l_seq, l_tok0, l_count = [], [], []
+        k = 0
+        while k < self.n_last:
+            j = k + 1
+            while (j < self.n_last and j - k < tile and host.last_rows[j] == host.last_rows[j - 1] + 1
+                   and host.last_seq[j] == host.last_seq[k]):
+                j += 1
+            l_seq.append(int(host.last_seq[k])), l_tok0.append(k), l_count.append(j - k)
+            k = j
+        order = sorted(range(len(l_seq)), key=lambda t: -(int(host.last_pos[l_tok0[t]]) + l_count[t]))
+        host.last_tile_seq = np.asarray([l_seq[t] for t in order], dtype=np.int32)
+        host.last_tile_tok0 = np.asarray([l_tok0[t] for t in order], dtype=np.int32)
+        host.last_tile_count = np.asarray([l_count[t] for t in order], dtype=np.int32)
         self.host = host
         self.all_decode = all(n == 1 for n in lens)
+        self.prune_last = not self.all_decode and self.n_last < self.n_tokens
         self.fuse_small = False      # set by the model for small decoding steps in bfloat16
         self.max_new = max(lens)
         self.max_end = int((host.seq_start + host.seq_new).max())
@@ -111,7 +135,8 @@ class StepContext:
                 self.host_tables[i] = wide
 
         names = ["tokens", "tok_seq", "tok_pos", "seq_slot", "seq_start", "seq_new", "cu", "want_rows",
-                 "tile_seq", "tile_tok0", "tile_count"]
+                 "tile_seq", "tile_tok0", "tile_count", "last_rows", "want_in_last", "last_seq", "last_pos",
+                 "last_tile_seq", "last_tile_tok0", "last_tile_count"]
         parts = [getattr(host, n) for n in names] + [t.reshape(-1) for t in self.host_tables]
         offsets, total = [], 0
         for p in parts:

@@ -156,15 +156,18 @@ class Model:
             stream = L.Stream(h)
             K.embed(self.embedding, ctx.dev.tokens, h)
         for i, run in enumerate(s.order):
-            self.blocks[run.layer].forward(stream, ctx, cache.entry(i), next_norm=firsts[i + 1])
+            stream = self.blocks[run.layer].forward(stream, ctx, cache.entry(i), next_norm=firsts[i + 1],
+                                                    last=i + 1 == len(s.order)) or stream
         n_rows = ctx.dev.want_rows.shape[0]
         if n_rows == 0:
             return torch.empty((0, s.vocab_size), dtype=torch.float32, device=self.device)
+        # the last block may have gone on with the wanted rows alone, numbered among themselves
+        want_rows = ctx.dev.want_in_last if getattr(stream, "of_last_rows", False) else ctx.dev.want_rows
         lazy = self.final_norm.lazy(stream) if ctx.fuse_small and hasattr(self.final_norm, "lazy") else None
         if lazy is not None and n_rows <= 16 and L.fusable(n_rows, self.head):
             logits = torch.empty((n_rows, s.vocab_size), dtype=torch.float32, device=self.device)
-            return K.fused_store(lazy.xw, self.head, logits, lazy.norm, rows=ctx.dev.want_rows)
-        x = self.final_norm.gather_add_norm(stream.h, stream.pending, ctx.dev.want_rows)
+            return K.fused_store(lazy.xw, self.head, logits, lazy.norm, rows=want_rows)
+        x = self.final_norm.gather_add_norm(stream.h, stream.pending, want_rows)
         return linear(x, self.head, out_dtype=torch.float32)
 
     def __repr__(self):

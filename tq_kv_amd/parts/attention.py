@@ -46,6 +46,7 @@ class Attention(Part):
         self.graph_safe = not hasattr(self.position, "apply") or getattr(self.position, "graph_safe", False)
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
         self.reads_other_cache = False      # set when a run of this layer reads another run's cache
+        self.takes_rows = True              # forward(..., last_rows=True) computes the step's last_rows only
 
     def tensors(self):
         q, kv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
@@ -92,7 +93,10 @@ class Attention(Part):
     def adds_to_stream(self, ctx):
         return fusable(ctx.n_tokens, self.w_o, adds=True) and self.b_o is None
 
-    def forward(self, x, ctx, entry, stream=None):
+    def forward(self, x, ctx, entry, stream=None, last_rows=False):
+        """x: the (normed) step [tokens, hidden], or a LazyNorm of it.  stream: add the output to
+        it instead of returning it.  last_rows: keys and values of all tokens go to the cache as
+        always, but the output is computed for ctx's last_rows alone, [n_last, hidden]."""
         lazy = isinstance(x, LazyNorm)
         n = x.xw.shape[0] if lazy else x.shape[0]
         dtype = torch.bfloat16 if lazy else x.dtype
@@ -107,6 +111,13 @@ class Attention(Part):
                         norm=x.norm if lazy else None)
         else:
             self._qkv(x, ctx, entry, table, q)
+        if last_rows:
+            d = ctx.dev
+            if ctx.n_last == 0:
+                return torch.empty((0, self.hidden), dtype=dtype, device=q.device)
+            y = torch.empty((ctx.n_last, self.n_heads * self.head_dim), dtype=dtype, device=q.device)
+            attend_rows(q.index_select(0, d.last_rows), entry, table, ctx, self.window, self.scale, y)
+            return linear(y, self.w_o, self.b_o)
         y = torch.empty((n, self.n_heads * self.head_dim), dtype=dtype, device=q.device)
         attend(q, entry, table, ctx, self.window, self.scale, y)
         if stream is not None:
@@ -153,3 +164,23 @@ def attend(q, entry, table, ctx, window, scale, out):
         return K.attention_prefill(q, entry.keys, entry.values, d.tok_pos, table, d.tile_seq, d.tile_tok0, d.tile_count,
                                    d.seq_start, d.seq_new, window, scale, out, tile_queries=ctx.tile_queries)
     return K.attention(q, entry.keys, entry.values, ctx.dev.tok_seq, ctx.dev.tok_pos, table, window, scale, out)
+
+
+DECODE_KERNEL_ROWS = 32     # up to so many rows of a prompt step go through the decoding kernel
+
+
+def attend_rows(q, entry, table, ctx, window, scale, out):
+    """The same for the step's last_rows alone (q holds their queries): the cache already holds
+    the keys and values of all the step's tokens."""
+    head_dim = q.shape[2]
+    d = ctx.dev
+    if (q.dtype == torch.bfloat16 and POLICY["decode_mfma"] and K.attention_decode_supported(head_dim)
+            and ctx.n_last <= DECODE_KERNEL_ROWS):
+        # few rows: the decoding kernel shares a row's keys out over many blocks, where the prompt
+        # kernel would walk them in one; a row is a sequence of its own to it
+        return K.attention_decode(q, entry.keys, entry.values, d.last_pos, table.index_select(0, d.last_seq), window, scale, out)
+    if q.dtype == torch.bfloat16 and POLICY["prefill_mfma"] and K.attention_prefill_supported(head_dim):
+        return K.attention_prefill(q, entry.keys, entry.values, d.last_pos, table, d.last_tile_seq, d.last_tile_tok0,
+                                   d.last_tile_count, d.seq_start, d.seq_new, window, scale, out,
+                                   tile_queries=ctx.tile_queries)
+    return K.attention(q, entry.keys, entry.values, d.last_seq, d.last_pos, table, window, scale, out)

@@ -11,6 +11,7 @@ framework's parts go further: a product that consumes a norm computes it itself
 that the norm kernels disappear; parts that do not offer this (`folds_norm`,
 `adds_to_stream`) are simply given tensors.
 """
+from .linear import POLICY
 from .registry import Part, register
 
 
@@ -90,9 +91,28 @@ class PreNormBlock(Part):
             stream.pending = out
             stream.invalidate()
 
-    def forward(self, stream, ctx, entry, next_norm=None):
-        """next_norm: the norm that reads the stream after this block."""
+    def forward(self, stream, ctx, entry, next_norm=None, last=False):
+        """next_norm: the norm that reads the stream after this block.  last: nothing but the
+        head reads the stream after this block, so where the step wants fewer rows than it has
+        tokens (ctx.prune_last) and the mixer can do so, only those rows are computed once the
+        mixer has seen all tokens: the stream of those rows is returned in place of `stream`."""
+        if last and ctx.prune_last and POLICY["prune_last"] and getattr(self.mixer, "takes_rows", False):
+            return self._forward_last_rows(stream, ctx, entry)
         x = self._normed(self.mixer_norm, stream, self.mixer, ctx)
         self._run(self.mixer, self.post_mixer_norm, self.ff_norm, x, stream, ctx, entry)
         x = self._normed(self.ff_norm, stream, self.feed_forward, ctx)
         self._run(self.feed_forward, self.post_ff_norm, next_norm, x, stream, ctx)
+        return stream
+
+    def _forward_last_rows(self, stream, ctx, entry):
+        x = self.mixer_norm.add_norm(stream.h, stream.pending)
+        y = self.mixer.forward(x, ctx, entry, last_rows=True)          # keys and values of all tokens, output of the rows
+        sub = type(stream)(stream.h.index_select(0, ctx.dev.last_rows))
+        sub.of_last_rows = True
+        if ctx.n_last == 0:
+            return sub
+        sub.pending = self.post_mixer_norm.forward(y) if self.post_mixer_norm is not None else y
+        x = self.ff_norm.add_norm(sub.h, sub.pending)
+        out = self.feed_forward.forward(x, ctx)
+        sub.pending = self.post_ff_norm.forward(out) if self.post_ff_norm is not None else out
+        return sub

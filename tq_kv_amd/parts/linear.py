@@ -19,7 +19,7 @@ from .. import kernels as K
 # plain kernel); nothing else reads these.
 # Measured on MI355X at the Qwen2.5-7B sizes: up to 16 rows the skinny kernel is ahead of the
 # library on every product; at 64 rows the library is ahead on every one.
-POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16, "fused": True}
+POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16, "fused": True, "prune_last": True}
 
 
 class Stream:

@@ -19,6 +19,10 @@ Categories and what each must offer beyond `tensors()` and `load()`:
                 not yet added to it, and next_norm is the norm that reads the stream after
                 this block; first_norm() -> the norm this block reads the stream with
 
+Optional, for a step that wants fewer rows than it has tokens: a mixer with `takes_rows` accepts
+`last_rows=True` in the last run of the order and returns its output for ctx's last_rows alone
+(its cache still takes all tokens); the block then goes on with those rows only.
+
 Optional, for small decoding steps (ctx.fuse_small), and never needed for a part to work:
 a norm with `foldable` and `lazy(stream)` lets the product after it do the division; a
 mixer or feed-forward with `folds_norm(ctx)` accepts a parts.linear.LazyNorm as x, and
