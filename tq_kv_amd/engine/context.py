@@ -101,25 +101,27 @@ class StepContext:
         host.tile_seq = np.asarray([t_seq[k] for k in order], dtype=np.int32)
         host.tile_tok0 = np.asarray([t_tok0[k] for k in order], dtype=np.int32)
         host.tile_count = np.asarray([t_count[k] for k in order], dtype=np.int32)
+        self.all_decode = all(n == 1 for n in lens)
+        self.prune_last = not self.all_decode and self.n_last < self.n_tokens
         # the same for the last run's rows, in their own numbering: runs of neighbouring rows of a sequence
-        host.last_seq = host.tok_seq[host.last_rows] if self.n_last else np.zeros(0, dtype=np.int32)
-        host.last_pos = host.tok_pos[host.last_rows] if self.n_last else np.zeros(0, dtype=np.int32)
         l_seq, l_tok0, l_count = [], [], []
-        k = 0
-        while k < self.n_last:
-            j = k + 1
-            while (j < self.n_last and j - k < tile and host.last_rows[j] == host.last_rows[j - 1] + 1
-                   and host.last_seq[j] == host.last_seq[k]):
-                j += 1
-            l_seq.append(int(host.last_seq[k])), l_tok0.append(k), l_count.append(j - k)
-            k = j
+        if self.prune_last:
+            host.last_seq, host.last_pos = host.tok_seq[host.last_rows], host.tok_pos[host.last_rows]
+            k = 0
+            while k < self.n_last:
+                j = k + 1
+                while (j < self.n_last and j - k < tile and host.last_rows[j] == host.last_rows[j - 1] + 1
+                       and host.last_seq[j] == host.last_seq[k]):
+                    j += 1
+                l_seq.append(int(host.last_seq[k])), l_tok0.append(k), l_count.append(j - k)
+                k = j
+        else:
+            host.last_rows = host.want_in_last = host.last_seq = host.last_pos = np.zeros(0, dtype=np.int32)
         order = sorted(range(len(l_seq)), key=lambda t: -(int(host.last_pos[l_tok0[t]]) + l_count[t]))
         host.last_tile_seq = np.asarray([l_seq[t] for t in order], dtype=np.int32)
         host.last_tile_tok0 = np.asarray([l_tok0[t] for t in order], dtype=np.int32)
         host.last_tile_count = np.asarray([l_count[t] for t in order], dtype=np.int32)
         self.host = host
-        self.all_decode = all(n == 1 for n in lens)
-        self.prune_last = not self.all_decode and self.n_last < self.n_tokens
         self.fuse_small = False      # set by the model for small decoding steps in bfloat16
         self.max_new = max(lens)
         self.max_end = int((host.seq_start + host.seq_new).max())
