@@ -257,6 +257,8 @@ def test_greedy_generation_float32_equals_plain(name):
     out = generate(eng, ps, GenerationParams(max_tokens=n_new, temperature=0.0, repeat_penalty=1.0))
     for p, o in zip(ps, out):
         assert o == plain.generate_greedy(w, cfg, p, n_new)
+    # prompts fed in pieces of at most 7 tokens (pieces of which nothing is wanted among them)
+    assert generate(eng, ps, GenerationParams(max_tokens=n_new, temperature=0.0, repeat_penalty=1.0), max_step_tokens=7) == out
     # stop tokens: ending one request early leaves the others as they were
     stop = out[1][2]
     out2 = generate(eng, ps, GenerationParams(max_tokens=n_new, temperature=0.0, repeat_penalty=1.0), eos_ids=[stop])
