@@ -1,7 +1,24 @@
-// The skinny product (up to 16 rows of x, bfloat16, MFMA, weights streamed once; see
-// skinny_gemm.hip for the mapping) with the neighbouring small operations of a decoding
-// step folded into its two ends, so that a layer takes six kernel launches instead of
-// nine.  At these sizes a launch costs as much as the work of a norm or a rotation.
+// y[M,N] = x[M,K] w[N,K]^T for few rows M (up to 16: decoding steps, chosen logit rows): the
+// weights are streamed from HBM exactly once and never staged; bfloat16 in, MFMA, float32
+// accumulation.  The reference runs these products as candle matmuls
+// (src/models/turbo_generic.rs:68-91); at these M they are bound by the weight bytes, so the
+// kernel is laid out for memory, not for the matrix cores.
+//
+// v_mfma_f32_16x16x32_bf16 computes D[16x16] += A[16x32] B[32x16].  Here A is a tile of w (16
+// output features x 32 k) and B a tile of x^T (32 k x 16 rows of x), so D[n][m] is a tile of
+// y^T.  Lane l holds, of A, row l%16 and the 8 consecutive k starting at 8*(l/16): 16
+// contiguous bytes of a weight row, loaded straight from global memory; of B the same 16
+// bytes of x's row l%16; of D column m = l%16 and rows n = 4*(l/16) .. +3.
+//
+// A block owns one tile of 16 output features, or a pair of tiles that meet the same x (gate
+// and up rows of one output; the two halves of a head that rotate with each other; two
+// neighbouring tiles of a very wide product).  Its waves split K between them in chunks and
+// add their partial tiles up through LDS in wave order, so the sum has a fixed order whatever
+// the timing, and one that depends on the product's shape alone, not on M.
+//
+// The neighbouring small operations of a decoding step are folded into the kernel's two ends,
+// so that a layer takes six kernel launches instead of nine: at these sizes a launch costs
+// as much as the work of a norm or a rotation.
 //
 // The norm between two products is split over them.  RMSNorm is x / rms(x) * weight
 // (src/models/turbo_generic.rs:41-51), and the division by the row's rms commutes with

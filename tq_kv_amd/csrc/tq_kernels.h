@@ -38,12 +38,6 @@ int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const void* weig
 int tqk_gemm(const void* x, int x_dtype, const void* w, int w_dtype, const void* bias,
              int bias_dtype, void* y, int y_dtype, int M, int N, int K, void* stream);
 
-/* Skinny product for few rows: y[M,N] = x[M,K] w[N,K]^T, bfloat16 in, MFMA, float32
- * accumulation; epilogue 0: store y (y_dtype), 1: w holds gate rows then up rows
- * (N = 2*inter), y[M,inter] = silu(gate)*up (bfloat16).  K must be a multiple of 32. */
-int tqk_skinny_bf16(const void* x, const void* w, void* y, int y_dtype, int M, int N, int K,
-                    int epilogue, void* stream);
-
 /* Skinny products (up to 16 rows, bfloat16, K a multiple of 32) with the small operations
  * around them folded in.  A norm between two products is split over them: the one that adds
  * to the stream h writes xw = bfloat16(h * weight of the next norm) and the sums of h^2 in

@@ -183,23 +183,6 @@ def argmax(logits, out):
     return out
 
 
-def has_skinny():
-    """Whether the library holds the MFMA kernel for products with few rows."""
-    return hasattr(library(), "tqk_skinny_bf16")
-
-
-def skinny_bf16(x, w, out, swiglu=False):
-    """out[M,N] = x[M,K] w[N,K]^T for few rows, bfloat16 in; with swiglu, w holds gate rows
-    then up rows and out[M, N/2] = silu(gate) * up."""
-    m, k = x.shape
-    n = w.shape[0]
-    n_out = n // 2 if swiglu else n
-    _check(library().tqk_skinny_bf16(
-        _dev(x, "x", torch.bfloat16, (m, k)), _dev(w, "w", torch.bfloat16, (n, k)),
-        _dev(out, "out", None, (m, n_out)), _code(out.dtype), m, n, k, 1 if swiglu else 0, _stream()), "skinny_bf16")
-    return out
-
-
 def repeat_penalty(logits, row_req, hist, times, hist_len, penalty):
     """In place: for every token in the history of the row's request, once per occurrence,
     l > 0 ? l / penalty : l * penalty.  hist, times, hist_len: as append_history keeps them."""

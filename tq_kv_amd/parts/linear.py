@@ -6,7 +6,8 @@ The reference's linear layers are candle matmuls, i.e. library GEMMs
   float32 anywhere (the 32-bit path, or a weight stored in 32-bit)
         -> the hand-written FMA kernel (no matrix cores, fixed summation order)
   bfloat16, up to 16 rows (decoding, chosen logit rows)
-        -> the hand-written weight-streaming MFMA kernel
+        -> the hand-written weight-streaming MFMA kernel (kernels.fused_*: alone here, with
+           the neighbouring norm, residual sum, gate or rotation folded in where parts ask)
   bfloat16, more rows (prompts, large decoding batches)
         -> the library GEMM (hipBLASLt through torch), float32 accumulation; float32
            output where logits are wanted
@@ -86,7 +87,7 @@ def freeze_library_tuning():
 
 def _skinny_ok(x, weight):
     return (POLICY["skinny"] and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-            and x.shape[1] % 32 == 0 and x.shape[0] <= POLICY["skinny_max_rows"] and K.has_skinny())
+            and x.shape[1] % 32 == 0 and x.shape[0] <= POLICY["skinny_max_rows"])
 
 
 def gated_silu_linear(x, weight_gate_up):
@@ -97,7 +98,7 @@ def gated_silu_linear(x, weight_gate_up):
     inter = weight_gate_up.shape[0] // 2
     act = torch.empty((m, inter), dtype=x.dtype, device=x.device)
     if _skinny_ok(x, weight_gate_up):
-        return K.skinny_bf16(x, weight_gate_up, act, swiglu=True)
+        return K.fused_gated(x, weight_gate_up, act)
     return K.swiglu(linear(x, weight_gate_up), act)
 
 
@@ -113,7 +114,7 @@ def linear(x, weight, bias=None, out_dtype=None):
     if both_bf16 and bias is None:
         if _skinny_ok(x, weight):
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-            return K.skinny_bf16(x, weight, out)
+            return K.fused_store(x, weight, out)
         if POLICY["library"] and m > POLICY["skinny_max_rows"]:
             if out_dtype == torch.bfloat16:
                 return torch.matmul(x, weight.t())
