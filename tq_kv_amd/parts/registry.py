@@ -14,10 +14,11 @@ Categories and what each must offer beyond `tensors()` and `load()`:
   mixer         cache_need() -> KVNeed | StateNeed | None;
                 forward(x, ctx, cache_entry) -> y, x and y [tokens, hidden]
   feed_forward  forward(x, ctx) -> y
-  block         the arrangement: forward(stream, ctx, cache_entry, next_norm), where stream
-                (parts.linear.Stream) holds the float32 residual stream h and the update
-                not yet added to it, and next_norm is the norm that reads the stream after
-                this block; first_norm() -> the norm this block reads the stream with
+  block         the arrangement: forward(stream, ctx, cache_entry, next_norm, last) -> stream,
+                where stream (parts.linear.Stream) holds the float32 residual stream h and
+                the update not yet added to it, next_norm is the norm that reads the stream
+                after this block, and last says that only the head does; first_norm() -> the
+                norm this block reads the stream with
 
 Optional, for a step that wants fewer rows than it has tokens: a mixer with `takes_rows` accepts
 `last_rows=True` in the last run of the order and returns its output for ctx's last_rows alone
