@@ -28,7 +28,7 @@ def ints(values):
 
 
 def test_library_is_built_and_loaded():
-    assert K.library().tqk_abi_version() == 3
+    assert K.library().tqk_abi_version() == 4
     assert K.library_path().endswith(".so")
     with pytest.raises(K.KernelError, match="GPU only"):
         K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
@@ -91,13 +91,19 @@ def test_gemm_generic(m, n, k, xd, wd, yd):
     torch.testing.assert_close(out.double(), want + b.double(), **tol)
 
 
-def test_gemm_generic_rows_do_not_depend_on_the_batch():
-    x, w = rand(70, 96, seed=8), rand(130, 96, seed=9)
-    full = torch.empty(70, 130, device=DEV)
-    K.gemm(x, w, None, full)
-    one = torch.empty(1, 130, device=DEV)
-    K.gemm(x[41:42].contiguous(), w, None, one)
-    assert torch.equal(one[0], full[41])
+@pytest.mark.parametrize("rows,n,k,bias", [(1, 130, 96, False), (3, 130, 2500, True), (16, 67, 1024, True),
+                                           (7, 64, 3076, False), (5, 200, 1030, True), (2, 130, 97, True)])
+def test_gemm_generic_rows_do_not_depend_on_the_batch(rows, n, k, bias):
+    """Up to 16 float32 rows go through the kernel for few rows (k a multiple of 4), more through
+    the tiled one: the same bits, over chunks and groups of k that are full or not."""
+    x, w = rand(70, k, seed=8), rand(n, k, seed=9)
+    b = rand(n, seed=10) if bias else None
+    full = torch.empty(70, n, device=DEV)
+    K.gemm(x, w, b, full)
+    torch.testing.assert_close(full.double(), x.double() @ w.double().t() + (b.double() if bias else 0), atol=2e-4, rtol=1e-5)
+    few = torch.full((rows, n), float("nan"), device=DEV)
+    K.gemm(x[41:41 + rows].contiguous(), w, b, few)
+    assert torch.equal(few, full[41:41 + rows])
 
 
 def value_place(p):

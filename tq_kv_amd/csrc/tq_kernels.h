@@ -34,9 +34,11 @@ int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const void* weig
                     int hidden, void* out, int write_back, void* stream);
 
 /* y[M,N] = x[M,K] w[N,K]^T (+ bias[N]); float32 accumulation in a fixed order that
- * does not depend on M.  Any sizes. */
+ * does not depend on M.  Any sizes.  scratch: tqk_gemm_scratch_bytes(...) bytes of device
+ * memory, 16-byte aligned (may be null: then, or where that is 0, the tiled kernel runs). */
+size_t tqk_gemm_scratch_bytes(int x_dtype, int w_dtype, int bias_dtype, int y_dtype, int M, int N, int K);
 int tqk_gemm(const void* x, int x_dtype, const void* w, int w_dtype, const void* bias,
-             int bias_dtype, void* y, int y_dtype, int M, int N, int K, void* stream);
+             int bias_dtype, void* y, int y_dtype, int M, int N, int K, void* scratch, void* stream);
 
 /* Skinny products (up to 16 rows, bfloat16, K a multiple of 32) with the small operations
  * around them folded in.  A norm between two products is split over them: the one that adds

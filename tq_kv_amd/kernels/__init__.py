@@ -33,6 +33,7 @@ def library():
         lib.tqk_last_error.restype = ctypes.c_char_p
         lib.tqk_abi_version.restype = ctypes.c_int
         lib.tqk_sample_scratch_bytes.restype = ctypes.c_size_t
+        lib.tqk_gemm_scratch_bytes.restype = ctypes.c_size_t
         _LIB = lib
     return _LIB
 
@@ -116,10 +117,14 @@ def gemm(x, w, bias, out):
     """out[M,N] = x[M,K] w[N,K]^T (+ bias[N]), float32 accumulation, any dtype mix."""
     m, k = x.shape
     n = w.shape[0]
-    _check(library().tqk_gemm(
+    lib = library()
+    bias_code = _code(bias.dtype) if bias is not None else 0
+    need = int(lib.tqk_gemm_scratch_bytes(_code(x.dtype), _code(w.dtype), bias_code, _code(out.dtype), m, n, k))
+    scratch = torch.empty((need,), dtype=torch.uint8, device=x.device) if need else None
+    _check(lib.tqk_gemm(
         _dev(x, "x", None, (m, k)), _code(x.dtype), _dev(w, "w", None, (n, k)), _code(w.dtype),
-        _opt(bias, "bias", None, (n,)), _code(bias.dtype) if bias is not None else 0,
-        _dev(out, "out", None, (m, n)), _code(out.dtype), m, n, k, _stream()), "gemm")
+        _opt(bias, "bias", None, (n,)), bias_code,
+        _dev(out, "out", None, (m, n)), _code(out.dtype), m, n, k, _opt(scratch, "scratch"), _stream()), "gemm")
     return out
 
 
