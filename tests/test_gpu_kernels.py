@@ -28,7 +28,7 @@ def ints(values):
 
 
 def test_library_is_built_and_loaded():
-    assert K.library().tqk_abi_version() == 4
+    assert K.library().tqk_abi_version() == 5
     assert K.library_path().endswith(".so")
     with pytest.raises(K.KernelError, match="GPU only"):
         K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
@@ -425,11 +425,38 @@ def test_sample_frequencies_follow_the_softmax():
     torch.testing.assert_close(got, torch.softmax(logits[0].cpu(), 0), atol=1e-3, rtol=0)
 
 
+FORMS = ["rows", "packed"]
+
+
+def in_form(w, form, parts=1):
+    """The weight as the checkpoint has it, or packed for the few-row kernels."""
+    return K.pack_weight(w, parts) if form == "packed" else w
+
+
+def test_packed_weight_layout():
+    n, k = 40, 96                                   # 3 tiles, the last half empty
+    w = rand(n, k, seed=29, dtype=torch.bfloat16)
+    packed = K.pack_weight(w)
+    assert tuple(packed.data.shape) == (3, 3, 64, 8) and packed.shape == (n, k) and packed.data.is_contiguous()
+    for row, col in [(0, 0), (17, 40), (39, 95), (16, 31), (5, 64)]:
+        lane = 16 * ((col % 32) // 8) + row % 16
+        assert packed.data[row // 16, col // 32, lane, col % 8] == w[row, col]
+    assert not packed.data[2, :, 8:16].any() and not packed.data[2, :, 24:32].any()       # rows 40..47 are zeros
+    two = K.pack_weight(torch.cat([w, -w]), parts=2)                   # each part padded by itself
+    assert tuple(two.data.shape) == (6, 3, 64, 8) and torch.equal(two.data[3:], -packed.data)
+    with pytest.raises(K.KernelError, match="multiple of 32"):
+        K.pack_weight(rand(16, 48, dtype=torch.bfloat16))
+    with pytest.raises(K.KernelError, match="packed weight is"):
+        K.fused_store(rand(2, k, dtype=torch.bfloat16), packed, torch.empty(2, n + 1, device=DEV))
+
+
+@pytest.mark.parametrize("form", FORMS)
 @pytest.mark.parametrize("m", [1, 3, 8, 16])
 @pytest.mark.parametrize("n,k", [(100, 96), (3584, 3584), (1000, 18944), (4608, 1536), (48, 32), (65610, 64)])
-def test_product_of_few_rows(m, n, k):
+def test_product_of_few_rows(m, n, k, form):
     x, w = rand(m, k, seed=30, dtype=torch.bfloat16), rand(n, k, seed=31, scale=0.05, dtype=torch.bfloat16)
     want = x.double() @ w.double().t()
+    w = in_form(w, form)
     out = torch.full((m, n), float("nan"), device=DEV)
     K.fused_store(x, w, out)
     torch.testing.assert_close(out.double(), want, atol=2e-3, rtol=1e-3)
@@ -557,49 +584,63 @@ def prepared(h, nw):
     return xw, (ss, parts)
 
 
+@pytest.mark.parametrize("form", FORMS)
 @pytest.mark.parametrize("m", [1, 5, 16])
 @pytest.mark.parametrize("n,k", [(100, 96), (3584, 3584), (1000, 1536), (65610, 64)])       # the last: blocks of two tiles
-def test_fused_store_with_and_without_norm(m, n, k):
+def test_fused_store_with_and_without_norm(m, n, k, form):
     h = rand(16, k, seed=100, scale=2.0)
     w = rand(n, k, seed=101, scale=1.0 / math.sqrt(k), dtype=torch.bfloat16)
+    w, w_rows = in_form(w, form), w
     nw = (1 + rand(k, seed=102, scale=0.1)).to(torch.bfloat16)
     rows = ints(list(range(15, 15 - m, -1)))                     # m rows of x, backwards
     out = torch.full((m, n), float("nan"), device=DEV)
     xb = h.to(torch.bfloat16)
     K.fused_store(xb, w, out, rows=rows)
-    torch.testing.assert_close(out.double(), xb.double()[rows.long()] @ w.double().t(), atol=2e-3, rtol=1e-3)
+    torch.testing.assert_close(out.double(), xb.double()[rows.long()] @ w_rows.double().t(), atol=2e-3, rtol=1e-3)
     eps = 1e-5
     xw, (ss, parts) = prepared(h, nw)
     K.fused_store(xw, w, out, (ss, parts, eps), rows=rows)
-    want = plain.rms_norm(h[rows.long()], nw.float(), eps).double() @ w.double().t()
+    want = plain.rms_norm(h[rows.long()], nw.float(), eps).double() @ w_rows.double().t()
     torch.testing.assert_close(out.double(), want, atol=2e-2, rtol=2e-2)
+    if form == "packed":            # the same sums in the same order as from the rows
+        same = torch.empty_like(out)
+        K.fused_store(xw, w_rows, same, (ss, parts, eps), rows=rows)
+        assert torch.equal(out, same)
 
 
+@pytest.mark.parametrize("form", FORMS)
 @pytest.mark.parametrize("m", [1, 8, 16])
-@pytest.mark.parametrize("inter,k", [(112, 64), (18944, 3584)])
-def test_fused_gated(m, inter, k):
+@pytest.mark.parametrize("inter,k", [(112, 64), (18944, 3584), (100, 96)])
+def test_fused_gated(m, inter, k, form):
     h = rand(m, k, seed=103, scale=1.5)
-    w = rand(2 * inter, k, seed=104, scale=0.4 / math.sqrt(k), dtype=torch.bfloat16)      # gate and up of size about 1
+    w_rows = rand(2 * inter, k, seed=104, scale=0.4 / math.sqrt(k), dtype=torch.bfloat16)      # gate and up of size about 1
+    w = in_form(w_rows, form, parts=2)
     nw = (1 + rand(k, seed=105, scale=0.1)).to(torch.bfloat16)
     out = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
     xw, (ss, parts) = prepared(h, nw)
     K.fused_gated(xw, w, out, (ss, parts, 1e-6))
-    gu = bf(plain.rms_norm(h, nw.float(), 1e-6).double() @ w.double().t())
+    gu = bf(plain.rms_norm(h, nw.float(), 1e-6).double() @ w_rows.double().t())
     torch.testing.assert_close(out.float(), F.silu(gu[:, :inter]) * gu[:, inter:], atol=3e-2, rtol=3e-2)
     xb = h.to(torch.bfloat16)
     K.fused_gated(xb, w, out)
-    gu = bf(xb.double() @ w.double().t())
+    gu = bf(xb.double() @ w_rows.double().t())
     torch.testing.assert_close(out.float(), F.silu(gu[:, :inter]) * gu[:, inter:], atol=3e-2, rtol=3e-2)
+    if form == "packed":
+        same = torch.empty_like(out)
+        K.fused_gated(xb, w_rows, same)
+        assert torch.equal(out, same)
 
 
+@pytest.mark.parametrize("form", FORMS)
 @pytest.mark.parametrize("m", [1, 7, 16])
 @pytest.mark.parametrize("n,k", [(96, 64), (3584, 18944), (100, 32)])
-def test_fused_residual_prepares_the_next_norm(m, n, k):
+def test_fused_residual_prepares_the_next_norm(m, n, k, form):
     x = rand(m, k, seed=106, dtype=torch.bfloat16)
-    w = rand(n, k, seed=107, scale=0.02, dtype=torch.bfloat16)
+    w_rows = rand(n, k, seed=107, scale=0.02, dtype=torch.bfloat16)
+    w = in_form(w_rows, form)
     nw = (1 + rand(n, seed=113, scale=0.1)).to(torch.bfloat16)
     h = rand(m, n, seed=108, scale=3.0)
-    want = h + bf((x.double() @ w.double().t()).float())
+    want = h + bf((x.double() @ w_rows.double().t()).float())
     xw = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
     ss = torch.full((K.fused_residual_parts(n, k), 16), float("nan"), device=DEV)
     parts = K.fused_residual(x, w, h, xw, nw, ss)
@@ -630,12 +671,13 @@ def test_embed_prepares_the_first_norm(hidden):
     torch.testing.assert_close(ss[0, :3], (h * h).sum(-1), rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("form", FORMS)
 @pytest.mark.parametrize("nh,nkv,d,k", [(28, 4, 128, 3584), (3, 1, 32, 96), (6, 2, 64, 160)])
-def test_fused_qkv_equals_product_then_rotation_kernel(nh, nkv, d, k):
+def test_fused_qkv_equals_product_then_rotation_kernel(nh, nkv, d, k, form):
     m, n_pages = 5, 9
     total = (nh + 2 * nkv) * d
     h = rand(m, k, seed=109, scale=1.5)
-    w = rand(total, k, seed=110, scale=1.0 / math.sqrt(k), dtype=torch.bfloat16)
+    w = in_form(rand(total, k, seed=110, scale=1.0 / math.sqrt(k), dtype=torch.bfloat16), form)
     bias = rand(total, seed=111, scale=0.3, dtype=torch.bfloat16)
     nw = (1 + rand(k, seed=112, scale=0.1)).to(torch.bfloat16)
     c, s = plain.rope_tables(d, 1e4, 400)

@@ -122,3 +122,24 @@ def test_model_lists_tensors_by_the_reference_names():
         want |= {p + "mlp.%s_proj.weight" % x for x in ("gate", "up", "down")}
         want |= {p + "input_layernorm.weight", p + "post_attention_layernorm.weight"}
     assert names == want
+
+
+def test_packed_copy_of_a_weight_holds_every_value_once():
+    """The few-row kernels' order: [tile of 16 rows][k / 32][lane][8], lane = 16 * ((k % 32) / 8) + row % 16,
+    rows padded with zeros to whole tiles, stacked parts padded one by one."""
+    from tq_kv_amd import kernels as K
+    n, k = 40, 96
+    w = torch.arange(n * k, dtype=torch.float32).reshape(n, k).to(torch.bfloat16)
+    packed = K.pack_weight(w)
+    assert tuple(packed.data.shape) == (3, 3, 64, 8) and packed.shape == (n, k) and packed.parts == 1
+    for row in range(n):
+        for col in range(0, k, 7):
+            lane = 16 * ((col % 32) // 8) + row % 16
+            assert packed.data[row // 16, col // 32, lane, col % 8] == w[row, col]
+    assert packed.data.float().sum() == w.float().sum()         # the padding is zeros
+    two = K.pack_weight(torch.cat([w, -w]), parts=2)
+    assert tuple(two.data.shape) == (6, 3, 64, 8) and torch.equal(two.data[3:], -packed.data)
+    with pytest.raises(K.KernelError, match="multiple of 32"):
+        K.pack_weight(torch.zeros(16, 48, dtype=torch.bfloat16))
+    with pytest.raises(K.KernelError, match="bfloat16"):
+        K.pack_weight(torch.zeros(16, 64))

@@ -44,20 +44,23 @@ int tqk_gemm(const void* x, int x_dtype, const void* w, int w_dtype, const void*
  * around them folded in.  A norm between two products is split over them: the one that adds
  * to the stream h writes xw = bfloat16(h * weight of the next norm) and the sums of h^2 in
  * pieces (tqk_fused_residual, tqk_embed); the one that consumes the norm takes xw and the
- * pieces (ss_parts [n_ss_parts, 16]) and divides its result by sqrt(sum / K + eps). */
+ * pieces (ss_parts [n_ss_parts, 16]) and divides its result by sqrt(sum / K + eps).
+ * w is [N, K] row by row, or with w_packed in the order the lanes take it:
+ * [tile of 16 rows][K/32][64 lanes][8 values], lane = 16 * ((k % 32) / 8) + row % 16, the rows
+ * padded with zeros to whole tiles (a gated weight: gate rows, then up rows, each padded). */
 int tqk_fused_store(const void* x, const int32_t* x_rows, const float* ss_parts, int n_ss_parts, float eps,
-                    const void* w, void* y, int y_dtype, int M, int N, int K, void* stream);
+                    const void* w, int w_packed, void* y, int y_dtype, int M, int N, int K, void* stream);
 /* y[M, N/2] = silu(gate) * up, w = gate rows then up rows */
-int tqk_fused_gated(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, void* y,
+int tqk_fused_gated(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, int w_packed, void* y,
                     int M, int N, int K, void* stream);
 /* h[M,N] += bfloat16(x w^T) in float32; xw_out = bfloat16(h * next_norm_w) or bfloat16(h);
  * ss_out (optional) [tqk_fused_residual_parts(N, K), 16] */
 int tqk_fused_residual_parts(int N, int K);
-int tqk_fused_residual(const void* x, const void* w, float* h, const void* next_norm_w, void* xw_out,
+int tqk_fused_residual(const void* x, const void* w, int w_packed, float* h, const void* next_norm_w, void* xw_out,
                        float* ss_out, int M, int N, int K, void* stream);
 /* q, k, v of a decoding step: + bias, rotation (halves over the whole head) at tok_pos[m],
  * q to q_out [M, heads, head_dim], k and v into the cache page of sequence m */
-int tqk_fused_qkv(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, const void* bias,
+int tqk_fused_qkv(const void* x, const float* ss_parts, int n_ss_parts, float eps, const void* w, int w_packed, const void* bias,
                   const float* cos_table, const float* sin_table, int max_positions,
                   const int32_t* tok_pos, const int32_t* page_table, int table_width,
                   void* keys, void* values, int n_pages, void* q_out,

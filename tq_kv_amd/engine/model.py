@@ -47,6 +47,7 @@ class Model:
                 mixer.reads_other_cache = True
         self.embedding = None
         self.head = None
+        self.few_head = None
         self.loaded = False
         # a step can be captured as a graph if every part's forward launches the same kernels
         # whatever the step's data are; up to 64 rows (beyond 16 the products are library calls,
@@ -76,6 +77,7 @@ class Model:
             block.load({name: tensors[layer.prefix + name] for name in block.tensors()})
         self.final_norm.load({name: tensors[s.final_norm_prefix + name] for name in self.final_norm.tensors()})
         self.head = self.embedding if s.head_name is None else tensors[s.head_name]
+        self.few_head = L.few_rows_form(self.head)      # the head's copy for the few-row kernel
         self.loaded = True
         return self
 
@@ -166,9 +168,9 @@ class Model:
         lazy = self.final_norm.lazy(stream) if ctx.fuse_small and hasattr(self.final_norm, "lazy") else None
         if lazy is not None and n_rows <= 16 and L.fusable(n_rows, self.head):
             logits = torch.empty((n_rows, s.vocab_size), dtype=torch.float32, device=self.device)
-            return K.fused_store(lazy.xw, self.head, logits, lazy.norm, rows=want_rows)
+            return K.fused_store(lazy.xw, self.few_head or self.head, logits, lazy.norm, rows=want_rows)
         x = self.final_norm.gather_add_norm(stream.h, stream.pending, want_rows)
-        return linear(x, self.head, out_dtype=torch.float32)
+        return linear(x, self.head, out_dtype=torch.float32, few=self.few_head)
 
     def __repr__(self):
         s = self.spec

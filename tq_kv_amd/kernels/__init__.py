@@ -293,17 +293,58 @@ def _norm_args(norm, m):
     return _dev(ss_parts, "ss_parts", torch.float32), int(n_parts), ctypes.c_float(eps)
 
 
+class PackedWeight:
+    """A bfloat16 weight [n, k] in the order the lanes of the few-row kernels take it:
+    data [tiles, k/32, 64, 8], where tile t holds 16 rows, lane = 16 * ((k % 32) / 8) + row % 16.
+    parts: the weight is that many stacked weights of n/parts rows (gate and up rows), each
+    padded with zero rows to whole tiles."""
+
+    dtype = torch.bfloat16
+
+    def __init__(self, data, n, k, parts):
+        self.data, self.shape, self.parts = data, (n, k), parts
+
+
+def pack_weight(weight, parts=1):
+    """The PackedWeight of a contiguous bfloat16 weight [n, k], k a multiple of 32 (runs
+    wherever the weight lives; takes the weight's size in new memory)."""
+    n, k = weight.shape
+    if weight.dtype != torch.bfloat16 or k % 32 or n % parts:
+        raise KernelError("pack_weight: needs bfloat16 [n, k] with k a multiple of 32 and n of %d parts, got %s %s"
+                          % (parts, weight.dtype, tuple(weight.shape)))
+    per = n // parts
+    tiles = (per + 15) // 16
+    w = weight.reshape(parts, per, k)
+    if per % 16:
+        w = torch.cat([w, w.new_zeros((parts, tiles * 16 - per, k))], dim=1)
+    # [part, tile, row, k step, k group, 8] -> [part, tile, k step, k group, row, 8]
+    data = w.reshape(parts, tiles, 16, k // 32, 4, 8).permute(0, 1, 3, 4, 2, 5).contiguous()
+    return PackedWeight(data.reshape(parts * tiles, k // 32, 64, 8), n, k, parts)
+
+
+def _weight(weight, name, n, k, parts=1):
+    """Pointer and packed flag of a product's weight, row by row [n, k] or packed."""
+    if isinstance(weight, PackedWeight):
+        if tuple(weight.shape) != (n, k) or weight.parts != parts:
+            raise KernelError("%s: the packed weight is %s in %d parts, wanted %s in %d"
+                              % (name, tuple(weight.shape), weight.parts, (n, k), parts))
+        return _dev(weight.data, name, torch.bfloat16), 1
+    return _dev(weight, name, torch.bfloat16, (n, k)), 0
+
+
 def fused_store(x, weight, out, norm=None, rows=None):
     """out[M,N] = x weight^T (divided by the rows' rms with `norm`); x bfloat16 [*, K]
-    (rows: int32 indices of the M rows used)."""
+    (rows: int32 indices of the M rows used).  Here and in the other fused_* products the
+    weight is a tensor [N, K] or its PackedWeight."""
     m, n = out.shape
     k = weight.shape[1]
     if x.shape[1] != k or (rows is None and x.shape[0] != m) or x.shape[0] > 16:
         raise KernelError("fused_store: x is %s for %d rows of %d (at most 16 rows)" % (tuple(x.shape), m, k))
     ss, n_parts, eps = _norm_args(norm, m)
+    w, packed = _weight(weight, "weight", n, k)
     _check(library().tqk_fused_store(
         _dev(x, "x", torch.bfloat16), _opt(rows, "rows", torch.int32, (m,)), ss, n_parts, eps,
-        _dev(weight, "weight", torch.bfloat16, (n, k)), _dev(out, "out"), _code(out.dtype), m, n, k, _stream()), "fused_store")
+        w, packed, _dev(out, "out"), _code(out.dtype), m, n, k, _stream()), "fused_store")
     return out
 
 
@@ -312,9 +353,10 @@ def fused_gated(x, weight_gate_up, out, norm=None):
     m, inter = out.shape
     k = weight_gate_up.shape[1]
     ss, n_parts, eps = _norm_args(norm, m)
+    w, packed = _weight(weight_gate_up, "weight", 2 * inter, k, parts=2)
     _check(library().tqk_fused_gated(
         _dev(x, "x", torch.bfloat16, (m, k)), ss, n_parts, eps,
-        _dev(weight_gate_up, "weight", torch.bfloat16, (2 * inter, k)), _dev(out, "out", torch.bfloat16), m, 2 * inter, k,
+        w, packed, _dev(out, "out", torch.bfloat16), m, 2 * inter, k,
         _stream()), "fused_gated")
     return out
 
@@ -334,8 +376,9 @@ def fused_residual(x, weight, h, xw, next_norm_weight=None, ss_out=None):
     parts = fused_residual_parts(n, k)
     if ss_out is not None and ss_out.numel() < parts * 16:
         raise KernelError("fused_residual: ss_out holds %d values, %d pieces of 16 are written" % (ss_out.numel(), parts))
+    w, packed = _weight(weight, "weight", n, k)
     _check(library().tqk_fused_residual(
-        _dev(x, "x", torch.bfloat16), _dev(weight, "weight", torch.bfloat16, (n, k)), _dev(h, "h", torch.float32, (m, n)),
+        _dev(x, "x", torch.bfloat16), w, packed, _dev(h, "h", torch.float32, (m, n)),
         _opt(next_norm_weight, "next_norm_weight", torch.bfloat16, (n,)), _dev(xw, "xw", torch.bfloat16, (m, n)),
         _opt(ss_out, "ss_out", torch.float32), m, n, k, _stream()), "fused_residual")
     return parts
@@ -351,9 +394,10 @@ def fused_qkv(x, weight, bias, cos, sin, tok_pos, page_table, keys, values, q_ou
     width = page_table.shape[1]
     max_pos = cos.shape[0]
     ss, n_parts, eps = _norm_args(norm, m)
+    w, packed = _weight(weight, "weight", total, k)
     _check(library().tqk_fused_qkv(
         _dev(x, "x", torch.bfloat16), ss, n_parts, eps,
-        _dev(weight, "weight", torch.bfloat16, (total, k)), _opt(bias, "bias", torch.bfloat16, (total,)),
+        w, packed, _opt(bias, "bias", torch.bfloat16, (total,)),
         _dev(cos, "cos", torch.float32, (max_pos, head_dim // 2)), _dev(sin, "sin", torch.float32, (max_pos, head_dim // 2)), max_pos,
         _dev(tok_pos, "tok_pos", torch.int32, (m,)), _dev(page_table, "page_table", torch.int32, (m, width)), width,
         _dev(keys, "keys", torch.bfloat16, (n_pages, n_kv_heads, 64, head_dim)),

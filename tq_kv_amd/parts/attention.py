@@ -11,7 +11,7 @@ import math
 import torch
 
 from .. import kernels as K
-from .linear import LazyNorm, fusable, linear
+from .linear import LazyNorm, few_rows_form, fusable, linear
 from .registry import Part, register
 from .spec import KVNeed, TensorSpec
 
@@ -45,6 +45,7 @@ class Attention(Part):
         self.position = env.shared[key]
         self.graph_safe = not hasattr(self.position, "apply") or getattr(self.position, "graph_safe", False)
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+        self.few_qkv = self.few_o = None    # the weights' copies for the few-row kernels
         self.reads_other_cache = False      # set when a run of this layer reads another run's cache
         self.takes_rows = True              # forward(..., last_rows=True) computes the step's last_rows only
 
@@ -68,6 +69,8 @@ class Attention(Part):
             self.b_qkv = torch.cat([b.to(bdtype) for b in bs], dim=0).contiguous()
         self.w_o = tensors["o_proj.weight"]
         self.b_o = tensors.get("o_proj.bias")
+        self.few_qkv = few_rows_form(self.w_qkv)
+        self.few_o = few_rows_form(self.w_o)
 
     def cache_need(self):
         return KVNeed(self.n_kv_heads, self.head_dim, self.window)
@@ -106,7 +109,7 @@ class Attention(Part):
             if lazy and not entry.writes:
                 raise RuntimeError("a run that reads another run's cache cannot take a folded norm")
             cos, sin, _, _ = self.position.tables()
-            K.fused_qkv(x.xw if lazy else x, self.w_qkv, self.b_qkv, cos, sin, ctx.dev.tok_pos, table,
+            K.fused_qkv(x.xw if lazy else x, self.few_qkv or self.w_qkv, self.b_qkv, cos, sin, ctx.dev.tok_pos, table,
                         entry.keys, entry.values, q, self.n_heads, self.n_kv_heads, self.head_dim,
                         norm=x.norm if lazy else None)
         else:
@@ -117,17 +120,17 @@ class Attention(Part):
                 return torch.empty((0, self.hidden), dtype=dtype, device=q.device)
             y = torch.empty((ctx.n_last, self.n_heads * self.head_dim), dtype=dtype, device=q.device)
             attend_rows(q.index_select(0, d.last_rows), entry, table, ctx, self.window, self.scale, y)
-            return linear(y, self.w_o, self.b_o)
+            return linear(y, self.w_o, self.b_o, few=self.few_o)
         y = torch.empty((n, self.n_heads * self.head_dim), dtype=dtype, device=q.device)
         attend(q, entry, table, ctx, self.window, self.scale, y)
         if stream is not None:
-            stream.add_product(y, self.w_o)
+            stream.add_product(y, self.few_o or self.w_o)
             return None
-        return linear(y, self.w_o, self.b_o)
+        return linear(y, self.w_o, self.b_o, few=self.few_o)
 
     def _qkv(self, x, ctx, entry, table, q):
         """Product, then bias, position encoding and cache write in their own kernel."""
-        qkv = linear(x, self.w_qkv)
+        qkv = linear(x, self.w_qkv, few=self.few_qkv)
         if hasattr(self.position, "apply"):
             # a position encoding of its own: bias first, then it changes q and k in place
             if self.b_qkv is not None:

@@ -4,7 +4,7 @@ up are one product with the weights stacked."""
 import torch
 
 from .. import kernels as K
-from .linear import LazyNorm, fusable, gated_silu_linear, linear
+from .linear import LazyNorm, few_rows_form, fusable, gated_silu_linear, linear
 from .registry import Part, register
 from .spec import TensorSpec
 
@@ -18,6 +18,7 @@ class GatedSiLU(Part):
         self.hidden = int(params["hidden"])
         self.inter = int(params["inter"])
         self.w_gate_up = self.w_down = None
+        self.few_gate_up = self.few_down = None         # the weights' copies for the few-row kernels
 
     def tensors(self):
         return {"gate_proj.weight": TensorSpec((self.inter, self.hidden)),
@@ -29,6 +30,8 @@ class GatedSiLU(Part):
         dtype = torch.float32 if any(w.dtype == torch.float32 for w in ws) else ws[0].dtype
         self.w_gate_up = torch.cat([w.to(dtype) for w in ws], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"]
+        self.few_gate_up = few_rows_form(self.w_gate_up, parts=2)
+        self.few_down = few_rows_form(self.w_down)
 
     def product_weights(self):
         return [(self.w_gate_up, None), (self.w_down, None)]
@@ -44,9 +47,9 @@ class GatedSiLU(Part):
         if lazy or stream is not None:
             xin = x.xw if lazy else x
             act = torch.empty((xin.shape[0], self.inter), dtype=torch.bfloat16, device=self.w_down.device)
-            K.fused_gated(xin, self.w_gate_up, act, x.norm if lazy else None)
+            K.fused_gated(xin, self.few_gate_up or self.w_gate_up, act, x.norm if lazy else None)
             if stream is None:
-                return linear(act, self.w_down)
-            stream.add_product(act, self.w_down)
+                return linear(act, self.w_down, few=self.few_down)
+            stream.add_product(act, self.few_down or self.w_down)
             return None
-        return linear(gated_silu_linear(x, self.w_gate_up), self.w_down)
+        return linear(gated_silu_linear(x, self.w_gate_up, self.few_gate_up), self.w_down, few=self.few_down)

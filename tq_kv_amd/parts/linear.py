@@ -7,7 +7,10 @@ The reference's linear layers are candle matmuls, i.e. library GEMMs
         -> the hand-written FMA kernel (no matrix cores, fixed summation order)
   bfloat16, up to 16 rows (decoding, chosen logit rows)
         -> the hand-written weight-streaming MFMA kernel (kernels.fused_*: alone here, with
-           the neighbouring norm, residual sum, gate or rotation folded in where parts ask)
+           the neighbouring norm, residual sum, gate or rotation folded in where parts ask).
+           It reads a second copy of the weight, packed at loading time in the order its
+           lanes take it (few_rows_form): a decoding step is bound by the weight bytes, and
+           in that order they stream faster.
   bfloat16, more rows (prompts, large decoding batches)
         -> the library GEMM (hipBLASLt through torch), float32 accumulation; float32
            output where logits are wanted
@@ -20,7 +23,9 @@ from .. import kernels as K
 # plain kernel); nothing else reads these.
 # Measured on MI355X at the Qwen2.5-7B sizes: up to 16 rows the skinny kernel is ahead of the
 # library on every product; at 64 rows the library is ahead on every one.
-POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16, "fused": True, "prune_last": True}
+# "packed": parts keep the second, packed copy of their weights for the few-row kernels (twice
+# the weight memory, about an eighth less time per decoding step).
+POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16, "fused": True, "prune_last": True, "packed": True}
 
 
 class Stream:
@@ -39,7 +44,8 @@ class Stream:
         self.next_norm = None
 
     def add_product(self, x, weight):
-        """h += bfloat16(x weight^T) in the product's epilogue, preparing next_norm."""
+        """h += bfloat16(x weight^T) in the product's epilogue, preparing next_norm.  weight:
+        [N, K] or its few-row form."""
         norm = self.next_norm if getattr(self.next_norm, "foldable", False) else None
         self.n_ss = K.fused_residual(x, weight, self.h, self.xw_buffer,
                                      norm.weight if norm is not None else None, self.ss_buffer)
@@ -57,6 +63,16 @@ class LazyNorm:
 
     def __init__(self, xw, ss, n_ss, eps):
         self.xw, self.norm = xw, (ss, n_ss, eps)
+
+
+def few_rows_form(weight, parts=1):
+    """The copy of a weight [N, K] that the few-row kernels stream fastest (parts: stacked
+    weights, as gate and up), or None where they take the weight as it is (float32, a K that
+    is no multiple of 32, the policy switched off, not on the GPU)."""
+    if not (POLICY["packed"] and POLICY["skinny"] and weight.dtype == torch.bfloat16 and weight.is_cuda
+            and weight.dim() == 2 and weight.shape[1] % 32 == 0 and weight.shape[0] % parts == 0):
+        return None
+    return K.pack_weight(weight, parts)
 
 
 def fusable(x_rows, weight, adds=False):
@@ -90,21 +106,22 @@ def _skinny_ok(x, weight):
             and x.shape[1] % 32 == 0 and x.shape[0] <= POLICY["skinny_max_rows"])
 
 
-def gated_silu_linear(x, weight_gate_up):
+def gated_silu_linear(x, weight_gate_up, few=None):
     """silu(x Wg^T) * (x Wu^T) with Wg stacked on Wu: [M, K] x [2I, K] -> [M, I].  For few
     rows of bfloat16 the gate and the up row of an output are computed by the same wave
-    and never written; otherwise one product and the SwiGLU kernel."""
+    and never written; otherwise one product and the SwiGLU kernel.  few: the weight's
+    few_rows_form (parts=2), if there is one."""
     m = x.shape[0]
     inter = weight_gate_up.shape[0] // 2
     act = torch.empty((m, inter), dtype=x.dtype, device=x.device)
     if _skinny_ok(x, weight_gate_up):
-        return K.fused_gated(x, weight_gate_up, act)
+        return K.fused_gated(x, few or weight_gate_up, act)
     return K.swiglu(linear(x, weight_gate_up), act)
 
 
-def linear(x, weight, bias=None, out_dtype=None):
+def linear(x, weight, bias=None, out_dtype=None, few=None):
     """x: [M,K]; weight: [N,K]; bias: [N] or None.  Returns [M,N] of out_dtype
-    (default: x's dtype)."""
+    (default: x's dtype).  few: the weight's few_rows_form, if there is one."""
     m, k = x.shape
     n = weight.shape[0]
     if weight.shape[1] != k:
@@ -114,7 +131,7 @@ def linear(x, weight, bias=None, out_dtype=None):
     if both_bf16 and bias is None:
         if _skinny_ok(x, weight):
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-            return K.fused_store(x, weight, out)
+            return K.fused_store(x, few or weight, out)
         if POLICY["library"] and m > POLICY["skinny_max_rows"]:
             if out_dtype == torch.bfloat16:
                 return torch.matmul(x, weight.t())
