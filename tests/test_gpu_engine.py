@@ -310,8 +310,8 @@ def test_sampled_generation_float32_equals_plain(name):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_many_sequences_decode_through_replayed_graphs(dtype):
-    # 40 sequences: more rows than the skinny products take, so the captured step holds library
-    # calls too; every replay is checked (with other work between the replays)
+    # 40 sequences: more rows than the few-row products take, so the captured step holds the
+    # products for 17 to 64 rows; every replay is checked (with other work between the replays)
     eng = G.engine("B", dtype, True)
     reqs = G.prompts("B", [3 + (7 * i) % 50 for i in range(40)], seed=1000)
     slots = [eng.open() for _ in reqs]

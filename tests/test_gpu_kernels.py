@@ -28,7 +28,7 @@ def ints(values):
 
 
 def test_library_is_built_and_loaded():
-    assert K.library().tqk_abi_version() == 5
+    assert K.library().tqk_abi_version() == 6
     assert K.library_path().endswith(".so")
     with pytest.raises(K.KernelError, match="GPU only"):
         K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
@@ -468,6 +468,51 @@ def test_product_of_few_rows(m, n, k, form):
         one = torch.empty(1, n, device=DEV)
         K.fused_store(x[m - 1:].contiguous(), w, one)
         assert torch.equal(one[0], out[m - 1])
+
+
+@pytest.mark.parametrize("m", [17, 32, 33, 64])
+@pytest.mark.parametrize("n,k", [(100, 96), (3584, 3584), (1000, 18944), (4608, 1536), (48, 32), (65610, 64), (152064, 128), (264, 1056)])
+def test_product_of_17_to_64_rows(m, n, k):
+    x, w = rand(m, k, seed=32, dtype=torch.bfloat16), rand(n, k, seed=33, scale=0.05, dtype=torch.bfloat16)
+    want = x.double() @ w.double().t()
+    packed = K.pack_weight(w)
+    out = torch.full((m, n), float("nan"), device=DEV)
+    K.mid_store(x, packed, out)
+    torch.testing.assert_close(out.double(), want, atol=2e-3, rtol=1e-3)
+    out16 = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    K.mid_store(x, packed, out16)
+    assert torch.equal(out16, out.to(torch.bfloat16))
+    # a row's result does not depend on the batch it is in: other rows, another number of rows
+    few = torch.empty(20, n, device=DEV)
+    K.mid_store(x[m - 20:].contiguous() if m >= 20 else torch.cat([x, x[:20 - m]]), packed, few)
+    assert torch.equal(few[-1] if m >= 20 else few[m - 1], out[m - 1])
+    with pytest.raises(K.KernelError, match="packed"):
+        K.mid_store(x, w, out)
+
+
+@pytest.mark.parametrize("m", [17, 40, 64])
+@pytest.mark.parametrize("inter,k", [(112, 64), (18944, 3584), (100, 96), (200, 1312)])
+def test_gated_product_of_17_to_64_rows(m, inter, k):
+    x = rand(m, k, seed=34, scale=1.5, dtype=torch.bfloat16)
+    w = rand(2 * inter, k, seed=35, scale=0.4 / math.sqrt(k), dtype=torch.bfloat16)       # gate and up of size about 1
+    out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+    K.mid_gated(x, K.pack_weight(w, parts=2), out)
+    gu = (x.double() @ w.double().t()).float().to(torch.bfloat16).float()
+    torch.testing.assert_close(out.float(), F.silu(gu[:, :inter]) * gu[:, inter:], atol=3e-2, rtol=3e-2)
+    # the same as the product, rounded, through the gate kernel
+    both = torch.empty(m, 2 * inter, dtype=torch.bfloat16, device=DEV)
+    K.mid_store(x, K.pack_weight(w), both)
+    act = torch.empty_like(out)
+    K.swiglu(both, act)
+    torch.testing.assert_close(out.float(), act.float(), atol=2e-2, rtol=2e-2)
+
+
+def test_products_of_17_to_64_rows_refuse_what_they_do_not_take():
+    w = K.pack_weight(rand(16, 64, dtype=torch.bfloat16))
+    with pytest.raises(K.KernelError, match="at most 64"):
+        K.mid_store(rand(65, 64, dtype=torch.bfloat16), w, torch.empty(65, 16, device=DEV))
+    with pytest.raises(K.KernelError, match="packed weight is"):
+        K.mid_gated(rand(20, 64, dtype=torch.bfloat16), w, torch.empty(20, 8, dtype=torch.bfloat16, device=DEV))
 
 
 @pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (3, 1, 96), (40, 2, 64), (4, 1, 256)])

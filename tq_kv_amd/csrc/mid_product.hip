@@ -1,0 +1,319 @@
+// y[M,N] = x[M,K] w[N,K]^T for 17 to 64 rows (decoding steps of larger batches, the wanted rows
+// of many prompts): bfloat16 in, MFMA, float32 accumulation.  The reference runs these products
+// as candle matmuls (src/models/turbo_generic.rs:68-91).  At these M the product is still bound
+// by the weight bytes, which are streamed from HBM once, straight into registers, from the copy
+// packed in the lanes' order ([tile of 16 rows][K/32][lane][8 values], see skinny_fused.hip).
+//
+// With up to 64 rows x is no longer small beside a tile of weights: every wave needs all of it.
+// So a block is 8 waves that walk K together in chunks of 128; each chunk of x is staged once
+// per block in LDS, in the order the lanes read it ([16 rows][k step][lane] x 16 bytes, so both
+// the block's write and the waves' reads are linear), double buffered with one barrier per
+// chunk, while each wave multiplies its own tiles of 16 output features with it.  The loads of
+// the next chunk (weights and x) are under way while the current one is multiplied.
+//
+// v_mfma_f32_16x16x32_bf16: A = a tile of w (16 features x 32 k), B = 32 k x 16 rows of x, so
+// D[n][m] is a tile of y^T: lane l holds row m = l%16 of its 16-row group and the four features
+// 4*(l/16) .. +3, which it stores as one 8- or 16-byte piece.
+//
+// Where N alone gives too few blocks for the chip, K is split over blockIdx.y: each split writes
+// its sums to scratch [split][M][N] and a second kernel adds them in split order and finishes
+// (store, or the gate: silu(gate) * up of src/models/turbo_generic.rs:105-111).  The number of
+// splits depends on the product's shape alone, never on M, so a row's result does not depend on
+// the batch it is in.
+#include "common.h"
+#include "tq_kernels.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+enum { MID_STORE = 0, MID_GATED = 1 };
+#define MID_CHUNK 128           // k per stage
+#define MID_WAVES 8
+#define MID_MAX_ROWS 64
+
+struct MidArgs {
+    const bf16_t* x;            // [M, K]
+    const bf16_t* w;            // packed [tiles][K/32][64][8]
+    void* y;                    // store: [M, N]; gated: [M, N/2] bfloat16
+    float* partial;             // [splits][M][N] when the grid has splits
+    int M, N, K, k_per_split;   // k_per_split: a multiple of MID_CHUNK
+};
+
+__device__ __forceinline__ uint2 pack4_bf16(float a, float b, float c, float d) {
+    return make_uint2((uint32_t)float_to_bf16_bits(a) | ((uint32_t)float_to_bf16_bits(b) << 16),
+                      (uint32_t)float_to_bf16_bits(c) | ((uint32_t)float_to_bf16_bits(d) << 16));
+}
+
+__device__ __forceinline__ float gate_times_up(float gate_sum, float up_sum) {
+    const float g = to_float(from_float<bf16_t>(gate_sum)), up = to_float(from_float<bf16_t>(up_sum));
+    return (g / (1.f + expf(-g))) * up;
+}
+
+// MT: groups of 16 rows of x (2: up to 32 rows, 4: up to 64).  TN: tiles of 16 features per wave
+// (gated: the gate tile and its up tile).
+template <int MT, int TN, int EPI, typename TY>
+__global__ __launch_bounds__(MID_WAVES * TQK_WAVE)
+void mid_product_kernel(const MidArgs p) {
+    constexpr int SLOTS = MT * 256;                 // 16-byte pieces of a chunk of x: [row group][k step][lane]
+    constexpr int XS = SLOTS / (MID_WAVES * TQK_WAVE);
+    static_assert(SLOTS % (MID_WAVES * TQK_WAVE) == 0 && (EPI != MID_GATED || TN == 2), "shape of a block");
+    extern __shared__ u32x4_t xs[];                 // [2][SLOTS]
+    const int lane = threadIdx.x % TQK_WAVE, wave = threadIdx.x / TQK_WAVE;
+    const int row = lane % 16, kgrp = lane / 16;
+    const int K = p.K;
+    const int k_begin = blockIdx.y * p.k_per_split, k_end = min(K, k_begin + p.k_per_split);
+
+    const int n_out = EPI == MID_GATED ? p.N / 2 : p.N;             // features one part of the weight has
+    const int part_tiles = (n_out + 15) / 16;
+    const int tile0 = (blockIdx.x * MID_WAVES + wave) * (EPI == MID_GATED ? 1 : TN);
+    const int n_lo0 = tile0 * 16;
+    const size_t tile_size = (size_t)(K / 32) * 512;
+    const bf16_t* wtile[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        // tiles past the end repeat the last one; their results are dropped
+        const int tile = EPI == MID_GATED ? t * part_tiles + min(tile0, part_tiles - 1) : min(tile0 + t, part_tiles - 1);
+        wtile[t] = p.w + (size_t)tile * tile_size + lane * 8;
+    }
+    // this thread's pieces of a chunk of x; rows past M repeat the last row
+    const bf16_t* xsrc[XS];
+    int xk[XS];
+#pragma unroll
+    for (int i = 0; i < XS; ++i) {
+        const int s = threadIdx.x + i * MID_WAVES * TQK_WAVE;
+        const int mt = s / 256, ks = (s / 64) % 4, ln = s % 64;
+        xk[i] = ks * 32 + (ln / 16) * 8;
+        xsrc[i] = p.x + (size_t)min(mt * 16 + ln % 16, p.M - 1) * K;
+    }
+    floatx4_t acc[TN][MT];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[t][mt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    // Loads past the end of K stay inside the row (and are valid memory); x is zeroed there as it
+    // goes into LDS, so they add nothing.  Nothing is under a condition: the waits can be counted.
+    auto load_x = [&](int c, u32x4_t (&xr)[XS]) {
+#pragma unroll
+        for (int i = 0; i < XS; ++i) xr[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + min(c + xk[i], K - 8));
+    };
+    auto store_x = [&](int c, int buf, const u32x4_t (&xr)[XS]) {
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+            u32x4_t v = xr[i];
+            if (c + xk[i] >= k_end) v = u32x4_t{0, 0, 0, 0};
+            xs[buf * SLOTS + threadIdx.x + i * MID_WAVES * TQK_WAVE] = v;
+        }
+    };
+    auto load_w = [&](int c, bf16x8_t (&a)[TN][4]) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const size_t at = (size_t)min(c / 32 + u, K / 32 - 1) * 512;
+#pragma unroll
+            for (int t = 0; t < TN; ++t) a[t][u] = *reinterpret_cast<const bf16x8_t*>(wtile[t] + at);
+        }
+    };
+    auto multiply = [&](int buf, const bf16x8_t (&a)[TN][4]) {
+        u32x4_t bx[2][MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) bx[0][mt] = xs[buf * SLOTS + (mt * 4) * 64 + lane];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (u < 3) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) bx[(u + 1) & 1][mt] = xs[buf * SLOTS + (mt * 4 + u + 1) * 64 + lane];
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int t = 0; t < TN; ++t)
+                    acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], __builtin_bit_cast(bf16x8_t, bx[u & 1][mt]), acc[t][mt], 0, 0, 0);
+        }
+    };
+
+    bf16x8_t a0[TN][4], a1[TN][4];
+    u32x4_t xr[XS];
+    load_x(k_begin, xr);
+    load_w(k_begin, a0);
+    store_x(k_begin, 0, xr);
+    __syncthreads();
+    // two chunks a turn, so that the two register sets and the two LDS buffers keep their names;
+    // a last chunk past the end multiplies zeros
+    const int n_pairs = ((k_end - k_begin + MID_CHUNK - 1) / MID_CHUNK + 1) / 2;
+    for (int i = 0; i < n_pairs; ++i) {
+        const int c = k_begin + 2 * i * MID_CHUNK;
+        load_x(c + MID_CHUNK, xr);
+        load_w(c + MID_CHUNK, a1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(0, a0);
+        store_x(c + MID_CHUNK, 1, xr);
+        __syncthreads();
+        load_x(c + 2 * MID_CHUNK, xr);
+        load_w(c + 2 * MID_CHUNK, a0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(1, a1);
+        store_x(c + 2 * MID_CHUNK, 0, xr);
+        __syncthreads();
+    }
+
+    const int nb = 4 * kgrp;
+    if (gridDim.y > 1) {
+        const bool vec = p.N % 4 == 0;
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int m = mt * 16 + row;
+                const int n = EPI == MID_GATED ? t * n_out + n_lo0 + nb : n_lo0 + 16 * t + nb;
+                const int n_lim = EPI == MID_GATED ? t * n_out + n_out : p.N;
+                if (m >= p.M) continue;
+                float* dst = p.partial + ((size_t)blockIdx.y * p.M + m) * p.N + n;
+                if (vec && n + 3 < n_lim) { *reinterpret_cast<floatx4_t*>(dst) = acc[t][mt]; continue; }
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < n_lim) dst[r] = acc[t][mt][r];
+            }
+        return;
+    }
+    if constexpr (EPI == MID_STORE) {
+        TY* y = (TY*)p.y;
+        const bool vec = p.N % 4 == 0;
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int m = mt * 16 + row;
+                const int n = n_lo0 + 16 * t + nb;
+                if (m >= p.M) continue;
+                TY* dst = y + (size_t)m * p.N + n;
+                if (vec && n + 3 < p.N) {
+                    if constexpr (sizeof(TY) == 4) *reinterpret_cast<floatx4_t*>(dst) = acc[t][mt];
+                    else *reinterpret_cast<uint2*>(dst) = pack4_bf16(acc[t][mt][0], acc[t][mt][1], acc[t][mt][2], acc[t][mt][3]);
+                    continue;
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < p.N) dst[r] = from_float<TY>(acc[t][mt][r]);
+            }
+    } else {
+        bf16_t* y = (bf16_t*)p.y;
+        const bool vec = n_out % 4 == 0;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + row;
+            const int n = n_lo0 + nb;
+            if (m >= p.M) continue;
+            float o[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] = gate_times_up(acc[0][mt][r], acc[TN - 1][mt][r]);
+            bf16_t* dst = y + (size_t)m * n_out + n;
+            if (vec && n + 3 < n_out) { *reinterpret_cast<uint2*>(dst) = pack4_bf16(o[0], o[1], o[2], o[3]); continue; }
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n + r < n_out) dst[r] = from_float<bf16_t>(o[r]);
+        }
+    }
+}
+
+// Adds the splits' sums in split order and finishes as the product kernel does without splits.
+template <int EPI, typename TY>
+__global__ void mid_finish_kernel(const float* __restrict__ partial, void* __restrict__ yv, int splits, int M, int N) {
+    const int n_out = EPI == MID_GATED ? N / 2 : N;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)M * n_out) return;
+    const int m = (int)(i / n_out), n = (int)(i % n_out);
+    float a = 0.f, b = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float* src = partial + ((size_t)s * M + m) * N;
+        a += src[n];
+        if (EPI == MID_GATED) b += src[n_out + n];
+    }
+    if (EPI == MID_GATED) ((bf16_t*)yv)[i] = from_float<bf16_t>(gate_times_up(a, b));
+    else ((TY*)yv)[i] = from_float<TY>(a);
+}
+
+// How a product of this shape is cut: tiles per wave and splits of K.  From N and K alone.
+struct MidPlan { int tn, blocks, splits, k_per_split; };
+
+static MidPlan mid_plan(int N, int K, bool gated) {
+    MidPlan plan;
+    const int n_out = gated ? N / 2 : N;
+    const int tiles = (n_out + 15) / 16;
+    // two tiles per wave halve the reads of x from LDS, but also the blocks: only where many are left
+    plan.tn = gated ? 2 : (tiles >= 2 * MID_WAVES * 512 ? 2 : 1);
+    const int per_block = MID_WAVES * (gated ? 1 : plan.tn);
+    plan.blocks = (tiles + per_block - 1) / per_block;
+    // measured: about one block of 8 waves per compute unit streams fastest; no split shorter than 4 chunks
+    const int chunks = (K + MID_CHUNK - 1) / MID_CHUNK;
+    int splits = 256 / plan.blocks;
+    if (splits > chunks / 4) splits = chunks / 4;
+    if (splits < 1) splits = 1;
+    const int per = (chunks + splits - 1) / splits;
+    plan.splits = (chunks + per - 1) / per;             // no empty split
+    plan.k_per_split = per * MID_CHUNK;
+    return plan;
+}
+
+extern "C" size_t tqk_mid_scratch_bytes(int M, int N, int K, int gated) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const MidPlan plan = mid_plan(N, K, gated != 0);
+    return plan.splits > 1 ? (size_t)plan.splits * M * N * sizeof(float) : 0;
+}
+
+template <int MT, int TN, int EPI, typename TY>
+static int launch_mid(const MidArgs& a, const MidPlan& plan, hipStream_t s) {
+    dim3 grid(plan.blocks, plan.splits);
+    mid_product_kernel<MT, TN, EPI, TY><<<grid, MID_WAVES * TQK_WAVE, 2 * MT * 256 * 16, s>>>(a);
+    if (tqk_check_launch("tqk_mid product")) return -1;
+    if (plan.splits > 1) {
+        const size_t total = (size_t)a.M * (EPI == MID_GATED ? a.N / 2 : a.N);
+        mid_finish_kernel<EPI, TY><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(a.partial, a.y, plan.splits, a.M, a.N);
+        return tqk_check_launch("tqk_mid finish");
+    }
+    return 0;
+}
+
+template <int EPI, typename TY>
+static int launch_rows(const MidArgs& a, const MidPlan& plan, hipStream_t s) {
+    if constexpr (EPI == MID_GATED) {
+        return a.M > 32 ? launch_mid<4, 2, EPI, TY>(a, plan, s) : launch_mid<2, 2, EPI, TY>(a, plan, s);
+    } else {
+        if (a.M > 32) return plan.tn == 2 ? launch_mid<4, 2, EPI, TY>(a, plan, s) : launch_mid<4, 1, EPI, TY>(a, plan, s);
+        return plan.tn == 2 ? launch_mid<2, 2, EPI, TY>(a, plan, s) : launch_mid<2, 1, EPI, TY>(a, plan, s);
+    }
+}
+
+static int check_mid(const MidArgs& a, const void* scratch, bool gated, const char* what) {
+    TQK_REQUIRE(a.x && a.w && a.y, "%s: null pointer", what);
+    TQK_REQUIRE(a.M >= 0 && a.M <= MID_MAX_ROWS, "%s: M=%d rows, this kernel takes at most %d", what, a.M, MID_MAX_ROWS);
+    TQK_REQUIRE(a.N > 0 && a.K > 0 && a.K % 32 == 0, "%s: K=%d must be a positive multiple of 32 (N=%d)", what, a.K, a.N);
+    TQK_REQUIRE(!gated || a.N % 2 == 0, "%s: odd N=%d", what, a.N);
+    TQK_REQUIRE(((((uintptr_t)a.x) | ((uintptr_t)a.w) | ((uintptr_t)a.y) | ((uintptr_t)scratch)) & 15) == 0,
+                "%s: x, w, y and scratch must be 16-byte aligned", what);
+    TQK_REQUIRE(scratch || tqk_mid_scratch_bytes(a.M, a.N, a.K, gated) == 0, "%s: no scratch given", what);
+    return 0;
+}
+
+/* y[M,N] = x w^T, M <= 64, w packed; scratch: tqk_mid_scratch_bytes(M, N, K, 0) bytes. */
+extern "C" int tqk_mid_store(const void* x, const void* w_packed, void* y, int y_dtype, int M, int N, int K,
+                             void* scratch, void* stream) {
+    MidArgs a = {(const bf16_t*)x, (const bf16_t*)w_packed, y, (float*)scratch, M, N, K, 0};
+    if (check_mid(a, scratch, false, "tqk_mid_store")) return -1;
+    TQK_REQUIRE(y_dtype == TQK_F32 || y_dtype == TQK_BF16, "tqk_mid_store: unknown output dtype %d", y_dtype);
+    if (M == 0) return 0;
+    const MidPlan plan = mid_plan(N, K, false);
+    a.k_per_split = plan.k_per_split;
+    hipStream_t s = (hipStream_t)stream;
+    return y_dtype == TQK_F32 ? launch_rows<MID_STORE, float>(a, plan, s) : launch_rows<MID_STORE, bf16_t>(a, plan, s);
+}
+
+/* y[M, N/2] = silu(gate) * up, w = gate rows then up rows, packed in two parts. */
+extern "C" int tqk_mid_gated(const void* x, const void* w_packed, void* y, int M, int N, int K, void* scratch, void* stream) {
+    MidArgs a = {(const bf16_t*)x, (const bf16_t*)w_packed, y, (float*)scratch, M, N, K, 0};
+    if (check_mid(a, scratch, true, "tqk_mid_gated")) return -1;
+    if (M == 0) return 0;
+    const MidPlan plan = mid_plan(N, K, true);
+    a.k_per_split = plan.k_per_split;
+    return launch_rows<MID_GATED, bf16_t>(a, plan, (hipStream_t)stream);
+}

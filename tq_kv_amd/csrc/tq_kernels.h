@@ -66,6 +66,13 @@ int tqk_fused_qkv(const void* x, const float* ss_parts, int n_ss_parts, float ep
                   void* keys, void* values, int n_pages, void* q_out,
                   int M, int n_heads, int n_kv_heads, int head_dim, int K, void* stream);
 
+/* Products of up to 64 rows (bfloat16, K a multiple of 32) from the packed copy of the weight;
+ * scratch: tqk_mid_scratch_bytes(...) bytes of device memory, 16-byte aligned (0: none needed). */
+size_t tqk_mid_scratch_bytes(int M, int N, int K, int gated);
+int tqk_mid_store(const void* x, const void* w_packed, void* y, int y_dtype, int M, int N, int K, void* scratch, void* stream);
+/* y[M, N/2] = silu(gate) * up, w = gate rows then up rows, packed in two parts */
+int tqk_mid_gated(const void* x, const void* w_packed, void* y, int M, int N, int K, void* scratch, void* stream);
+
 /* For each token t and head: add bias, rotate q and k heads by the angle table row
  * tok_pos[t] (style 0: none, 1: halves (j, j+rot/2), 2: pairs (2j, 2j+1)), write q to
  * q_out [tokens, heads, head_dim] and, if write_kv, k and v into the pages of the

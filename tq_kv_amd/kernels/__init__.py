@@ -34,6 +34,7 @@ def library():
         lib.tqk_abi_version.restype = ctypes.c_int
         lib.tqk_sample_scratch_bytes.restype = ctypes.c_size_t
         lib.tqk_gemm_scratch_bytes.restype = ctypes.c_size_t
+        lib.tqk_mid_scratch_bytes.restype = ctypes.c_size_t
         _LIB = lib
     return _LIB
 
@@ -358,6 +359,40 @@ def fused_gated(x, weight_gate_up, out, norm=None):
         _dev(x, "x", torch.bfloat16, (m, k)), ss, n_parts, eps,
         w, packed, _dev(out, "out", torch.bfloat16), m, 2 * inter, k,
         _stream()), "fused_gated")
+    return out
+
+
+MID_MAX_ROWS = 64
+
+
+def _mid_scratch(m, n, k, gated, device):
+    need = int(library().tqk_mid_scratch_bytes(m, n, k, 1 if gated else 0))
+    return torch.empty((need,), dtype=torch.uint8, device=device) if need else None
+
+
+def mid_store(x, weight, out):
+    """out[M,N] = x weight^T for up to 64 rows of bfloat16; weight: a PackedWeight."""
+    m, n = out.shape
+    k = x.shape[1]
+    if not isinstance(weight, PackedWeight):
+        raise KernelError("mid_store: the weight must be packed (pack_weight)")
+    w, _ = _weight(weight, "weight", n, k)
+    scratch = _mid_scratch(m, n, k, False, x.device)
+    _check(library().tqk_mid_store(_dev(x, "x", torch.bfloat16, (m, k)), w, _dev(out, "out"), _code(out.dtype), m, n, k,
+                                   _opt(scratch, "scratch"), _stream()), "mid_store")
+    return out
+
+
+def mid_gated(x, weight_gate_up, out):
+    """out[M, I] = silu(gate) * up of x [gate; up]^T for up to 64 rows; weight: a PackedWeight in 2 parts."""
+    m, inter = out.shape
+    k = x.shape[1]
+    if not isinstance(weight_gate_up, PackedWeight):
+        raise KernelError("mid_gated: the weight must be packed (pack_weight with parts=2)")
+    w, _ = _weight(weight_gate_up, "weight", 2 * inter, k, parts=2)
+    scratch = _mid_scratch(m, 2 * inter, k, True, x.device)
+    _check(library().tqk_mid_gated(_dev(x, "x", torch.bfloat16, (m, k)), w, _dev(out, "out", torch.bfloat16), m, 2 * inter, k,
+                                   _opt(scratch, "scratch"), _stream()), "mid_gated")
     return out
 
 

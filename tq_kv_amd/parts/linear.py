@@ -11,6 +11,9 @@ The reference's linear layers are candle matmuls, i.e. library GEMMs
            It reads a second copy of the weight, packed at loading time in the order its
            lanes take it (few_rows_form): a decoding step is bound by the weight bytes, and
            in that order they stream faster.
+  bfloat16, 17 to 64 rows (decoding steps of larger batches) where the weight has a packed copy
+        -> the hand-written kernel that stages x in LDS and streams the packed weights
+           (kernels.mid_store, kernels.mid_gated)
   bfloat16, more rows (prompts, large decoding batches)
         -> the library GEMM (hipBLASLt through torch), float32 accumulation; float32
            output where logits are wanted
@@ -22,10 +25,12 @@ from .. import kernels as K
 # The bfloat16 routines can be switched off one by one (tests compare each with the
 # plain kernel); nothing else reads these.
 # Measured on MI355X at the Qwen2.5-7B sizes: up to 16 rows the skinny kernel is ahead of the
-# library on every product; at 64 rows the library is ahead on every one.
+# library on every product; at 64 rows the library is ahead of it on every one, and the kernel
+# for 17 to 64 rows ("mid") ahead of the library.
 # "packed": parts keep the second, packed copy of their weights for the few-row kernels (twice
 # the weight memory, about an eighth less time per decoding step).
-POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16, "fused": True, "prune_last": True, "packed": True}
+POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16, "fused": True, "prune_last": True, "packed": True,
+          "mid": True}
 
 
 class Stream:
@@ -106,6 +111,11 @@ def _skinny_ok(x, weight):
             and x.shape[1] % 32 == 0 and x.shape[0] <= POLICY["skinny_max_rows"])
 
 
+def _mid_ok(x, weight, few):
+    return (POLICY["mid"] and few is not None and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+            and POLICY["skinny_max_rows"] < x.shape[0] <= K.MID_MAX_ROWS)
+
+
 def gated_silu_linear(x, weight_gate_up, few=None):
     """silu(x Wg^T) * (x Wu^T) with Wg stacked on Wu: [M, K] x [2I, K] -> [M, I].  For few
     rows of bfloat16 the gate and the up row of an output are computed by the same wave
@@ -116,6 +126,8 @@ def gated_silu_linear(x, weight_gate_up, few=None):
     act = torch.empty((m, inter), dtype=x.dtype, device=x.device)
     if _skinny_ok(x, weight_gate_up):
         return K.fused_gated(x, few or weight_gate_up, act)
+    if _mid_ok(x, weight_gate_up, few):
+        return K.mid_gated(x, few, act)
     return K.swiglu(linear(x, weight_gate_up), act)
 
 
@@ -132,6 +144,9 @@ def linear(x, weight, bias=None, out_dtype=None, few=None):
         if _skinny_ok(x, weight):
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
             return K.fused_store(x, few or weight, out)
+        if _mid_ok(x, weight, few):
+            out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+            return K.mid_store(x, few, out)
         if POLICY["library"] and m > POLICY["skinny_max_rows"]:
             if out_dtype == torch.bfloat16:
                 return torch.matmul(x, weight.t())
