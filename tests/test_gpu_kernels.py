@@ -28,7 +28,7 @@ def ints(values):
 
 
 def test_library_is_built_and_loaded():
-    assert K.library().tqk_abi_version() == 6
+    assert K.library().tqk_abi_version() == 7
     assert K.library_path().endswith(".so")
     with pytest.raises(K.KernelError, match="GPU only"):
         K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
@@ -505,6 +505,30 @@ def test_gated_product_of_17_to_64_rows(m, inter, k):
     act = torch.empty_like(out)
     K.swiglu(both, act)
     torch.testing.assert_close(out.float(), act.float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("m,n,k", [(40, 96, 2048), (64, 3584, 3584), (17, 100, 1056), (33, 2050, 1024)])
+def test_unfinished_sums_of_a_product_are_finished_by_the_next_norm(m, n, k):
+    x, w = rand(m, k, seed=36, dtype=torch.bfloat16), rand(n, k, seed=37, scale=0.05, dtype=torch.bfloat16)
+    packed = K.pack_weight(w)
+    nw = (1 + rand(n, seed=38, scale=0.1)).to(torch.bfloat16)
+    h = rand(m, n, seed=39, scale=2.0)
+    done = K.mid_store(x, packed, torch.empty(m, n, dtype=torch.bfloat16, device=DEV))
+    left = K.mid_store(x, packed, torch.empty(m, n, dtype=torch.bfloat16, device=DEV), finish=False)
+    assert isinstance(left, K.PartialSums) and left.sums.shape[0] > 1 and left.shape == (m, n)     # these shapes are cut
+    h1, h2 = h.clone(), h.clone()
+    out1 = K.add_rmsnorm(h1, done, nw, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV), write_back=True)
+    out2 = K.add_rmsnorm(h2, left, nw, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV), write_back=True)
+    assert torch.equal(h1, h2) and torch.equal(out1, out2)
+    torch.testing.assert_close(h1, h + done.float(), atol=0, rtol=0)
+    # some rows only, h left as it is; and without a stream
+    rows = ints([m - 1, 0, 5])
+    g1 = K.add_rmsnorm(h, done, nw, 1e-6, torch.empty(3, n, dtype=torch.bfloat16, device=DEV), rows=rows)
+    g2 = K.add_rmsnorm(h, left, nw, 1e-6, torch.empty(3, n, dtype=torch.bfloat16, device=DEV), rows=rows)
+    assert torch.equal(g1, g2)
+    n1 = K.add_rmsnorm(None, done, nw, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV))
+    n2 = K.add_rmsnorm(None, left, nw, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV))
+    assert torch.equal(n1, n2)
 
 
 def test_products_of_17_to_64_rows_refuse_what_they_do_not_take():

@@ -102,8 +102,22 @@ extern "C" int tqk_embed(const void* table, int table_dtype, const int32_t* ids,
 // ---- residual add + RMSNorm -----------------------------------------------------
 // y = x / sqrt(mean(x^2) + eps) * w in float32, cast last, as
 // src/models/turbo_generic.rs:41-51 does (division by the root, weight inside).
+//
+// The update can also come as a product's unfinished sums: float32 [n_sums][rows][hidden], the
+// sums of the product over n_sums pieces of its K (mid_product.hip).  They are added up in their
+// order and rounded to the activation type, as the finished product would have been, and then
+// added as any other update: the product's own finishing pass and its round trip disappear.
+struct PartSums { const float* sums; int n; size_t stride; };       // stride: rows * hidden
+
+template <typename TA>
+__device__ __forceinline__ float summed(const PartSums& ps, size_t at) {
+    float a = 0.f;
+    for (int s = 0; s < ps.n; ++s) a += ps.sums[(size_t)s * ps.stride + at];
+    return to_float(from_float<TA>(a));
+}
+
 template <typename TA, typename TW>
-__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__ delta,
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__ delta, const PartSums ps,
                                    const TW* __restrict__ weight, float eps,
                                    const int32_t* __restrict__ rows, int hidden,
                                    TA* __restrict__ out, int write_back) {
@@ -114,8 +128,14 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__
     const TA* dr = delta ? delta + row * hidden : nullptr;
     TA* o = out + (size_t)r * hidden;
     float ss = 0.f;
+    auto value = [&](int i) {
+        float v = hr ? hr[i] : 0.f;
+        if (dr) v += to_float(dr[i]);
+        if (ps.sums) v += summed<TA>(ps, row * hidden + i);
+        return v;
+    };
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-        float v = (hr ? hr[i] : 0.f) + (dr ? to_float(dr[i]) : 0.f);
+        const float v = value(i);
         if (write_back) hr[i] = v;
         ss += v * v;
     }
@@ -123,7 +143,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TA* __restrict__
     const float rms = sqrtf(total / (float)hidden + eps);
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         // the same thread wrote h[i] above, so with write_back the value is read back exactly
-        float v = write_back ? hr[i] : ((hr ? hr[i] : 0.f) + (dr ? to_float(dr[i]) : 0.f));
+        const float v = write_back ? hr[i] : value(i);
         o[i] = from_float<TA>((v / rms) * to_float(weight[i]));
     }
 }
@@ -148,7 +168,7 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float a, f
 }
 
 template <typename TA, typename TW, int VPT>
-__global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TA* __restrict__ delta,
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TA* __restrict__ delta, const PartSums ps,
                                        const TW* __restrict__ weight, float eps,
                                        const int32_t* __restrict__ rows, int hidden,
                                        TA* __restrict__ out, int write_back) {
@@ -170,6 +190,24 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TA* __restri
                 d.v = *reinterpret_cast<const decltype(d.v)*>(dr + i);
                 hv.x += d.get(0); hv.y += d.get(1); hv.z += d.get(2); hv.w += d.get(3);
             }
+            if (ps.sums) {
+                float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+                const float* at = ps.sums + row * hidden + i;
+                int s = 0;
+                for (; s + 4 <= ps.n; s += 4) {             // four loads under way together, added in order
+                    float4 part[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) part[u] = *reinterpret_cast<const float4*>(at + (size_t)(s + u) * ps.stride);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) { a.x += part[u].x; a.y += part[u].y; a.z += part[u].z; a.w += part[u].w; }
+                }
+                for (; s < ps.n; ++s) {
+                    const float4 part = *reinterpret_cast<const float4*>(at + (size_t)s * ps.stride);
+                    a.x += part.x; a.y += part.y; a.z += part.z; a.w += part.w;
+                }
+                hv.x += to_float(from_float<TA>(a.x)); hv.y += to_float(from_float<TA>(a.y));
+                hv.z += to_float(from_float<TA>(a.z)); hv.w += to_float(from_float<TA>(a.w));
+            }
             if (write_back) *reinterpret_cast<float4*>(hr + i) = hv;
             v[j][0] = hv.x; v[j][1] = hv.y; v[j][2] = hv.z; v[j][3] = hv.w;
             ss += hv.x * hv.x + hv.y * hv.y + hv.z * hv.z + hv.w * hv.w;
@@ -189,25 +227,27 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TA* __restri
     }
 }
 
-extern "C" int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const void* weight,
-                               int weight_dtype, float eps, const int32_t* rows, int n_rows,
-                               int hidden, void* out, int write_back, void* stream) {
+static int add_rmsnorm(float* h, const void* delta, const PartSums ps, int act_dtype, const void* weight,
+                       int weight_dtype, float eps, const int32_t* rows, int n_rows,
+                       int hidden, void* out, int write_back, void* stream) {
     TQK_REQUIRE(weight && out, "tqk_add_rmsnorm: null pointer");
-    TQK_REQUIRE(h || delta, "tqk_add_rmsnorm: neither h nor delta given");
+    TQK_REQUIRE(h || delta || ps.sums, "tqk_add_rmsnorm: neither h nor an update given");
     TQK_REQUIRE(!write_back || (h && !rows), "tqk_add_rmsnorm: write_back needs h and no row list");
     TQK_REQUIRE(n_rows >= 0 && hidden > 0, "tqk_add_rmsnorm: bad sizes rows=%d hidden=%d", n_rows, hidden);
     TQK_REQUIRE(act_dtype == TQK_F32 || act_dtype == TQK_BF16, "tqk_add_rmsnorm: unknown activation dtype %d", act_dtype);
     TQK_REQUIRE(weight_dtype == TQK_F32 || weight_dtype == TQK_BF16, "tqk_add_rmsnorm: unknown weight dtype %d", weight_dtype);
     if (n_rows == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    const bool aligned = ((((uintptr_t)h) | ((uintptr_t)delta) | ((uintptr_t)weight) | ((uintptr_t)out)) & 15) == 0;
+    const bool aligned = ((((uintptr_t)h) | ((uintptr_t)delta) | ((uintptr_t)weight) | ((uintptr_t)out) | ((uintptr_t)ps.sums)) & 15) == 0;
     const int code = act_dtype * 2 + weight_dtype;
     if (hidden % 4 == 0 && hidden <= 8192 && aligned) {
-        const int threads = 256;
+        // sums of a product: several times the bytes per row, and few rows: more threads per row
+        const int threads = ps.sums ? 1024 : 256;
 #define LAUNCHV(TA, TW, VPT) add_rmsnorm_vec_kernel<TA, TW, VPT><<<n_rows, threads, 0, s>>>( \
-        h, (const TA*)delta, (const TW*)weight, eps, rows, hidden, (TA*)out, write_back)
-#define PICK(TA, TW) do { if (hidden <= 1024) LAUNCHV(TA, TW, 1); else if (hidden <= 2048) LAUNCHV(TA, TW, 2); \
-        else if (hidden <= 4096) LAUNCHV(TA, TW, 4); else LAUNCHV(TA, TW, 8); } while (0)
+        h, (const TA*)delta, ps, (const TW*)weight, eps, rows, hidden, (TA*)out, write_back)
+#define PICK(TA, TW) do { const int per = (hidden + threads * 4 - 1) / (threads * 4); \
+        if (per <= 1) LAUNCHV(TA, TW, 1); else if (per <= 2) LAUNCHV(TA, TW, 2); \
+        else if (per <= 4) LAUNCHV(TA, TW, 4); else LAUNCHV(TA, TW, 8); } while (0)
         switch (code) {
             case 0: PICK(float, float); break;
             case 1: PICK(float, bf16_t); break;
@@ -220,7 +260,7 @@ extern "C" int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const
     }
     const int threads = hidden >= 2048 ? 512 : 256;
 #define LAUNCH(TA, TW) add_rmsnorm_kernel<TA, TW><<<n_rows, threads, 0, s>>>( \
-        h, (const TA*)delta, (const TW*)weight, eps, rows, hidden, (TA*)out, write_back)
+        h, (const TA*)delta, ps, (const TW*)weight, eps, rows, hidden, (TA*)out, write_back)
     switch (code) {
         case 0: LAUNCH(float, float); break;
         case 1: LAUNCH(float, bf16_t); break;
@@ -229,6 +269,23 @@ extern "C" int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const
     }
 #undef LAUNCH
     return tqk_check_launch("tqk_add_rmsnorm");
+}
+
+extern "C" int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const void* weight,
+                               int weight_dtype, float eps, const int32_t* rows, int n_rows,
+                               int hidden, void* out, int write_back, void* stream) {
+    return add_rmsnorm(h, delta, PartSums{nullptr, 0, 0}, act_dtype, weight, weight_dtype, eps, rows, n_rows, hidden, out,
+                       write_back, stream);
+}
+
+/* The same with the update given as a product's sums over n_sums pieces of its K, float32
+ * [n_sums][sum_rows][hidden] (row r of the update is row rows[r], or r, of each piece). */
+extern "C" int tqk_add_rmsnorm_sums(float* h, const float* sums, int n_sums, int sum_rows, int act_dtype, const void* weight,
+                                    int weight_dtype, float eps, const int32_t* rows, int n_rows,
+                                    int hidden, void* out, int write_back, void* stream) {
+    TQK_REQUIRE(sums && n_sums > 0 && sum_rows > 0, "tqk_add_rmsnorm_sums: no sums given");
+    return add_rmsnorm(h, nullptr, PartSums{sums, n_sums, (size_t)sum_rows * hidden}, act_dtype, weight, weight_dtype, eps,
+                       rows, n_rows, hidden, out, write_back, stream);
 }
 
 // ---- bias + rotation + cache write ------------------------------------------------

@@ -255,18 +255,23 @@ static MidPlan mid_plan(int N, int K, bool gated) {
     return plan;
 }
 
-extern "C" size_t tqk_mid_scratch_bytes(int M, int N, int K, int gated) {
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
-    const MidPlan plan = mid_plan(N, K, gated != 0);
-    return plan.splits > 1 ? (size_t)plan.splits * M * N * sizeof(float) : 0;
+/* Into how many pieces the product's K is cut (1: none, no scratch is needed). */
+extern "C" int tqk_mid_splits(int N, int K, int gated) {
+    if (N <= 0 || K <= 0) return 1;
+    return mid_plan(N, K, gated != 0).splits;
+}
+
+static size_t mid_scratch_bytes(int M, int N, int K, bool gated) {
+    const int splits = tqk_mid_splits(N, K, gated);
+    return splits > 1 && M > 0 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 
 template <int MT, int TN, int EPI, typename TY>
-static int launch_mid(const MidArgs& a, const MidPlan& plan, hipStream_t s) {
+static int launch_mid(const MidArgs& a, const MidPlan& plan, bool finish, hipStream_t s) {
     dim3 grid(plan.blocks, plan.splits);
     mid_product_kernel<MT, TN, EPI, TY><<<grid, MID_WAVES * TQK_WAVE, 2 * MT * 256 * 16, s>>>(a);
     if (tqk_check_launch("tqk_mid product")) return -1;
-    if (plan.splits > 1) {
+    if (plan.splits > 1 && finish) {
         const size_t total = (size_t)a.M * (EPI == MID_GATED ? a.N / 2 : a.N);
         mid_finish_kernel<EPI, TY><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(a.partial, a.y, plan.splits, a.M, a.N);
         return tqk_check_launch("tqk_mid finish");
@@ -275,45 +280,49 @@ static int launch_mid(const MidArgs& a, const MidPlan& plan, hipStream_t s) {
 }
 
 template <int EPI, typename TY>
-static int launch_rows(const MidArgs& a, const MidPlan& plan, hipStream_t s) {
+static int launch_rows(const MidArgs& a, const MidPlan& plan, bool finish, hipStream_t s) {
     if constexpr (EPI == MID_GATED) {
-        return a.M > 32 ? launch_mid<4, 2, EPI, TY>(a, plan, s) : launch_mid<2, 2, EPI, TY>(a, plan, s);
+        return a.M > 32 ? launch_mid<4, 2, EPI, TY>(a, plan, finish, s) : launch_mid<2, 2, EPI, TY>(a, plan, finish, s);
     } else {
-        if (a.M > 32) return plan.tn == 2 ? launch_mid<4, 2, EPI, TY>(a, plan, s) : launch_mid<4, 1, EPI, TY>(a, plan, s);
-        return plan.tn == 2 ? launch_mid<2, 2, EPI, TY>(a, plan, s) : launch_mid<2, 1, EPI, TY>(a, plan, s);
+        if (a.M > 32) return plan.tn == 2 ? launch_mid<4, 2, EPI, TY>(a, plan, finish, s) : launch_mid<4, 1, EPI, TY>(a, plan, finish, s);
+        return plan.tn == 2 ? launch_mid<2, 2, EPI, TY>(a, plan, finish, s) : launch_mid<2, 1, EPI, TY>(a, plan, finish, s);
     }
 }
 
-static int check_mid(const MidArgs& a, const void* scratch, bool gated, const char* what) {
-    TQK_REQUIRE(a.x && a.w && a.y, "%s: null pointer", what);
+static int check_mid(const MidArgs& a, const void* scratch, bool gated, bool finish, const char* what) {
+    TQK_REQUIRE(a.x && a.w, "%s: null pointer", what);
+    TQK_REQUIRE(a.y || (!finish && tqk_mid_splits(a.N, a.K, gated) > 1), "%s: null output", what);
     TQK_REQUIRE(a.M >= 0 && a.M <= MID_MAX_ROWS, "%s: M=%d rows, this kernel takes at most %d", what, a.M, MID_MAX_ROWS);
     TQK_REQUIRE(a.N > 0 && a.K > 0 && a.K % 32 == 0, "%s: K=%d must be a positive multiple of 32 (N=%d)", what, a.K, a.N);
     TQK_REQUIRE(!gated || a.N % 2 == 0, "%s: odd N=%d", what, a.N);
     TQK_REQUIRE(((((uintptr_t)a.x) | ((uintptr_t)a.w) | ((uintptr_t)a.y) | ((uintptr_t)scratch)) & 15) == 0,
                 "%s: x, w, y and scratch must be 16-byte aligned", what);
-    TQK_REQUIRE(scratch || tqk_mid_scratch_bytes(a.M, a.N, a.K, gated) == 0, "%s: no scratch given", what);
+    TQK_REQUIRE(scratch || mid_scratch_bytes(a.M, a.N, a.K, gated) == 0, "%s: no scratch given", what);
     return 0;
 }
 
-/* y[M,N] = x w^T, M <= 64, w packed; scratch: tqk_mid_scratch_bytes(M, N, K, 0) bytes. */
+/* y[M,N] = x w^T, M <= 64, w packed; scratch: float32 [tqk_mid_splits(N, K, 0)][M][N] where that
+ * is more than 1.  finish == 0: with more than one piece the pieces' sums are left in scratch
+ * (for tqk_add_rmsnorm_sums) and y is not written. */
 extern "C" int tqk_mid_store(const void* x, const void* w_packed, void* y, int y_dtype, int M, int N, int K,
-                             void* scratch, void* stream) {
+                             void* scratch, int finish, void* stream) {
     MidArgs a = {(const bf16_t*)x, (const bf16_t*)w_packed, y, (float*)scratch, M, N, K, 0};
-    if (check_mid(a, scratch, false, "tqk_mid_store")) return -1;
+    if (check_mid(a, scratch, false, finish != 0, "tqk_mid_store")) return -1;
     TQK_REQUIRE(y_dtype == TQK_F32 || y_dtype == TQK_BF16, "tqk_mid_store: unknown output dtype %d", y_dtype);
     if (M == 0) return 0;
     const MidPlan plan = mid_plan(N, K, false);
     a.k_per_split = plan.k_per_split;
     hipStream_t s = (hipStream_t)stream;
-    return y_dtype == TQK_F32 ? launch_rows<MID_STORE, float>(a, plan, s) : launch_rows<MID_STORE, bf16_t>(a, plan, s);
+    return y_dtype == TQK_F32 ? launch_rows<MID_STORE, float>(a, plan, finish != 0, s)
+                              : launch_rows<MID_STORE, bf16_t>(a, plan, finish != 0, s);
 }
 
 /* y[M, N/2] = silu(gate) * up, w = gate rows then up rows, packed in two parts. */
 extern "C" int tqk_mid_gated(const void* x, const void* w_packed, void* y, int M, int N, int K, void* scratch, void* stream) {
     MidArgs a = {(const bf16_t*)x, (const bf16_t*)w_packed, y, (float*)scratch, M, N, K, 0};
-    if (check_mid(a, scratch, true, "tqk_mid_gated")) return -1;
+    if (check_mid(a, scratch, true, true, "tqk_mid_gated")) return -1;
     if (M == 0) return 0;
     const MidPlan plan = mid_plan(N, K, true);
     a.k_per_split = plan.k_per_split;
-    return launch_rows<MID_GATED, bf16_t>(a, plan, (hipStream_t)stream);
+    return launch_rows<MID_GATED, bf16_t>(a, plan, true, (hipStream_t)stream);
 }

@@ -32,6 +32,12 @@ int tqk_embed(const void* table, int table_dtype, const int32_t* ids, int n_toke
 int tqk_add_rmsnorm(float* h, const void* delta, int act_dtype, const void* weight,
                     int weight_dtype, float eps, const int32_t* rows, int n_rows,
                     int hidden, void* out, int write_back, void* stream);
+/* the same, the update being a product's sums over n_sums pieces of its K (tqk_mid_store with
+ * finish == 0): float32 [n_sums][sum_rows][hidden], added up in order and rounded to the
+ * activation type first */
+int tqk_add_rmsnorm_sums(float* h, const float* sums, int n_sums, int sum_rows, int act_dtype, const void* weight,
+                         int weight_dtype, float eps, const int32_t* rows, int n_rows,
+                         int hidden, void* out, int write_back, void* stream);
 
 /* y[M,N] = x[M,K] w[N,K]^T (+ bias[N]); float32 accumulation in a fixed order that
  * does not depend on M.  Any sizes.  scratch: tqk_gemm_scratch_bytes(...) bytes of device
@@ -66,10 +72,13 @@ int tqk_fused_qkv(const void* x, const float* ss_parts, int n_ss_parts, float ep
                   void* keys, void* values, int n_pages, void* q_out,
                   int M, int n_heads, int n_kv_heads, int head_dim, int K, void* stream);
 
-/* Products of up to 64 rows (bfloat16, K a multiple of 32) from the packed copy of the weight;
- * scratch: tqk_mid_scratch_bytes(...) bytes of device memory, 16-byte aligned (0: none needed). */
-size_t tqk_mid_scratch_bytes(int M, int N, int K, int gated);
-int tqk_mid_store(const void* x, const void* w_packed, void* y, int y_dtype, int M, int N, int K, void* scratch, void* stream);
+/* Products of up to 64 rows (bfloat16, K a multiple of 32) from the packed copy of the weight.
+ * K is cut into tqk_mid_splits(N, K, gated) pieces; where that is more than 1, scratch is
+ * float32 [pieces][M][N], 16-byte aligned.  finish == 0: with more than one piece the pieces'
+ * sums stay in scratch (tqk_add_rmsnorm_sums adds them up) and y is not written. */
+int tqk_mid_splits(int N, int K, int gated);
+int tqk_mid_store(const void* x, const void* w_packed, void* y, int y_dtype, int M, int N, int K, void* scratch,
+                  int finish, void* stream);
 /* y[M, N/2] = silu(gate) * up, w = gate rows then up rows, packed in two parts */
 int tqk_mid_gated(const void* x, const void* w_packed, void* y, int M, int N, int K, void* scratch, void* stream);
 

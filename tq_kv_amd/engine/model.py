@@ -145,6 +145,9 @@ class Model:
         # small decoding steps: products fold the norms and the residual sums around them in
         ctx.fuse_small = (L.POLICY["fused"] and self.dtype == torch.bfloat16 and ctx.all_decode
                           and ctx.n_tokens <= 16 and s.hidden_size % 32 == 0)
+        # steps of 17 to 64 tokens: a part's last product may leave its sums to the next norm's kernel
+        ctx.fuse_mid = (L.POLICY["mid"] and self.dtype == torch.bfloat16
+                        and L.POLICY["skinny_max_rows"] < ctx.n_tokens <= K.MID_MAX_ROWS)
         # the norm that reads the stream first in every run, and after the last one
         firsts = [self.blocks[run.layer].first_norm() for run in s.order] + [self.final_norm]
         if ctx.fuse_small:

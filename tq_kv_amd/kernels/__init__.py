@@ -34,7 +34,6 @@ def library():
         lib.tqk_abi_version.restype = ctypes.c_int
         lib.tqk_sample_scratch_bytes.restype = ctypes.c_size_t
         lib.tqk_gemm_scratch_bytes.restype = ctypes.c_size_t
-        lib.tqk_mid_scratch_bytes.restype = ctypes.c_size_t
         _LIB = lib
     return _LIB
 
@@ -99,13 +98,24 @@ def embed(table, ids, out, copy=None, copy_weight=None, ss_out=None):
 def add_rmsnorm(h, delta, weight, eps, out, rows=None, write_back=False):
     """out = rmsnorm(h + delta) * weight; with write_back h becomes h + delta.
 
-    h: [T,H] float32 or None.  delta: [T,H] of out's dtype or None.  rows: int32 row
-    indices (then out has one row per index) or None for all rows."""
+    h: [T,H] float32 or None.  delta: [T,H] of out's dtype, a product's PartialSums, or None.
+    rows: int32 row indices (then out has one row per index) or None for all rows."""
     hidden = weight.shape[0]
     n_rows = out.shape[0]
     src_rows = (h if h is not None else delta).shape[0]
     if rows is None and src_rows != n_rows:
         raise KernelError("add_rmsnorm: %d input rows but %d output rows" % (src_rows, n_rows))
+    if isinstance(delta, PartialSums):
+        pieces = delta.sums.shape[0]
+        if delta.dtype != out.dtype or tuple(delta.shape) != (src_rows, hidden):
+            raise KernelError("add_rmsnorm: the update's sums are %s of %s, wanted %s of %s"
+                              % (delta.shape, delta.dtype, (src_rows, hidden), out.dtype))
+        _check(library().tqk_add_rmsnorm_sums(
+            _opt(h, "h", torch.float32, (src_rows, hidden)), _dev(delta.sums, "sums", torch.float32), pieces, src_rows,
+            _code(out.dtype), _dev(weight, "weight", None, (hidden,)), _code(weight.dtype), ctypes.c_float(eps),
+            _opt(rows, "rows", torch.int32, (n_rows,)), n_rows, hidden, _dev(out, "out", None, (n_rows, hidden)),
+            1 if write_back else 0, _stream()), "add_rmsnorm")
+        return out
     _check(library().tqk_add_rmsnorm(
         _opt(h, "h", torch.float32, (src_rows, hidden)), _opt(delta, "delta", out.dtype, (src_rows, hidden)),
         _code(out.dtype), _dev(weight, "weight", None, (hidden,)), _code(weight.dtype), ctypes.c_float(eps),
@@ -365,22 +375,41 @@ def fused_gated(x, weight_gate_up, out, norm=None):
 MID_MAX_ROWS = 64
 
 
+class PartialSums:
+    """A product [rows, n] that has not been added up: sums float32 [pieces, rows, n] over pieces
+    of its K.  add_rmsnorm takes it as the update (adds the pieces in order, rounds to `dtype`
+    as the finished product would be)."""
+
+    def __init__(self, sums, dtype):
+        self.sums, self.dtype = sums, dtype
+        self.shape = tuple(sums.shape[1:])
+
+
 def _mid_scratch(m, n, k, gated, device):
-    need = int(library().tqk_mid_scratch_bytes(m, n, k, 1 if gated else 0))
-    return torch.empty((need,), dtype=torch.uint8, device=device) if need else None
+    splits = int(library().tqk_mid_splits(n, k, 1 if gated else 0))
+    return torch.empty((splits, m, n), dtype=torch.float32, device=device) if splits > 1 else None
 
 
-def mid_store(x, weight, out):
-    """out[M,N] = x weight^T for up to 64 rows of bfloat16; weight: a PackedWeight."""
-    m, n = out.shape
-    k = x.shape[1]
+def mid_store(x, weight, out=None, finish=True):
+    """out[M,N] = x weight^T for up to 64 rows of bfloat16; weight: a PackedWeight.  finish=False:
+    where the kernel cuts K into pieces, their PartialSums (of out's dtype, which need not be
+    given then: bfloat16) are returned in place of out."""
+    m, k = x.shape
     if not isinstance(weight, PackedWeight):
         raise KernelError("mid_store: the weight must be packed (pack_weight)")
+    n = weight.shape[0]
     w, _ = _weight(weight, "weight", n, k)
     scratch = _mid_scratch(m, n, k, False, x.device)
-    _check(library().tqk_mid_store(_dev(x, "x", torch.bfloat16, (m, k)), w, _dev(out, "out"), _code(out.dtype), m, n, k,
-                                   _opt(scratch, "scratch"), _stream()), "mid_store")
-    return out
+    leave = not finish and scratch is not None
+    if out is None:
+        if not leave:
+            raise KernelError("mid_store: no output given")
+        dtype = torch.bfloat16
+    else:
+        dtype = out.dtype
+    _check(library().tqk_mid_store(_dev(x, "x", torch.bfloat16, (m, k)), w, _opt(None if leave else out, "out", None, (m, n)),
+                                   _code(dtype), m, n, k, _opt(scratch, "scratch"), 0 if leave else 1, _stream()), "mid_store")
+    return PartialSums(scratch, dtype) if leave else out
 
 
 def mid_gated(x, weight_gate_up, out):

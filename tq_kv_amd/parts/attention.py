@@ -11,7 +11,7 @@ import math
 import torch
 
 from .. import kernels as K
-from .linear import LazyNorm, few_rows_form, fusable, linear
+from .linear import LazyNorm, few_rows_form, fusable, leaves_sums, linear
 from .registry import Part, register
 from .spec import KVNeed, TensorSpec
 
@@ -94,7 +94,7 @@ class Attention(Part):
         return self._fused_qkv_ok(ctx) and not self.reads_other_cache
 
     def adds_to_stream(self, ctx):
-        return fusable(ctx.n_tokens, self.w_o, adds=True) and self.b_o is None
+        return self.b_o is None and (fusable(ctx.n_tokens, self.w_o, adds=True) or leaves_sums(ctx.n_tokens, self.w_o, self.few_o))
 
     def forward(self, x, ctx, entry, stream=None, last_rows=False):
         """x: the (normed) step [tokens, hidden], or a LazyNorm of it.  stream: add the output to

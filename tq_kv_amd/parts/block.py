@@ -5,7 +5,9 @@ x = x + mixer(norm(x)); x = x + ff(norm(x)), with optional norms on the mixer's 
 the feed-forward's outputs (:1965-1968, :1976-1979).
 
 The residual stream is float32 (parts.linear.Stream).  A part's output is left pending
-on the stream and added inside the next norm's kernel.  In small decoding steps the
+on the stream and added inside the next norm's kernel (for steps of 17 to 64 tokens a
+part's last product may even leave its sums over pieces of K pending: the norm's kernel
+adds those up too).  In small decoding steps the
 framework's parts go further: a product that consumes a norm computes it itself
 (LazyNorm) and a part's last product adds its result to the stream in its epilogue, so
 that the norm kernels disappear; parts that do not offer this (`folds_norm`,
@@ -80,7 +82,8 @@ class PreNormBlock(Part):
     def _run(self, part, post_norm, next_norm, x, stream, ctx, *extra):
         """Run a part; its output is added to the stream by the part itself (it returns None)
         or is left pending for the next norm's kernel."""
-        if ctx.fuse_small and post_norm is None and getattr(part, "adds_to_stream", None) and part.adds_to_stream(ctx):
+        if ((ctx.fuse_small or getattr(ctx, "fuse_mid", False)) and post_norm is None
+                and getattr(part, "adds_to_stream", None) and part.adds_to_stream(ctx)):
             stream.next_norm = next_norm
             out = part.forward(x, ctx, *extra, stream=stream)
         else:

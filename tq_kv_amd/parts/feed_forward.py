@@ -4,7 +4,7 @@ up are one product with the weights stacked."""
 import torch
 
 from .. import kernels as K
-from .linear import LazyNorm, few_rows_form, fusable, gated_silu_linear, linear
+from .linear import LazyNorm, few_rows_form, fusable, gated_silu_linear, leaves_sums, linear
 from .registry import Part, register
 from .spec import TensorSpec
 
@@ -40,10 +40,14 @@ class GatedSiLU(Part):
         return fusable(ctx.n_tokens, self.w_gate_up)
 
     def adds_to_stream(self, ctx):
-        return fusable(ctx.n_tokens, self.w_down, adds=True) and fusable(ctx.n_tokens, self.w_gate_up)
+        return ((fusable(ctx.n_tokens, self.w_down, adds=True) and fusable(ctx.n_tokens, self.w_gate_up))
+                or leaves_sums(ctx.n_tokens, self.w_down, self.few_down))
 
     def forward(self, x, ctx, stream=None):
         lazy = isinstance(x, LazyNorm)
+        if stream is not None and not lazy and x.shape[0] > 16:
+            stream.add_product(gated_silu_linear(x, self.w_gate_up, self.few_gate_up), self.few_down)
+            return None
         if lazy or stream is not None:
             xin = x.xw if lazy else x
             act = torch.empty((xin.shape[0], self.inter), dtype=torch.bfloat16, device=self.w_down.device)

@@ -49,8 +49,15 @@ class Stream:
         self.next_norm = None
 
     def add_product(self, x, weight):
-        """h += bfloat16(x weight^T) in the product's epilogue, preparing next_norm.  weight:
-        [N, K] or its few-row form."""
+        """h += bfloat16(x weight^T), preparing next_norm.  weight: [N, K] or its few-row form.
+        Up to 16 rows: in the product's epilogue.  17 to 64 rows (weight in its few-row form):
+        the product, or where next_norm can add them up its sums over pieces of K, is left
+        pending for the next norm's kernel."""
+        if x.shape[0] > POLICY["skinny_max_rows"]:
+            out = torch.empty((x.shape[0], weight.shape[0]), dtype=x.dtype, device=x.device)
+            self.pending = K.mid_store(x, weight, out, finish=not getattr(self.next_norm, "takes_partial_sums", False))
+            self.invalidate()
+            return
         norm = self.next_norm if getattr(self.next_norm, "foldable", False) else None
         self.n_ss = K.fused_residual(x, weight, self.h, self.xw_buffer,
                                      norm.weight if norm is not None else None, self.ss_buffer)
@@ -78,6 +85,13 @@ def few_rows_form(weight, parts=1):
             and weight.dim() == 2 and weight.shape[1] % 32 == 0 and weight.shape[0] % parts == 0):
         return None
     return K.pack_weight(weight, parts)
+
+
+def leaves_sums(x_rows, weight, few):
+    """Whether a product of x_rows rows with this weight (few: its few-row form) goes through the
+    kernel for 17 to 64 rows, which can leave its sums to the next norm (Stream.add_product)."""
+    return (POLICY["mid"] and few is not None and weight.dtype == torch.bfloat16
+            and POLICY["skinny_max_rows"] < x_rows <= K.MID_MAX_ROWS)
 
 
 def fusable(x_rows, weight, adds=False):
@@ -112,8 +126,7 @@ def _skinny_ok(x, weight):
 
 
 def _mid_ok(x, weight, few):
-    return (POLICY["mid"] and few is not None and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-            and POLICY["skinny_max_rows"] < x.shape[0] <= K.MID_MAX_ROWS)
+    return x.dtype == torch.bfloat16 and leaves_sums(x.shape[0], weight, few)
 
 
 def gated_silu_linear(x, weight_gate_up, few=None):
