@@ -5,11 +5,11 @@
 // packed in the lanes' order ([tile of 16 rows][K/32][lane][8 values], see skinny_fused.hip).
 //
 // With up to 64 rows x is no longer small beside a tile of weights: every wave needs all of it.
-// So a block is 8 waves that walk K together in chunks of 128; each chunk of x is staged once
+// So a block is 4 to 8 waves that walk K together in chunks of 128; each chunk of x is staged once
 // per block in LDS, in the order the lanes read it ([16 rows][k step][lane] x 16 bytes, so both
 // the block's write and the waves' reads are linear), double buffered with one barrier per
 // chunk, while each wave multiplies its own tiles of 16 output features with it.  The loads of
-// the next chunk (weights and x) are under way while the current one is multiplied.
+// the next two chunks are under way while the current one is multiplied.
 //
 // v_mfma_f32_16x16x32_bf16: A = a tile of w (16 features x 32 k), B = 32 k x 16 rows of x, so
 // D[n][m] is a tile of y^T: lane l holds row m = l%16 of its 16-row group and the four features
@@ -29,7 +29,8 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 enum { MID_STORE = 0, MID_GATED = 1 };
 #define MID_CHUNK 128           // k per stage
-#define MID_WAVES 8
+#define MID_MIN_WAVES 4          // waves per block: from the product's shape (mid_plan)
+#define MID_MAX_WAVES 8
 #define MID_MAX_ROWS 64
 
 struct MidArgs {
@@ -53,20 +54,21 @@ __device__ __forceinline__ float gate_times_up(float gate_sum, float up_sum) {
 // MT: groups of 16 rows of x (2: up to 32 rows, 4: up to 64).  TN: tiles of 16 features per wave
 // (gated: the gate tile and its up tile).
 template <int MT, int TN, int EPI, typename TY>
-__global__ __launch_bounds__(MID_WAVES * TQK_WAVE)
+__global__ __launch_bounds__(MID_MAX_WAVES * TQK_WAVE)
 void mid_product_kernel(const MidArgs p) {
     constexpr int SLOTS = MT * 256;                 // 16-byte pieces of a chunk of x: [row group][k step][lane]
-    constexpr int XS = SLOTS / (MID_WAVES * TQK_WAVE);
-    static_assert(SLOTS % (MID_WAVES * TQK_WAVE) == 0 && (EPI != MID_GATED || TN == 2), "shape of a block");
+    constexpr int XS = SLOTS / (MID_MIN_WAVES * TQK_WAVE);          // pieces per thread at most
+    static_assert(EPI != MID_GATED || TN == 2, "a gated block holds pairs of tiles");
     extern __shared__ u32x4_t xs[];                 // [2][SLOTS]
     const int lane = threadIdx.x % TQK_WAVE, wave = threadIdx.x / TQK_WAVE;
+    const int n_waves = blockDim.x / TQK_WAVE;
     const int row = lane % 16, kgrp = lane / 16;
     const int K = p.K;
     const int k_begin = blockIdx.y * p.k_per_split, k_end = min(K, k_begin + p.k_per_split);
 
     const int n_out = EPI == MID_GATED ? p.N / 2 : p.N;             // features one part of the weight has
     const int part_tiles = (n_out + 15) / 16;
-    const int tile0 = (blockIdx.x * MID_WAVES + wave) * (EPI == MID_GATED ? 1 : TN);
+    const int tile0 = (blockIdx.x * n_waves + wave) * (EPI == MID_GATED ? 1 : TN);
     const int n_lo0 = tile0 * 16;
     const size_t tile_size = (size_t)(K / 32) * 512;
     const bf16_t* wtile[TN];
@@ -76,12 +78,13 @@ void mid_product_kernel(const MidArgs p) {
         const int tile = EPI == MID_GATED ? t * part_tiles + min(tile0, part_tiles - 1) : min(tile0 + t, part_tiles - 1);
         wtile[t] = p.w + (size_t)tile * tile_size + lane * 8;
     }
-    // this thread's pieces of a chunk of x; rows past M repeat the last row
+    // this thread's pieces of a chunk of x; rows past M repeat the last row.  Pieces past the
+    // chunk's end (whole waves of them, with more than 4 waves) are loaded again and not stored.
     const bf16_t* xsrc[XS];
     int xk[XS];
 #pragma unroll
     for (int i = 0; i < XS; ++i) {
-        const int s = threadIdx.x + i * MID_WAVES * TQK_WAVE;
+        const int s = min((int)threadIdx.x + i * (int)blockDim.x, SLOTS - 1);
         const int mt = s / 256, ks = (s / 64) % 4, ln = s % 64;
         xk[i] = ks * 32 + (ln / 16) * 8;
         xsrc[i] = p.x + (size_t)min(mt * 16 + ln % 16, p.M - 1) * K;
@@ -103,7 +106,8 @@ void mid_product_kernel(const MidArgs p) {
         for (int i = 0; i < XS; ++i) {
             u32x4_t v = xr[i];
             if (c + xk[i] >= k_end) v = u32x4_t{0, 0, 0, 0};
-            xs[buf * SLOTS + threadIdx.x + i * MID_WAVES * TQK_WAVE] = v;
+            const int s = threadIdx.x + i * blockDim.x;
+            if (s < SLOTS) xs[buf * SLOTS + s] = v;
         }
     };
     auto load_w = [&](int c, bf16x8_t (&a)[TN][4]) {
@@ -132,30 +136,44 @@ void mid_product_kernel(const MidArgs p) {
         }
     };
 
-    bf16x8_t a0[TN][4], a1[TN][4];
-    u32x4_t xr[XS];
-    load_x(k_begin, xr);
-    load_w(k_begin, a0);
-    store_x(k_begin, 0, xr);
+    // Chunk j is multiplied while the weights of chunks j+1 and j+2 and x of chunk j+2 are on their
+    // way: what a step waits for was asked for two steps (weights) or one step (x, which comes
+    // from the cache) earlier.  Three register sets of weights, two of x and two LDS buffers take
+    // turns, so six steps are written out for the names to come round.
+    bf16x8_t a[3][TN][4];
+    u32x4_t xr[2][XS];
+    load_w(k_begin, a[0]);
+    load_w(k_begin + MID_CHUNK, a[1]);
+    load_x(k_begin, xr[0]);
+    load_x(k_begin + MID_CHUNK, xr[1]);
+    store_x(k_begin, 0, xr[0]);
     __syncthreads();
-    // two chunks a turn, so that the two register sets and the two LDS buffers keep their names;
-    // a last chunk past the end multiplies zeros
-    const int n_pairs = ((k_end - k_begin + MID_CHUNK - 1) / MID_CHUNK + 1) / 2;
-    for (int i = 0; i < n_pairs; ++i) {
-        const int c = k_begin + 2 * i * MID_CHUNK;
-        load_x(c + MID_CHUNK, xr);
-        load_w(c + MID_CHUNK, a1);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(0, a0);
-        store_x(c + MID_CHUNK, 1, xr);
-        __syncthreads();
-        load_x(c + 2 * MID_CHUNK, xr);
-        load_w(c + 2 * MID_CHUNK, a0);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(1, a1);
-        store_x(c + 2 * MID_CHUNK, 0, xr);
-        __syncthreads();
+#define MID_STEP(J) { \
+        const int c = base + (J) * MID_CHUNK; \
+        load_x(c + 2 * MID_CHUNK, xr[(J) % 2]); \
+        load_w(c + 2 * MID_CHUNK, a[((J) + 2) % 3]); \
+        __builtin_amdgcn_sched_barrier(0); \
+        multiply((J) % 2, a[(J) % 3]); \
+        store_x(c + MID_CHUNK, ((J) + 1) % 2, xr[((J) + 1) % 2]); \
+        __syncthreads(); }
+    int base = k_begin, left = (k_end - k_begin + MID_CHUNK - 1) / MID_CHUNK;
+    for (; left >= 6; left -= 6, base += 6 * MID_CHUNK) {
+        MID_STEP(0) MID_STEP(1) MID_STEP(2) MID_STEP(3) MID_STEP(4) MID_STEP(5)
     }
+    if (left > 0) {
+        MID_STEP(0)
+        if (left > 1) {
+            MID_STEP(1)
+            if (left > 2) {
+                MID_STEP(2)
+                if (left > 3) {
+                    MID_STEP(3)
+                    if (left > 4) MID_STEP(4)
+                }
+            }
+        }
+    }
+#undef MID_STEP
 
     const int nb = 4 * kgrp;
     if (gridDim.y > 1) {
@@ -233,24 +251,44 @@ __global__ void mid_finish_kernel(const float* __restrict__ partial, void* __res
     else ((TY*)yv)[i] = from_float<TY>(a);
 }
 
-// How a product of this shape is cut: tiles per wave and splits of K.  From N and K alone.
-struct MidPlan { int tn, blocks, splits, k_per_split; };
+// How a product of this shape is cut: tiles per wave, waves per block, splits of K.  From N and K
+// alone.  Measured: the time is that of the compute unit with the most blocks, so the blocks
+// should fall evenly on the 256 units, and about one block per unit streams fastest.
+struct MidPlan { int tn, waves, blocks, splits, k_per_split; };
+#define MID_UNITS 256
 
 static MidPlan mid_plan(int N, int K, bool gated) {
     MidPlan plan;
     const int n_out = gated ? N / 2 : N;
     const int tiles = (n_out + 15) / 16;
-    // two tiles per wave halve the reads of x from LDS, but also the blocks: only where many are left
-    plan.tn = gated ? 2 : (tiles >= 2 * MID_WAVES * 512 ? 2 : 1);
-    const int per_block = MID_WAVES * (gated ? 1 : plan.tn);
-    plan.blocks = (tiles + per_block - 1) / per_block;
-    // measured: about one block of 8 waves per compute unit streams fastest; no split shorter than 4 chunks
+    // two tiles per wave halve the reads of x from LDS, but also the waves: only where many are left
+    plan.tn = gated ? 2 : (tiles >= 8192 ? 2 : 1);
+    const int items = gated ? tiles : (tiles + plan.tn - 1) / plan.tn;        // what a wave takes
     const int chunks = (K + MID_CHUNK - 1) / MID_CHUNK;
-    int splits = 256 / plan.blocks;
-    if (splits > chunks / 4) splits = chunks / 4;
-    if (splits < 1) splits = 1;
-    const int per = (chunks + splits - 1) / splits;
-    plan.splits = (chunks + per - 1) / per;             // no empty split
+    plan.waves = MID_MAX_WAVES;
+    plan.splits = 1;
+    if (items >= MID_UNITS * MID_MIN_WAVES) {
+        // enough for every unit: the waves per block and rounds of blocks that leave the fewest idle
+        double best = 0.0;
+        for (int rounds = 1; rounds <= 8; ++rounds) {
+            int waves = (items + MID_UNITS * rounds - 1) / (MID_UNITS * rounds);
+            if (waves > MID_MAX_WAVES) continue;
+            if (waves < MID_MIN_WAVES) waves = MID_MIN_WAVES;
+            const double used = (double)items / ((double)MID_UNITS * rounds * waves);
+            if (used > best + 0.02) { best = used; plan.waves = waves; }
+        }
+        plan.blocks = (items + plan.waves - 1) / plan.waves;
+    } else {
+        // few features: blocks of 8 waves, K cut so that there is about a block per unit, no piece
+        // shorter than 4 chunks
+        plan.blocks = (items + plan.waves - 1) / plan.waves;
+        int splits = MID_UNITS / plan.blocks;
+        if (splits > chunks / 4) splits = chunks / 4;
+        if (splits < 1) splits = 1;
+        plan.splits = splits;
+    }
+    const int per = (chunks + plan.splits - 1) / plan.splits;
+    plan.splits = (chunks + per - 1) / per;             // no empty piece
     plan.k_per_split = per * MID_CHUNK;
     return plan;
 }
@@ -269,7 +307,7 @@ static size_t mid_scratch_bytes(int M, int N, int K, bool gated) {
 template <int MT, int TN, int EPI, typename TY>
 static int launch_mid(const MidArgs& a, const MidPlan& plan, bool finish, hipStream_t s) {
     dim3 grid(plan.blocks, plan.splits);
-    mid_product_kernel<MT, TN, EPI, TY><<<grid, MID_WAVES * TQK_WAVE, 2 * MT * 256 * 16, s>>>(a);
+    mid_product_kernel<MT, TN, EPI, TY><<<grid, plan.waves * TQK_WAVE, 2 * MT * 256 * 16, s>>>(a);
     if (tqk_check_launch("tqk_mid product")) return -1;
     if (plan.splits > 1 && finish) {
         const size_t total = (size_t)a.M * (EPI == MID_GATED ? a.N / 2 : a.N);
