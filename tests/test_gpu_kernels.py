@@ -28,7 +28,7 @@ def ints(values):
 
 
 def test_library_is_built_and_loaded():
-    assert K.library().tqk_abi_version() == 7
+    assert K.library().tqk_abi_version() == 8
     assert K.library_path().endswith(".so")
     with pytest.raises(K.KernelError, match="GPU only"):
         K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
@@ -529,6 +529,37 @@ def test_unfinished_sums_of_a_product_are_finished_by_the_next_norm(m, n, k):
     n1 = K.add_rmsnorm(None, done, nw, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV))
     n2 = K.add_rmsnorm(None, left, nw, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV))
     assert torch.equal(n1, n2)
+
+
+@pytest.mark.parametrize("nh,nkv,d,k", [(28, 4, 128, 3584), (3, 1, 32, 2048), (6, 2, 64, 1056)])
+def test_unfinished_sums_of_q_k_v_are_finished_by_the_rotation_kernel(nh, nkv, d, k):
+    m, n_pages = 20, 24
+    total = (nh + 2 * nkv) * d
+    x = rand(m, k, seed=40, dtype=torch.bfloat16)
+    packed = K.pack_weight(rand(total, k, seed=41, scale=1.0 / math.sqrt(k), dtype=torch.bfloat16))
+    bias = rand(total, seed=42, scale=0.3, dtype=torch.bfloat16)
+    c, s = plain.rope_tables(d, 1e4, 400)
+    cos, sin = c.to(DEV), s.to(DEV)
+    pos = ints([(37 * i) % 400 for i in range(m)])
+    seq = ints(list(range(m)))
+    table = ints([[(i + j) % n_pages for j in range(7)] for i in range(m)])
+    assert K.rope_store_takes_sums(torch.bfloat16, bias, d, K.STYLE_HALVES, d)
+    assert not K.rope_store_takes_sums(torch.bfloat16, bias, d // 2, K.STYLE_HALVES, d)
+    done = K.mid_store(x, packed, torch.empty(m, total, dtype=torch.bfloat16, device=DEV))
+    left = K.mid_store(x, packed, torch.empty(m, total, dtype=torch.bfloat16, device=DEV), finish=False)
+    assert isinstance(left, K.PartialSums)
+    res = []
+    for qkv in (done, left):
+        keys, values = make_cache(n_pages, nkv, d, torch.bfloat16)
+        q = torch.empty(m, nh, d, dtype=torch.bfloat16, device=DEV)
+        K.rope_store(qkv, bias, cos, sin, d, K.STYLE_HALVES, seq, pos, table, keys, values, q, nh, nkv, d)
+        res.append((q, keys, values))
+    for a, b in zip(res[0], res[1]):
+        assert torch.equal(torch.isnan(a.float()), torch.isnan(b.float()))
+        assert torch.equal(torch.nan_to_num(a.float()), torch.nan_to_num(b.float()))
+    with pytest.raises(K.KernelError, match="only bfloat16"):
+        K.rope_store(left, bias, cos[:, :d // 4].contiguous(), sin[:, :d // 4].contiguous(), d // 2, K.STYLE_HALVES, seq, pos, table,
+                     keys, values, q, nh, nkv, d)
 
 
 def test_products_of_17_to_64_rows_refuse_what_they_do_not_take():

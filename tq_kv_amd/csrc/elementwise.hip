@@ -354,8 +354,9 @@ __global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restri
 
 // The common case in bfloat16 (halves layout over the whole head, head_dim a multiple of 8): a
 // thread takes 4 neighbouring elements of the first half and the 4 they rotate with, 8 bytes
-// per load and store; 16 heads of a token per block.
-__global__ void rope_store_halves_bf16_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict__ bias,
+// per load and store; 16 heads of a token per block.  The q, k, v product may come unfinished, as
+// its sums over pieces of K (see PartSums): they are added up and rounded here.
+__global__ void rope_store_halves_bf16_kernel(const bf16_t* __restrict__ qkv, const PartSums ps, const bf16_t* __restrict__ bias,
                                               const float* __restrict__ cos_table, const float* __restrict__ sin_table,
                                               int max_positions, const int32_t* __restrict__ tok_seq,
                                               const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table,
@@ -371,12 +372,28 @@ __global__ void rope_store_halves_bf16_kernel(const bf16_t* __restrict__ qkv, co
     if (kind != 0 && !write_kv) return;
     const int pos = tok_pos[t];
     const size_t total = (size_t)(n_heads + 2 * n_kv_heads) * head_dim;
-    const bf16_t* src = qkv + (size_t)t * total + (size_t)head * head_dim;
-    const uint2 lo_raw = *reinterpret_cast<const uint2*>(src + i), hi_raw = *reinterpret_cast<const uint2*>(src + i + half);
-    float lo[4] = {__uint_as_float(lo_raw.x << 16), __uint_as_float(lo_raw.x & 0xffff0000u),
-                   __uint_as_float(lo_raw.y << 16), __uint_as_float(lo_raw.y & 0xffff0000u)};
-    float hi[4] = {__uint_as_float(hi_raw.x << 16), __uint_as_float(hi_raw.x & 0xffff0000u),
-                   __uint_as_float(hi_raw.y << 16), __uint_as_float(hi_raw.y & 0xffff0000u)};
+    float lo[4], hi[4];
+    if (ps.sums) {
+        const float* at = ps.sums + (size_t)t * total + (size_t)head * head_dim + i;
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+        for (int s = 0; s < ps.n; ++s) {
+            const float4 pa = *reinterpret_cast<const float4*>(at + (size_t)s * ps.stride);
+            const float4 pb = *reinterpret_cast<const float4*>(at + (size_t)s * ps.stride + half);
+            a.x += pa.x; a.y += pa.y; a.z += pa.z; a.w += pa.w;
+            b.x += pb.x; b.y += pb.y; b.z += pb.z; b.w += pb.w;
+        }
+        lo[0] = to_float(from_float<bf16_t>(a.x)); lo[1] = to_float(from_float<bf16_t>(a.y));
+        lo[2] = to_float(from_float<bf16_t>(a.z)); lo[3] = to_float(from_float<bf16_t>(a.w));
+        hi[0] = to_float(from_float<bf16_t>(b.x)); hi[1] = to_float(from_float<bf16_t>(b.y));
+        hi[2] = to_float(from_float<bf16_t>(b.z)); hi[3] = to_float(from_float<bf16_t>(b.w));
+    } else {
+        const bf16_t* src = qkv + (size_t)t * total + (size_t)head * head_dim;
+        const uint2 lo_raw = *reinterpret_cast<const uint2*>(src + i), hi_raw = *reinterpret_cast<const uint2*>(src + i + half);
+        lo[0] = __uint_as_float(lo_raw.x << 16); lo[1] = __uint_as_float(lo_raw.x & 0xffff0000u);
+        lo[2] = __uint_as_float(lo_raw.y << 16); lo[3] = __uint_as_float(lo_raw.y & 0xffff0000u);
+        hi[0] = __uint_as_float(hi_raw.x << 16); hi[1] = __uint_as_float(hi_raw.x & 0xffff0000u);
+        hi[2] = __uint_as_float(hi_raw.y << 16); hi[3] = __uint_as_float(hi_raw.y & 0xffff0000u);
+    }
     if (bias) {
         const bf16_t* b = bias + (size_t)head * head_dim;
         const uint2 bl = *reinterpret_cast<const uint2*>(b + i), bh = *reinterpret_cast<const uint2*>(b + i + half);
@@ -424,13 +441,18 @@ __global__ void rope_store_halves_bf16_kernel(const bf16_t* __restrict__ qkv, co
     *reinterpret_cast<uint2*>(dst + i + half) = make_uint2(hi_bits[0] | (hi_bits[1] << 16), hi_bits[2] | (hi_bits[3] << 16));
 }
 
-extern "C" int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, int bias_dtype,
-                              const float* cos_table, const float* sin_table, int rot_dim, int style,
-                              int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
-                              const int32_t* page_table, int table_width, int n_seqs, void* keys, void* values,
-                              int n_pages, void* q_out, int n_tokens, int n_heads, int n_kv_heads,
-                              int head_dim, int write_kv, void* stream) {
-    TQK_REQUIRE(qkv && tok_pos && q_out, "tqk_rope_store: null pointer");
+// Whether the 8-byte kernel takes these (then the product may also come as its sums).
+static bool rope_store_vector_case(int act_dtype, const void* bias, int bias_dtype, int rot_dim, int style, int head_dim) {
+    return act_dtype == TQK_BF16 && (!bias || bias_dtype == TQK_BF16) && style == 1 && rot_dim == head_dim && head_dim % 8 == 0;
+}
+
+static int rope_store(const void* qkv, const PartSums ps, int act_dtype, const void* bias, int bias_dtype,
+                      const float* cos_table, const float* sin_table, int rot_dim, int style,
+                      int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
+                      const int32_t* page_table, int table_width, int n_seqs, void* keys, void* values,
+                      int n_pages, void* q_out, int n_tokens, int n_heads, int n_kv_heads,
+                      int head_dim, int write_kv, void* stream) {
+    TQK_REQUIRE((qkv || ps.sums) && tok_pos && q_out, "tqk_rope_store: null pointer");
     TQK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0, "tqk_rope_store: bad sizes");
     TQK_REQUIRE(style >= 0 && style <= 2, "tqk_rope_store: unknown rotation style %d", style);
     if (style != 0) {
@@ -446,16 +468,18 @@ extern "C" int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, 
     }
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    if (act_dtype == TQK_BF16 && (!bias || bias_dtype == TQK_BF16) && style == 1 && rot_dim == head_dim && head_dim % 8 == 0 &&
-        ((((uintptr_t)qkv) | ((uintptr_t)bias) | ((uintptr_t)cos_table) | ((uintptr_t)sin_table) | ((uintptr_t)keys) |
-          ((uintptr_t)q_out)) & 15) == 0) {
+    if (rope_store_vector_case(act_dtype, bias, bias_dtype, rot_dim, style, head_dim) &&
+        ((((uintptr_t)qkv) | ((uintptr_t)ps.sums) | ((uintptr_t)bias) | ((uintptr_t)cos_table) | ((uintptr_t)sin_table) |
+          ((uintptr_t)keys) | ((uintptr_t)q_out)) & 15) == 0) {
         const int slots = (n_heads + 2 * n_kv_heads) * (head_dim / 8);
         dim3 vgrid(n_tokens, (slots + 255) / 256);
         rope_store_halves_bf16_kernel<<<vgrid, 256, 0, s>>>(
-            (const bf16_t*)qkv, (const bf16_t*)bias, cos_table, sin_table, max_positions, tok_seq, tok_pos, page_table,
+            (const bf16_t*)qkv, ps, (const bf16_t*)bias, cos_table, sin_table, max_positions, tok_seq, tok_pos, page_table,
             table_width, (bf16_t*)keys, (bf16_t*)values, (bf16_t*)q_out, n_heads, n_kv_heads, head_dim, write_kv);
         return tqk_check_launch("tqk_rope_store");
     }
+    TQK_REQUIRE(!ps.sums, "tqk_rope_store_sums: only bfloat16, rotation in halves over the whole head, head_dim a multiple of 8, "
+                          "16-byte aligned operands");
     dim3 grid(n_tokens, (n_heads + 2 * n_kv_heads + 3) / 4);
     const int threads = 4 * TQK_WAVE;
 #define LAUNCH(TA, TB) rope_store_kernel<TA, TB><<<grid, threads, 0, s>>>( \
@@ -468,6 +492,37 @@ extern "C" int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, 
     else return tqk_fail("tqk_rope_store: unknown dtypes act=%d bias=%d", act_dtype, bias_dtype);
 #undef LAUNCH
     return tqk_check_launch("tqk_rope_store");
+}
+
+extern "C" int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, int bias_dtype,
+                              const float* cos_table, const float* sin_table, int rot_dim, int style,
+                              int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
+                              const int32_t* page_table, int table_width, int n_seqs, void* keys, void* values,
+                              int n_pages, void* q_out, int n_tokens, int n_heads, int n_kv_heads,
+                              int head_dim, int write_kv, void* stream) {
+    return rope_store(qkv, PartSums{nullptr, 0, 0}, act_dtype, bias, bias_dtype, cos_table, sin_table, rot_dim, style, max_positions,
+                      tok_seq, tok_pos, page_table, table_width, n_seqs, keys, values, n_pages, q_out, n_tokens, n_heads,
+                      n_kv_heads, head_dim, write_kv, stream);
+}
+
+/* Whether tqk_rope_store_sums takes this case (bfloat16, bias none or bfloat16, halves over the whole head). */
+extern "C" int tqk_rope_store_takes_sums(int act_dtype, int has_bias, int bias_dtype, int rot_dim, int style, int head_dim) {
+    return rope_store_vector_case(act_dtype, has_bias ? (const void*)1 : nullptr, bias_dtype, rot_dim, style, head_dim) ? 1 : 0;
+}
+
+/* The same with the q, k, v product given as its sums over n_sums pieces of K, float32
+ * [n_sums][n_tokens][(heads + 2 kv heads) * head_dim]; bfloat16 activations only. */
+extern "C" int tqk_rope_store_sums(const float* sums, int n_sums, const void* bias, int bias_dtype,
+                                   const float* cos_table, const float* sin_table, int rot_dim, int style,
+                                   int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
+                                   const int32_t* page_table, int table_width, int n_seqs, void* keys, void* values,
+                                   int n_pages, void* q_out, int n_tokens, int n_heads, int n_kv_heads,
+                                   int head_dim, int write_kv, void* stream) {
+    TQK_REQUIRE(sums && n_sums > 0, "tqk_rope_store_sums: no sums given");
+    const size_t stride = (size_t)n_tokens * (n_heads + 2 * n_kv_heads) * head_dim;
+    return rope_store(nullptr, PartSums{sums, n_sums, stride}, TQK_BF16, bias, bias_dtype, cos_table, sin_table, rot_dim, style,
+                      max_positions, tok_seq, tok_pos, page_table, table_width, n_seqs, keys, values, n_pages, q_out, n_tokens,
+                      n_heads, n_kv_heads, head_dim, write_kv, stream);
 }
 
 // ---- SwiGLU ----------------------------------------------------------------------

@@ -94,6 +94,16 @@ int tqk_rope_store(const void* qkv, int act_dtype, const void* bias, int bias_dt
                    const int32_t* page_table, int table_width, int n_seqs, void* keys, void* values,
                    int n_pages, void* q_out, int n_tokens, int n_heads, int n_kv_heads,
                    int head_dim, int write_kv, void* stream);
+/* the same with the q, k, v product given as its sums over n_sums pieces of K (tqk_mid_store with
+ * finish == 0), float32 [n_sums][n_tokens][(heads + 2 kv heads) * head_dim]; only where
+ * tqk_rope_store_takes_sums says so */
+int tqk_rope_store_takes_sums(int act_dtype, int has_bias, int bias_dtype, int rot_dim, int style, int head_dim);
+int tqk_rope_store_sums(const float* sums, int n_sums, const void* bias, int bias_dtype,
+                        const float* cos_table, const float* sin_table, int rot_dim, int style,
+                        int max_positions, const int32_t* tok_seq, const int32_t* tok_pos,
+                        const int32_t* page_table, int table_width, int n_seqs, void* keys, void* values,
+                        int n_pages, void* q_out, int n_tokens, int n_heads, int n_kv_heads,
+                        int head_dim, int write_kv, void* stream);
 
 /* Softmax attention of each token's query over its sequence's cached positions
  * lo..tok_pos[t], lo = max(0, tok_pos - window + 1) if window > 0 else 0.  One wave

@@ -50,8 +50,8 @@ class Model:
         self.few_head = None
         self.loaded = False
         # a step can be captured as a graph if every part's forward launches the same kernels
-        # whatever the step's data are; up to 64 rows (beyond 16 the products are library calls,
-        # which capture as they are)
+        # whatever the step's data are; up to 64 rows (the hand-written products; where a weight
+        # has no packed copy the library's, which capture as they are)
         self.graph_safe = all(getattr(b, "graph_safe", False) for b in self.blocks) and getattr(self.final_norm, "graph_safe", False)
         self.graph_max_rows = 64
 
@@ -117,9 +117,10 @@ class Model:
 
     def tune_library(self, rows):
         """Let the library try its kernels once for every product of the model at `rows`
-        rows (more than 16: fewer never reach the library) and keep the fastest for later
-        calls.  Takes seconds per distinct weight shape."""
-        if self.dtype != torch.bfloat16 or rows <= L.POLICY["skinny_max_rows"]:
+        rows (more than 64, or 16 without packed weights: fewer never reach the library) and
+        keep the fastest for later calls.  Takes seconds per distinct weight shape."""
+        own_rows = K.MID_MAX_ROWS if L.POLICY["mid"] and L.POLICY["packed"] else L.POLICY["skinny_max_rows"]
+        if self.dtype != torch.bfloat16 or rows <= own_rows:
             return
         L.tune_library(True)
         seen = set()

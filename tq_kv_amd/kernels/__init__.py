@@ -142,7 +142,8 @@ def gemm(x, w, bias, out):
 def rope_store(qkv, bias, cos, sin, rot_dim, style, tok_seq, tok_pos, page_table, keys, values, q_out,
                n_heads, n_kv_heads, head_dim, write_kv=True):
     """Bias, rotation of q and k, q to q_out, k and v into the cache pages
-    (keys [pages, kv heads, 64, d], values [pages, kv heads, d, 64])."""
+    (keys [pages, kv heads, 64, d], values [pages, kv heads, d, 64]).  qkv: [T, total], or where
+    rope_store_takes_sums says so the product's PartialSums."""
     n = qkv.shape[0]
     total = (n_heads + 2 * n_kv_heads) * head_dim
     max_pos = 0
@@ -156,6 +157,19 @@ def rope_store(qkv, bias, cos, sin, rot_dim, style, tok_seq, tok_pos, page_table
         n_pages = keys.shape[0]
         _dev(keys, "keys", qkv.dtype, (n_pages, n_kv_heads, 64, head_dim))
         _dev(values, "values", qkv.dtype, (n_pages, n_kv_heads, head_dim, 64))
+    if isinstance(qkv, PartialSums):
+        if tuple(qkv.shape) != (n, total) or qkv.dtype != torch.bfloat16:
+            raise KernelError("rope_store: the product's sums are %s of %s, wanted %s of bfloat16" % (qkv.shape, qkv.dtype, (n, total)))
+        _check(library().tqk_rope_store_sums(
+            _dev(qkv.sums, "sums", torch.float32), qkv.sums.shape[0], _opt(bias, "bias", None, (total,)),
+            _code(bias.dtype) if bias is not None else 0,
+            _opt(cos if style != STYLE_NONE else None, "cos"), _opt(sin if style != STYLE_NONE else None, "sin"),
+            rot_dim, style, max_pos, _opt(tok_seq, "tok_seq", torch.int32, (n,)), _dev(tok_pos, "tok_pos", torch.int32, (n,)),
+            _opt(page_table if write_kv else None, "page_table", torch.int32), width, n_seqs,
+            _opt(keys if write_kv else None, "keys"), _opt(values if write_kv else None, "values"), n_pages,
+            _dev(q_out, "q_out", torch.bfloat16, (n, n_heads, head_dim)), n, n_heads, n_kv_heads, head_dim,
+            1 if write_kv else 0, _stream()), "rope_store")
+        return q_out
     _check(library().tqk_rope_store(
         _dev(qkv, "qkv", None, (n, total)), _code(qkv.dtype), _opt(bias, "bias", None, (total,)),
         _code(bias.dtype) if bias is not None else 0,
@@ -166,6 +180,14 @@ def rope_store(qkv, bias, cos, sin, rot_dim, style, tok_seq, tok_pos, page_table
         _dev(q_out, "q_out", qkv.dtype, (n, n_heads, head_dim)), n, n_heads, n_kv_heads, head_dim,
         1 if write_kv else 0, _stream()), "rope_store")
     return q_out
+
+
+def rope_store_takes_sums(act_dtype, bias, rot_dim, style, head_dim):
+    """Whether rope_store takes a product's PartialSums in this case."""
+    if act_dtype != torch.bfloat16:
+        return False
+    return bool(library().tqk_rope_store_takes_sums(BF16, 0 if bias is None else 1, _code(bias.dtype) if bias is not None else 0,
+                                                    int(rot_dim), int(style), int(head_dim)))
 
 
 def attention(q, keys, values, tok_seq, tok_pos, page_table, window, scale, out):

@@ -130,8 +130,13 @@ class Attention(Part):
 
     def _qkv(self, x, ctx, entry, table, q):
         """Product, then bias, position encoding and cache write in their own kernel."""
-        qkv = linear(x, self.w_qkv, few=self.few_qkv)
-        if hasattr(self.position, "apply"):
+        own = hasattr(self.position, "apply")
+        sums_ok = False
+        if not own:
+            _, _, rot_dim, style = self.position.tables()
+            sums_ok = K.rope_store_takes_sums(x.dtype, self.b_qkv, rot_dim, style, self.head_dim)
+        qkv = linear(x, self.w_qkv, few=self.few_qkv, leave_sums=sums_ok)      # may come as its sums over pieces of K
+        if own:
             # a position encoding of its own: bias first, then it changes q and k in place
             if self.b_qkv is not None:
                 qkv += self.b_qkv.to(qkv.dtype)

@@ -144,9 +144,11 @@ def gated_silu_linear(x, weight_gate_up, few=None):
     return K.swiglu(linear(x, weight_gate_up), act)
 
 
-def linear(x, weight, bias=None, out_dtype=None, few=None):
+def linear(x, weight, bias=None, out_dtype=None, few=None, leave_sums=False):
     """x: [M,K]; weight: [N,K]; bias: [N] or None.  Returns [M,N] of out_dtype
-    (default: x's dtype).  few: the weight's few_rows_form, if there is one."""
+    (default: x's dtype).  few: the weight's few_rows_form, if there is one.  leave_sums: the
+    caller also takes the product unfinished, as kernels.PartialSums (the kernel for 17 to 64
+    rows gives those where it cuts K into pieces)."""
     m, k = x.shape
     n = weight.shape[0]
     if weight.shape[1] != k:
@@ -159,7 +161,7 @@ def linear(x, weight, bias=None, out_dtype=None, few=None):
             return K.fused_store(x, few or weight, out)
         if _mid_ok(x, weight, few):
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-            return K.mid_store(x, few, out)
+            return K.mid_store(x, few, out, finish=not leave_sums)
         if POLICY["library"] and m > POLICY["skinny_max_rows"]:
             if out_dtype == torch.bfloat16:
                 return torch.matmul(x, weight.t())
