@@ -1,7 +1,9 @@
 // Attention for decoding: one new token per sequence attends over its sequence's pages
 // of the cache.  bfloat16 in, MFMA, float32 softmax.  Bound by the bytes of keys and
 // values, so the work is cut for memory: a block of 4 waves per (sequence, kv head,
-// partition of the pages), each wave taking every fourth page of the partition; all
+// partition of the pages); the partitions take the live pages in turn (partition p the pages
+// first + p, first + p + parts, ...: however long the sequence is, they get the same share)
+// and so do the four waves inside a partition; all
 // query heads that share the kv head ride in the same wave, so keys and values are
 // read once for the whole group (the reference expands them per query head instead,
 // src/models/turbo_generic.rs:195-204, 1620-1621).  The waves' results are merged
@@ -42,7 +44,7 @@ __global__ __launch_bounds__(AD_WAVES * TQK_WAVE)
 void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ keys,
                              const bf16_t* __restrict__ values, const int32_t* __restrict__ tok_pos,
                              const int32_t* __restrict__ page_table, int table_width, int window, float scale,
-                             int pages_per_part, int n_parts, int n_heads, int n_kv_heads, int q_blocks,
+                             int n_parts, int n_heads, int n_kv_heads, int q_blocks,
                              float* __restrict__ part_out, float* __restrict__ part_ml,
                              bf16_t* __restrict__ out) {
     constexpr int KB = D / 32;          // k-blocks of the score product
@@ -63,16 +65,15 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     const bool head_live = rep < n_rep;
     const int head = kvh * n_rep + (head_live ? rep : 0);
 
-    const int first_page = part * pages_per_part;
-    const int last_page = min(first_page + pages_per_part - 1, pos / TQK_PAGE);
-    const int start_page = max(first_page, lo / TQK_PAGE);
+    const int last_page = pos / TQK_PAGE;
+    const int start_page = lo / TQK_PAGE + part + wave * n_parts;       // this wave's first page
 
     float m = -INFINITY, l = 0.f;
     floatx4_t o[DB];
 #pragma unroll
     for (int i = 0; i < DB; ++i) o[i] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    if (start_page + wave <= last_page) {
+    if (start_page <= last_page) {
         pack8 zero;
         zero.q = make_uint4(0, 0, 0, 0);
         // the heads' queries: B operand of the score product
@@ -84,7 +85,7 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 
         const int32_t* pages = page_table + (size_t)seq * table_width;
         const size_t page_stride = (size_t)n_kv_heads * TQK_PAGE * D;
-        for (int pg = start_page + wave; pg <= last_page; pg += AD_WAVES) {
+        for (int pg = start_page; pg <= last_page; pg += AD_WAVES * n_parts) {
             const int page = pages[pg];
             if (page < 0) continue;                     // the host never lets this happen
             const bf16_t* kp = keys + (size_t)page * page_stride + (size_t)kvh * TQK_PAGE * D;
@@ -244,7 +245,7 @@ extern "C" int tqk_attention_decode_supported(int head_dim) {
 
 extern "C" int tqk_attention_decode(const void* q, const void* keys, const void* values, const int32_t* tok_pos,
                                     const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window,
-                                    float scale, int pages_per_part, int n_parts, void* part_out, void* part_ml,
+                                    float scale, int n_parts, void* part_out, void* part_ml,
                                     void* out, int n_heads, int n_kv_heads, int head_dim, void* stream) {
     TQK_REQUIRE(q && keys && values && tok_pos && page_table && out, "tqk_attention_decode: null pointer");
     TQK_REQUIRE(n_parts == 1 || (part_out && part_ml), "tqk_attention_decode: more than one partition needs part_out and part_ml");
@@ -252,8 +253,7 @@ extern "C" int tqk_attention_decode(const void* q, const void* keys, const void*
     TQK_REQUIRE(n_heads % n_kv_heads == 0, "tqk_attention_decode: %d heads are not a multiple of %d kv heads", n_heads, n_kv_heads);
     TQK_REQUIRE(tqk_attention_decode_supported(head_dim), "tqk_attention_decode: head_dim %d is not one of 32, 64, 96, 128, 256", head_dim);
     TQK_REQUIRE(table_width > 0 && n_pages > 0, "tqk_attention_decode: empty page table");
-    TQK_REQUIRE(pages_per_part > 0 && n_parts > 0 && (long long)n_parts * pages_per_part >= table_width,
-                "tqk_attention_decode: %d partitions of %d pages do not cover %d pages", n_parts, pages_per_part, table_width);
+    TQK_REQUIRE(n_parts > 0 && n_parts <= 65535, "tqk_attention_decode: %d partitions", n_parts);
     TQK_REQUIRE(window >= 0, "tqk_attention_decode: negative window");
     const int q_blocks = (n_heads / n_kv_heads + 15) / 16;
     TQK_REQUIRE(n_seqs <= 65535 && n_kv_heads * q_blocks <= 65535, "tqk_attention_decode: grid too large");
@@ -262,7 +262,7 @@ extern "C" int tqk_attention_decode(const void* q, const void* keys, const void*
     dim3 grid(n_parts, n_kv_heads * q_blocks, n_seqs);
 #define LAUNCH(DD) attention_decode_kernel<DD><<<grid, AD_WAVES * TQK_WAVE, 0, s>>>( \
         (const bf16_t*)q, (const bf16_t*)keys, (const bf16_t*)values, tok_pos, page_table, table_width, window, scale, \
-        pages_per_part, n_parts, n_heads, n_kv_heads, q_blocks, (float*)part_out, (float*)part_ml, (bf16_t*)out)
+        n_parts, n_heads, n_kv_heads, q_blocks, (float*)part_out, (float*)part_ml, (bf16_t*)out)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;

@@ -114,14 +114,14 @@ int tqk_attention(const void* q, const void* keys, const void* values, int act_d
                   int n_tokens, int n_heads, int n_kv_heads, int head_dim, void* stream);
 
 /* Decoding: sequence b's one new token (query row b, position tok_pos[b]) over its pages,
- * bfloat16, MFMA; the pages are cut into n_parts partitions of pages_per_part pages.  With
+ * bfloat16, MFMA; n_parts partitions take the sequence's live pages in turn.  With
  * one partition the result goes straight to out [seqs, heads*head_dim]; with more, the
  * partitions' results go to part_out [seqs, heads, n_parts, head_dim] and part_ml [seqs,
  * heads, n_parts, 2] (float32) and a second kernel merges them into out. */
 int tqk_attention_decode_supported(int head_dim);
 int tqk_attention_decode(const void* q, const void* keys, const void* values, const int32_t* tok_pos,
                          const int32_t* page_table, int table_width, int n_seqs, int n_pages, int window,
-                         float scale, int pages_per_part, int n_parts, void* part_out, void* part_ml,
+                         float scale, int n_parts, void* part_out, void* part_ml,
                          void* out, int n_heads, int n_kv_heads, int head_dim, void* stream);
 
 /* Prompts: tiles of up to 64 consecutive queries of one sequence (tile i: sequence

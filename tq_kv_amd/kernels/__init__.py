@@ -271,9 +271,8 @@ def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, t
         raise KernelError("attention_decode: %d query rows for %d sequences (one token each is required)" % (n, n_seqs))
     q_blocks = (n_heads // n_kv_heads + 15) // 16
     groups = max(1, n * n_kv_heads * q_blocks)
-    want_parts = max(1, min(width, (target_blocks + groups - 1) // groups))
-    per_part = (width + want_parts - 1) // want_parts
-    n_parts = (width + per_part - 1) // per_part
+    # partitions take the live pages in turn, four waves each: no more than a quarter of the pages there can be
+    n_parts = max(1, min((width + 3) // 4, (target_blocks + groups - 1) // groups))
     part_out = part_ml = None
     if n_parts > 1:
         part_out = torch.empty((n, n_heads, n_parts, head_dim), dtype=torch.float32, device=q.device)
@@ -282,7 +281,7 @@ def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, t
         _dev(q, "q", torch.bfloat16), _dev(keys, "keys", torch.bfloat16, (n_pages, n_kv_heads, 64, head_dim)),
         _dev(values, "values", torch.bfloat16, (n_pages, n_kv_heads, head_dim, 64)),
         _dev(tok_pos, "tok_pos", torch.int32, (n,)), _dev(page_table, "page_table", torch.int32), width, n, n_pages,
-        int(window or 0), ctypes.c_float(scale), per_part, n_parts, _opt(part_out, "part_out"), _opt(part_ml, "part_ml"),
+        int(window or 0), ctypes.c_float(scale), n_parts, _opt(part_out, "part_out"), _opt(part_ml, "part_ml"),
         _dev(out, "out", torch.bfloat16, (n, n_heads * head_dim)), n_heads, n_kv_heads, head_dim, _stream()),
         "attention_decode")
     return out
