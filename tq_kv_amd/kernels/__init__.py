@@ -412,9 +412,9 @@ def _mid_scratch(m, n, k, gated, device):
 
 
 def mid_store(x, weight, out=None, finish=True):
-    """out[M,N] = x weight^T for up to 64 rows of bfloat16; weight: a PackedWeight.  finish=False:
-    where the kernel cuts K into pieces, their PartialSums (of out's dtype, which need not be
-    given then: bfloat16) are returned in place of out."""
+    """out[M,N] = x weight^T for up to 64 rows of bfloat16; weight: a PackedWeight; out: bfloat16
+    or float32, made here (bfloat16) if not given.  finish=False: where the kernel cuts K into
+    pieces, their PartialSums (of out's dtype) are returned in place of out."""
     m, k = x.shape
     if not isinstance(weight, PackedWeight):
         raise KernelError("mid_store: the weight must be packed (pack_weight)")
@@ -422,12 +422,9 @@ def mid_store(x, weight, out=None, finish=True):
     w, _ = _weight(weight, "weight", n, k)
     scratch = _mid_scratch(m, n, k, False, x.device)
     leave = not finish and scratch is not None
-    if out is None:
-        if not leave:
-            raise KernelError("mid_store: no output given")
-        dtype = torch.bfloat16
-    else:
-        dtype = out.dtype
+    dtype = out.dtype if out is not None else torch.bfloat16
+    if out is None and not leave:
+        out = torch.empty((m, n), dtype=dtype, device=x.device)
     _check(library().tqk_mid_store(_dev(x, "x", torch.bfloat16, (m, k)), w, _opt(None if leave else out, "out", None, (m, n)),
                                    _code(dtype), m, n, k, _opt(scratch, "scratch"), 0 if leave else 1, _stream()), "mid_store")
     return PartialSums(scratch, dtype) if leave else out

@@ -34,8 +34,9 @@ POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16, "fused": True,
 
 
 class Stream:
-    """The residual stream of a step.  h: float32 [tokens, hidden].  pending: an update (of
-    the activation dtype) that has not been added to h yet, or None.
+    """The residual stream of a step.  h: float32 [tokens, hidden].  pending: an update that
+    has not been added to h yet (a tensor of the activation dtype, or a product's
+    kernels.PartialSums for a norm that takes those), or None.
 
     In small decoding steps the kernels that add to h also prepare the next norm: xw is
     bfloat16(h * weight of norm `xw_for`) and ss the rows' sums of squares in n_ss pieces
@@ -54,8 +55,7 @@ class Stream:
         the product, or where next_norm can add them up its sums over pieces of K, is left
         pending for the next norm's kernel."""
         if x.shape[0] > POLICY["skinny_max_rows"]:
-            out = torch.empty((x.shape[0], weight.shape[0]), dtype=x.dtype, device=x.device)
-            self.pending = K.mid_store(x, weight, out, finish=not getattr(self.next_norm, "takes_partial_sums", False))
+            self.pending = K.mid_store(x, weight, finish=not getattr(self.next_norm, "takes_partial_sums", False))
             self.invalidate()
             return
         norm = self.next_norm if getattr(self.next_norm, "foldable", False) else None
