@@ -38,6 +38,7 @@ def main():
 
     from tq_kv_amd import Engine, GenerationParams, Model, generate
     from tq_kv_amd.config import catalog
+    from tq_kv_amd.parts.linear import POLICY
 
     t_start = time.perf_counter()
 
@@ -67,12 +68,10 @@ def main():
 
     # -- prefill of one prompt --------------------------------------------------------------
     if not args.no_tune:
-        # products of more than 16 rows are the library's: let it try its kernels once for the
-        # shapes of the measured steps (a prompt of prompt_len tokens, decoding at batch 64)
-        note("library tuning for %d and 64 rows" % args.prompt_len)
+        # products of more than 64 rows are the library's: let it try its kernels once for the
+        # shapes of the measured prompt pass
+        note("library tuning for %d rows" % args.prompt_len)
         model.tune_library(args.prompt_len)
-        if not args.no_points:
-            model.tune_library(64)
     p = prompts(1)[0]
     times = []
     note("prefill of %d tokens" % args.prompt_len)
@@ -133,7 +132,7 @@ def main():
                    "layers": layers, "layers_of_shape": full_layers, "hidden": H, "heads": nh, "kv_heads": nkv,
                    "head_dim": d, "intermediate": I, "vocab": V, "prompt_len": args.prompt_len,
                    "new_tokens": args.warmup + args.steps + 2, "weights": "random N(0,0.02)", "sampling": "greedy",
-                   "library_tuning": not args.no_tune},
+                   "library_tuning": not args.no_tune, "packed_weight_copy": bool(POLICY["packed"])},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK["hbm_gbs"], "unit": "GB/s",
                      "frac": round(achieved / PEAK["hbm_gbs"], 4)},
@@ -151,8 +150,6 @@ def mixed_workload(args, model, engine, raw, note):
     gen = torch.Generator().manual_seed(1)
     lens = torch.randint(16, args.prompt_len + 1, (args.batch,), generator=gen).tolist()
     prompts = [torch.randint(0, raw["vocab_size"], (n,), generator=gen).tolist() for n in lens]
-    if not args.no_tune:
-        model.tune_library(min(args.batch, 64))
     marks, calls = {}, [0]
 
     def on_tokens(pairs):
