@@ -95,6 +95,31 @@ def test_unequal_batches_one_after_another(name, sharp, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,seed", [("A", 1), ("B", 2), ("B", 3), ("C", 4)])
+def test_batches_of_random_sizes_shrink_through_every_kind_of_step(name, seed, dtype):
+    """Up to 44 requests start together with unequal prompts and tails of unequal lengths, so the
+    steps run from many rows down to one: through the library's products (prompts), the kernels
+    for 17 to 64 rows, the folded few-row kernels, and every change from one to the next."""
+    import random
+    rng = random.Random(seed)
+    sharp = name != "A"
+    eng = G.engine(name, dtype, sharp)
+    top = {"A": 100, "B": 80, "C": 120}[name]
+    for round_ in range(2):
+        n = rng.choice([18, 33, 44]) if round_ == 0 else rng.randint(2, 30)
+        lens = [rng.randint(2, top) for _ in range(n)]
+        reqs = G.prompts(name, lens, seed=900 + 17 * seed + round_)
+        tails = [rng.randint(0, min(len(r) - 1, 24)) for r in reqs]
+        G.poison_free_pages(eng)
+        outs, _ = run_batch(eng, reqs, tails)
+        for i, (r, o) in enumerate(zip(reqs, outs)):
+            G.close(o, G.plain_logits(name, r, sharp), dtype, "%s seed %d round %d request %d (len %d, tail %d)"
+                    % (name, seed, round_, i, len(r), tails[i]))
+        eng.cache.check()
+        assert eng.cache.slots.n_held == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(dtype):
     # 70 prompt tokens, then 400 single steps: across pages and far beyond the window
     eng = G.engine("C", dtype, True)
