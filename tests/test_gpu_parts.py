@@ -400,3 +400,89 @@ def test_toy_feed_forward_with_routing_and_toy_position_encoding(dtype):
         got_b, want_b = got_b[close], want_b[close]
     torch.testing.assert_close(got_a, want_a, **tol)
     torch.testing.assert_close(got_b, want_b, **tol)
+
+
+# ---- a toy norm: none of the folding hooks ---------------------------------------------------
+@register("norm", "toy_centered")
+class ToyCentered(Part):
+    """y = (x - mean(x)) / sqrt(var(x) + eps) * weight: a norm with another formula and without
+    `lazy`, `foldable` or `takes_partial_sums`.  The framework's products around it must hand it
+    finished tensors whatever the size of the step."""
+    graph_safe = True
+
+    def __init__(self, params, env):
+        self.size, self.eps, self.env = params["size"], params["eps"], env
+
+    def tensors(self):
+        return {"weight": TensorSpec((self.size,), init="one_plus_normal")}
+
+    def load(self, tensors):
+        self.weight = tensors["weight"]
+
+    def _norm(self, x):
+        x = x.float()
+        x = x - x.mean(-1, keepdim=True)
+        return (x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()).to(self.env.act_dtype)
+
+    def forward(self, x):
+        return self._norm(x)
+
+    def add_norm(self, h, delta):
+        if delta is not None:
+            assert isinstance(delta, torch.Tensor)          # never a product's unfinished sums
+            h += delta.float()
+        return self._norm(h)
+
+    def gather_add_norm(self, h, delta, rows):
+        x = h[rows.long()]
+        if delta is not None:
+            assert isinstance(delta, torch.Tensor)
+            x = x + delta[rows.long()].float()
+        return self._norm(x)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_norm_between_the_frameworks_products_in_steps_of_every_size(dtype):
+    cfg = dict(helpers.TINY_B)
+    spec = tiny_spec(cfg)
+    toy = PartSpec("toy_centered", {"size": cfg["hidden_size"], "eps": 1e-5})
+    for layer in spec.layers:
+        layer.block.params["mixer_norm"] = layer.block.params["ff_norm"] = toy
+    import dataclasses
+    model = Model(dataclasses.replace(spec, final_norm=toy), dtype, DEV)
+    # weights small enough that the logits stay near 1: the bfloat16 tolerance is an absolute one (measured at
+    # 0.08: logits up to 2.6 and rounding errors up to 0.038 whichever kernels run, the library's included)
+    specs = {n: TensorSpec(s.shape, s.init, 0.04 if s.init == "normal" else 0.1) for n, s in model.tensor_specs().items()}
+    w = random_tensors(specs, 9, DT[dtype], "cpu")
+    model.load({k: v.to(DEV) for k, v in w.items()})
+    w = {k: v.float() for k, v in w.items()}
+
+    def norm(x, weight):
+        x = x - x.mean(-1, keepdim=True)
+        return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + 1e-5) * weight
+
+    def plain_forward(tokens):
+        x = w["model.embed_tokens.weight"][tokens]
+        for l in range(cfg["num_hidden_layers"]):
+            p = "model.layers.%d." % l
+            x = x + plain.attention(norm(x, w[p + "input_layernorm.weight"]), w, p + "self_attn.", cfg, plain.layer_window(cfg, l))
+            x = x + plain.swiglu_mlp(norm(x, w[p + "post_attention_layernorm.weight"]), w, p + "mlp.")
+        return plain.linear(norm(x, w["model.norm.weight"]), w["lm_head.weight"])
+
+    eng = Engine(model, max_tokens=4096)
+    # 24 sequences: a prompt step of 24 x 3 = 72 tokens (the library's products), then steps of 24
+    # rows (the products for 17 to 64 rows), then, as sequences end, of 8 rows (the few-row products)
+    reqs = [helpers.random_tokens(8 if i < 8 else 6, cfg["vocab_size"], 50 + i) for i in range(24)]
+    slots = [eng.open() for _ in reqs]
+    got = [[eng_out] for eng_out in eng.step([(s, r[:3], [0, 1, 2]) for s, r in zip(slots, reqs)]).split(3)]
+    for t in range(3, 8):
+        live = [i for i, r in enumerate(reqs) if t < len(r)]
+        out = eng.step([(slots[i], [reqs[i][t]], [0]) for i in live])
+        for j, i in enumerate(live):
+            got[i].append(out[j:j + 1])
+    for s in slots:
+        eng.close(s)
+    eng.cache.check()
+    tol = dict(atol=2e-5, rtol=2e-5) if dtype == "float32" else G.TOL["bfloat16"]
+    for i, r in enumerate(reqs):
+        torch.testing.assert_close(torch.cat(got[i]).cpu(), plain_forward(r), msg=lambda m: "request %d: %s" % (i, m), **tol)

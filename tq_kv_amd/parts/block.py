@@ -70,7 +70,7 @@ class PreNormBlock(Part):
 
     def _normed(self, norm, stream, part, ctx):
         """The part's input: the norm of the stream, computed now, or left to the part."""
-        if ctx.fuse_small and getattr(part, "folds_norm", None) and part.folds_norm(ctx):
+        if ctx.fuse_small and hasattr(norm, "lazy") and getattr(part, "folds_norm", None) and part.folds_norm(ctx):
             lazy = norm.lazy(stream)
             if lazy is not None:
                 return lazy
