@@ -491,7 +491,7 @@ def test_product_of_17_to_64_rows(m, n, k):
 
 
 @pytest.mark.parametrize("m", [17, 40, 64])
-@pytest.mark.parametrize("inter,k", [(112, 64), (18944, 3584), (100, 96), (200, 1312)])
+@pytest.mark.parametrize("inter,k", [(112, 64), (18944, 3584), (100, 96), (200, 1312), (18, 1312), (50, 2048), (7, 96)])
 def test_gated_product_of_17_to_64_rows(m, inter, k):
     x = rand(m, k, seed=34, scale=1.5, dtype=torch.bfloat16)
     w = rand(2 * inter, k, seed=35, scale=0.4 / math.sqrt(k), dtype=torch.bfloat16)       # gate and up of size about 1

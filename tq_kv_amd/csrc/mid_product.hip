@@ -177,7 +177,7 @@ void mid_product_kernel(const MidArgs p) {
 
     const int nb = 4 * kgrp;
     if (gridDim.y > 1) {
-        const bool vec = p.N % 4 == 0;
+        const bool vec = p.N % 4 == 0 && n_out % 4 == 0;           // the up rows' sums start at n_out
 #pragma unroll
         for (int t = 0; t < TN; ++t)
 #pragma unroll
