@@ -55,6 +55,33 @@ def test_bfloat16_tracks_float32_at_large_sizes(shape):
     torch.testing.assert_close(outs["bfloat16"], outs["float32"], atol=0.03 * max(1.0, scale), rtol=0.03)
 
 
+@pytest.mark.parametrize("shape,n_seqs", [("qwen2.5:7b", 20), ("qwen2.5:32b", 40)])
+def test_bfloat16_tracks_float32_in_steps_of_17_to_64_rows_at_large_sizes(shape, n_seqs):
+    """The kernels for 17 to 64 rows at the real widths (sums over pieces of K finished by the norm
+    and the rotation kernels, the head product with float32 output): a short prompt step of 24
+    tokens, then two decoding steps of n_seqs rows."""
+    raw = two_layer(shape)
+    tensors = tensors_for(raw, 5)
+    first = [helpers.random_tokens(1 + i % 3, raw["vocab_size"], 80 + i) for i in range(n_seqs)]
+    nxt = [[(17 * i + 3) % raw["vocab_size"], (29 * i + 5) % raw["vocab_size"]] for i in range(n_seqs)]
+    outs = {}
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine(build(raw, dtype, tensors), max_tokens=64 * n_seqs)
+        slots = [eng.open() for _ in first]
+        got = [eng.step([(s, p, [len(p) - 1]) for s, p in zip(slots[:12], first[:12])])]          # 24 tokens, 12 wanted
+        eng.step([(s, p, []) for s, p in zip(slots[12:], first[12:])])
+        for step in range(2):
+            got.append(eng.step([(s, [t[step]], [0]) for s, t in zip(slots, nxt)]))
+        outs[dtype] = torch.cat(got).cpu()
+        for s in slots:
+            eng.close(s)
+        del eng
+        torch.cuda.empty_cache()
+    scale = outs["float32"].abs().max().item()
+    assert 0.05 < scale < 50
+    torch.testing.assert_close(outs["bfloat16"], outs["float32"], atol=0.03 * max(1.0, scale), rtol=0.03)
+
+
 def test_float32_path_equals_plain_at_7b_sizes():
     raw = two_layer("qwen2.5:7b")
     tensors = tensors_for(raw, 4)
