@@ -507,7 +507,7 @@ def test_gated_product_of_17_to_64_rows(m, inter, k):
     torch.testing.assert_close(out.float(), act.float(), atol=2e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("m,n,k", [(40, 96, 2048), (64, 3584, 3584), (17, 100, 1056), (33, 2050, 1024)])
+@pytest.mark.parametrize("m,n,k", [(40, 96, 2048), (64, 3584, 3584), (17, 100, 1056), (33, 2050, 1024), (64, 3584, 18944)])
 def test_unfinished_sums_of_a_product_are_finished_by_the_next_norm(m, n, k):
     x, w = rand(m, k, seed=36, dtype=torch.bfloat16), rand(n, k, seed=37, scale=0.05, dtype=torch.bfloat16)
     packed = K.pack_weight(w)
@@ -519,16 +519,18 @@ def test_unfinished_sums_of_a_product_are_finished_by_the_next_norm(m, n, k):
     h1, h2 = h.clone(), h.clone()
     out1 = K.add_rmsnorm(h1, done, nw, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV), write_back=True)
     out2 = K.add_rmsnorm(h2, left, nw, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV), write_back=True)
-    assert torch.equal(h1, h2) and torch.equal(out1, out2)
+    assert torch.equal(h1, h2)                       # the same sums, rounded the same way, added the same way
     torch.testing.assert_close(h1, h + done.float(), atol=0, rtol=0)
+    # the norm's own sum of squares runs over more threads when it also adds up pieces: one bfloat16 step at most
+    torch.testing.assert_close(out1.float(), out2.float(), atol=1e-3, rtol=2 ** -7)
     # some rows only, h left as it is; and without a stream
     rows = ints([m - 1, 0, 5])
     g1 = K.add_rmsnorm(h, done, nw, 1e-6, torch.empty(3, n, dtype=torch.bfloat16, device=DEV), rows=rows)
     g2 = K.add_rmsnorm(h, left, nw, 1e-6, torch.empty(3, n, dtype=torch.bfloat16, device=DEV), rows=rows)
-    assert torch.equal(g1, g2)
+    torch.testing.assert_close(g1.float(), g2.float(), atol=1e-3, rtol=2 ** -7)
     n1 = K.add_rmsnorm(None, done, nw, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV))
     n2 = K.add_rmsnorm(None, left, nw, 1e-6, torch.empty(m, n, dtype=torch.bfloat16, device=DEV))
-    assert torch.equal(n1, n2)
+    torch.testing.assert_close(n1.float(), n2.float(), atol=1e-3, rtol=2 ** -7)
 
 
 @pytest.mark.parametrize("nh,nkv,d,k", [(28, 4, 128, 3584), (3, 1, 32, 2048), (6, 2, 64, 1056)])
