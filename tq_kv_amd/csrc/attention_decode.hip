@@ -59,6 +59,9 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     const int n_rep = n_heads / n_kv_heads;
     const int pos = tok_pos[seq];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    // exponentials to base 2 (one instruction each): the scores carry log2(e), and so do the running
+    // maxima m here, in part_ml and in the merge kernel
+    const float scale2 = scale * 1.4426950408889634f;
 
     // the query head of this lane's column
     const int rep = qb * 16 + col;
@@ -123,14 +126,14 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int j = key0 + t * 16 + g * 4 + r;
-                    const float v = (j >= lo && j <= pos) ? s[t][r] * scale : -INFINITY;
+                    const float v = (j >= lo && j <= pos) ? s[t][r] * scale2 : -INFINITY;
                     s[t][r] = v;
                     mx = fmaxf(mx, v);
                 }
             mx = fmaxf(mx, __shfl_xor(mx, 16, TQK_WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));
             // mx is finite: the page holds at least one key of [lo, pos]
-            const float alpha = expf(m - mx);
+            const float alpha = __builtin_amdgcn_exp2f(m - mx);     // 2^(-inf) = 0 on the wave's first page
             m = mx;
             float psum = 0.f;
             pack8 pb[2];
@@ -138,7 +141,7 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
             for (int t = 0; t < 4; ++t)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float p = s[t][r] == -INFINITY ? 0.f : expf(s[t][r] - mx);
+                    const float p = __builtin_amdgcn_exp2f(s[t][r] - mx);          // a masked key: 2^(-inf) = 0
                     // the probability enters the product as bfloat16; the sum uses the same rounded value
                     const uint16_t pbits = float_to_bf16_bits(p);
                     psum += __uint_as_float(((uint32_t)pbits) << 16);
@@ -185,7 +188,7 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
             const float m2 = theirs[DB * 4], l2 = theirs[DB * 4 + 1];
             if (m2 == -INFINITY) continue;
             const float mn = fmaxf(m, m2);
-            const float a1 = m == -INFINITY ? 0.f : expf(m - mn), a2 = expf(m2 - mn);
+            const float a1 = __builtin_amdgcn_exp2f(m - mn), a2 = __builtin_amdgcn_exp2f(m2 - mn);
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -231,7 +234,7 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_out, const
             const float2 s = ml[p];
             const float v = po[(size_t)p * head_dim];
             const bool live = s.x != -INFINITY;
-            const float wgt = live ? expf(s.x - M) : 0.f;
+            const float wgt = live ? __builtin_amdgcn_exp2f(s.x - M) : 0.f;
             denom += wgt * s.y;
             acc += live ? wgt * v : 0.f;
         }

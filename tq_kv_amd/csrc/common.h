@@ -14,11 +14,9 @@ struct bf16_t { uint16_t bits; };
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
 
+// Round to nearest even, NaN stays NaN: gfx950 has an instruction for it (v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);   // NaN stays NaN
-    u += 0x7fffu + ((u >> 16) & 1u);                                               // round to nearest even
-    return (uint16_t)(u >> 16);
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
 
 template <typename T> __device__ __forceinline__ T from_float(float v);
