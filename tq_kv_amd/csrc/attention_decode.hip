@@ -121,15 +121,25 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
             // mask, scale, running maximum (the lane's head is its column; its keys are
             // key0 + 16 t + 4 g + r)
             float mx = m;
+            if (edge) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < 4; ++t)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int j = key0 + t * 16 + g * 4 + r;
-                    const float v = (j >= lo && j <= pos) ? s[t][r] * scale2 : -INFINITY;
-                    s[t][r] = v;
-                    mx = fmaxf(mx, v);
-                }
+                    for (int r = 0; r < 4; ++r) {
+                        const int j = key0 + t * 16 + g * 4 + r;
+                        const float v = (j >= lo && j <= pos) ? s[t][r] * scale2 : -INFINITY;
+                        s[t][r] = v;
+                        mx = fmaxf(mx, v);
+                    }
+            } else {                                    // a page wholly inside [lo, pos]: nothing to mask
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        s[t][r] *= scale2;
+                        mx = fmaxf(mx, s[t][r]);
+                    }
+            }
             mx = fmaxf(mx, __shfl_xor(mx, 16, TQK_WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));
             // mx is finite: the page holds at least one key of [lo, pos]
