@@ -108,6 +108,7 @@ def tune_library(on=True, seconds=30):
     import torch.cuda.tunable as tunable
     tunable.enable(bool(on))
     tunable.tuning_enable(bool(on))
+    tunable.write_file_on_exit(False)           # what it finds is for this process; no file is left behind
     if on:
         tunable.set_max_tuning_duration(int(seconds * 1000))
         tunable.record_untuned_enable(False)
