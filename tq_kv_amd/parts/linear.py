@@ -108,7 +108,10 @@ def tune_library(on=True, seconds=30):
     import torch.cuda.tunable as tunable
     tunable.enable(bool(on))
     tunable.tuning_enable(bool(on))
-    tunable.write_file_on_exit(False)           # what it finds is for this process; no file is left behind
+    # what it finds is for this process: the file it may write when the process ends goes to the temp folder
+    import os
+    import tempfile
+    tunable.set_filename(os.path.join(tempfile.gettempdir(), "tq_kv_amd_tunableop_%d.csv" % os.getpid()))
     if on:
         tunable.set_max_tuning_duration(int(seconds * 1000))
         tunable.record_untuned_enable(False)
