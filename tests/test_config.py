@@ -104,3 +104,53 @@ def test_catalog_find():
     for name, tag in catalog.entries():
         config_from_dict(catalog.find("%s:%s" % (name, tag)))
     assert catalog.find("tiny:a") == TINY_A and catalog.find("tiny:b") == TINY_B
+
+
+# ---- stop tokens of a model folder (src/engine.rs:301-316) ---------------------------------------
+def _folder_with(tmp_path, config_eos=None, generation=None, tokenizer=None):
+    raw = dict(TINY_A)
+    if config_eos is not None:
+        raw["eos_token_id"] = config_eos
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    if generation is not None:
+        (tmp_path / "generation_config.json").write_text(json.dumps(generation))
+    if tokenizer is not None:
+        (tmp_path / "tokenizer.json").write_text(json.dumps(tokenizer))
+    return str(tmp_path)
+
+
+def test_stop_tokens_are_the_union_of_every_place_that_names_them(tmp_path):
+    from tq_kv_amd.config.generation import stop_token_ids
+    folder = _folder_with(
+        tmp_path, config_eos=7, generation={"eos_token_id": [9, 7], "temperature": 0.7},
+        tokenizer={"added_tokens": [{"id": 9, "content": "<|im_end|>"}, {"id": 11, "content": "<|endoftext|>"},
+                                    {"id": 12, "content": "<|im_start|>"}],
+                   "model": {"vocab": {"</s>": 2, "a": 3}}})
+    cfg = load_config(folder)[1]
+    assert cfg.eos_token_ids == (7,)
+    # config.json first, then generation_config.json, then the reference's stop strings; each once
+    assert stop_token_ids(folder, cfg.eos_token_ids) == (7, 9, 11, 2)
+
+
+def test_stop_tokens_of_each_place_alone(tmp_path):
+    from tq_kv_amd.config.generation import stop_token_ids
+    a, b, c, d = [tmp_path / n for n in "abcd"]
+    for p in (a, b, c, d):
+        p.mkdir()
+    assert stop_token_ids(_folder_with(a)) == ()                       # random weights: none, no fallback id
+    assert stop_token_ids(_folder_with(b, generation={"eos_token_id": 5})) == (5,)
+    assert stop_token_ids(_folder_with(c, generation={"max_new_tokens": 3})) == ()
+    with pytest.raises(ConfigError, match="generation_config.json.*eos_token_id"):
+        stop_token_ids(_folder_with(d, generation={"eos_token_id": "x"}))
+    (d / "generation_config.json").write_text("{ not json")
+    with pytest.raises(ConfigError, match="Invalid generation_config.json"):
+        stop_token_ids(str(d))
+
+
+def test_a_loaded_model_carries_its_folders_stop_tokens(tmp_path):
+    from tq_kv_amd import Model
+    folder = Model.write_random_folder(str(tmp_path / "m"), dict(TINY_A, eos_token_id=3), seed=0)
+    with open(tmp_path / "m" / "generation_config.json", "w") as f:
+        json.dump({"eos_token_id": [3, 200]}, f)
+    model = Model.from_dir(folder, dtype="float32", device="cpu")
+    assert model.spec.eos_token_ids == (3,) and model.stop_token_ids == (3, 200)

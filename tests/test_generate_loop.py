@@ -235,3 +235,14 @@ def test_running_ahead_wastes_one_row_on_a_stop_token():
     # request 0's stop token 99 was fed once, because the step was started before it was read
     assert eng.steps[3] == [(0, [99]), (1, [22])] and eng.steps[4] == [(1, [23])]
     assert eng.seen == {}
+
+
+def test_stop_tokens_default_to_those_the_model_names():
+    class Named(FakeEngine):
+        class model:
+            stop_token_ids = (99,)
+    make = lambda p, ids: ScriptSampler([[10, 99, 12]], ids)
+    params = GenerationParams(max_tokens=8, temperature=0.0)
+    assert generate(Named(), [[1]], params, make_sampler=make) == [[10]]
+    assert generate(Named(), [[1]], params, eos_ids=(), make_sampler=lambda p, ids: ScriptSampler([[10, 99, 12] + [1] * 8], ids))[0][:3] == [10, 99, 12]
+    assert generate(FakeEngine(), [[1]], GenerationParams(max_tokens=3, temperature=0.0), make_sampler=make) == [[10, 99, 12]]

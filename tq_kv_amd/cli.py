@@ -54,7 +54,7 @@ def build_parser():
     g.add_argument("--prompt-file", help="A file with one prompt per line, as token ids")
     g.add_argument("--prompt", action="append", default=[], help="A prompt as text (needs tokenizer.json in the model folder)")
     g.add_argument("-s", "--system", default=None, help="System prompt: wrap text prompts in the chat template")
-    g.add_argument("--eos", default=None, help="Stop token ids, e.g. 151645,151643 (default: eos_token_id of config.json)")
+    g.add_argument("--eos", default=None, help="Stop token ids, e.g. 151645,151643 (default: eos_token_id of config.json and generation_config.json, stop strings of tokenizer.json)")
     g.add_argument("--json", action="store_true", help="Output results as JSON")
     _add_sampling(g, 512)
     b = sub.add_parser("bench", help="Run a generation benchmark")
@@ -118,7 +118,7 @@ def cmd_generate(args):
     model = load_model(args.model, args.dtype, args.weights_seed)
     params = GenerationParams(max_tokens=args.max_tokens, temperature=args.temperature, top_p=args.top_p,
                               top_k=args.top_k, repeat_penalty=args.repeat_penalty, seed=args.seed)
-    eos = _ids(args.eos) if args.eos is not None else list(model.spec.eos_token_ids)
+    eos = _ids(args.eos) if args.eos is not None else list(model.stop_token_ids)
     # room for one batch of the generation loop (at most 64 requests at a time)
     rooms = sorted(((len(p) + args.max_tokens + PAGE - 1) // PAGE * PAGE for p in prompts), reverse=True)
     engine = Engine(model, max_tokens=args.max_cache_tokens or sum(rooms[:64]))

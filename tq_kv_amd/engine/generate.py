@@ -45,16 +45,19 @@ def plan_batches(prompt_lens, max_new, max_tokens, max_batch):
     return batches
 
 
-def generate(engine, prompts, params=None, eos_ids=(), on_tokens=None, max_batch=64, make_sampler=None,
+def generate(engine, prompts, params=None, eos_ids=None, on_tokens=None, max_batch=64, make_sampler=None,
              max_step_tokens=8192):
     """prompts: token-id lists.  Returns for each prompt the emitted token ids.
 
-    eos_ids: stop tokens.  on_tokens(pairs): called after every step with the
+    eos_ids: stop tokens (default: those the engine's model names, Model.stop_token_ids; give ()
+    for none).  on_tokens(pairs): called after every step with the
     (request index, token) pairs emitted by it.  make_sampler(params, request_ids): the
     sampler of a batch (default: the device sampler).  max_step_tokens: most tokens one step
     runs; a batch's prompts are fed in as many steps as that takes (whole prompts together
     while they fit, a longer prompt in pieces), which bounds the step's working memory."""
     params = params or GenerationParams()
+    if eos_ids is None:
+        eos_ids = getattr(getattr(engine, "model", None), "stop_token_ids", ())
     eos = set(int(t) for t in eos_ids)
     prompts = [list(p) for p in prompts]
     for i, p in enumerate(prompts):

@@ -8,6 +8,7 @@ import torch
 from .. import kernels as K
 from ..config import catalog
 from ..config.base import ConfigError, read_config_json
+from ..config.generation import stop_token_ids
 from ..config.registry import config_from_dict, spec_for
 from ..parts import linear as L
 from ..parts.linear import linear
@@ -29,6 +30,8 @@ class Model:
     def __init__(self, spec, dtype="bfloat16", device="cuda", config=None):
         self.spec = spec
         self.config = config
+        # stop tokens: what the configuration names; a model folder may add more (from_dir)
+        self.stop_token_ids = tuple(spec.eos_token_ids)
         self.dtype = run_dtype(dtype)
         self.device = torch.device(device)
         self.env = BuildEnv(self.device, self.dtype)
@@ -91,6 +94,7 @@ class Model:
     def from_dir(cls, model_dir, dtype="bfloat16", device="cuda"):
         """A model folder: config.json picks the architecture, *.safetensors hold the weights."""
         model = cls.from_config_dict(read_config_json(model_dir), dtype, device)
+        model.stop_token_ids = stop_token_ids(model_dir, model.spec.eos_token_ids)
         return model.load(load_folder(model_dir, model.tensor_specs(), model.dtype, model.device))
 
     @classmethod
