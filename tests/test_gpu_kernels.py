@@ -818,3 +818,39 @@ def test_fused_kernels_refuse_what_they_do_not_take():
         K.fused_store(rand(17, 64, dtype=torch.bfloat16), w, torch.empty(17, 16, device=DEV))
     with pytest.raises(K.KernelError, match="multiple of 32"):
         K.fused_store(rand(2, 48, dtype=torch.bfloat16), rand(16, 48, dtype=torch.bfloat16), torch.empty(2, 16, device=DEV))
+
+
+# ---- random weights: the same bits on the host and on the GPU ------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_random_normal_on_the_gpu_equals_the_hosts_bit_for_bit(dtype):
+    import numpy as np
+    from tq_kv_amd.weights.random_init import standard_normal_host, tensor_key
+    key = tensor_key(11, "some.weight")
+    n = 3_000_001
+    for std, plus_one in ((0.02, False), (0.02, True), (1.0, False)):
+        out = K.random_normal(torch.empty((n,), dtype=dtype, device="cuda"), key, std, plus_one)
+        want = standard_normal_host(key, 0, n) * np.float32(std)
+        if plus_one:
+            want = np.float32(1.0) + want
+        want = torch.from_numpy(want).to(dtype)
+        got = out.cpu()
+        view = torch.int32 if dtype == torch.float32 else torch.int16
+        bad = (got.view(view) != want.view(view)).nonzero()
+        assert bad.numel() == 0, "first difference at element %d: %r vs %r" % (bad[0], got[bad[0]], want[bad[0]])
+
+
+def test_a_random_model_on_the_gpu_equals_the_folder_the_host_writes(tmp_path):
+    """Model.random on the GPU and write_random_folder on the host: one seed, one model."""
+    from safetensors.torch import load_file
+    from tq_kv_amd import Model
+    from tq_kv_amd.weights import random_tensors
+    import helpers
+    for name, (cfg, seed) in helpers.CONFIGS.items():
+        for store in (torch.bfloat16, torch.float32):
+            folder = Model.write_random_folder(str(tmp_path / ("%s_%s" % (name, store))), cfg, seed=seed, store_dtype=store)
+            stored = load_file(folder + "/model.safetensors")
+            specs = Model.from_config_dict(cfg, "float32", "cpu").tensor_specs()
+            made = random_tensors(specs, seed, store, "cuda")
+            assert set(made) == set(stored)
+            for k in stored:
+                assert torch.equal(made[k].cpu(), stored[k]), k

@@ -113,6 +113,24 @@ def test_random_folder_is_seeded_and_has_the_stated_distributions(tmp_path):
     assert "lm_head.weight" not in tied and torch.equal(tied["model.norm.weight"], a["model.norm.weight"])
 
 
+def test_random_stream_is_a_function_of_key_and_index_alone():
+    """Element i is the same whatever piece of the stream is asked for; the values are standard
+    normal (moments and a Kolmogorov-Smirnov distance), bounded by sqrt(48 ln 2), never NaN."""
+    import numpy as np
+    from tq_kv_amd.weights.random_init import standard_normal_host, tensor_key
+    key = tensor_key(3, "model.embed_tokens.weight")
+    assert key == tensor_key(3, "model.embed_tokens.weight") != tensor_key(4, "model.embed_tokens.weight")
+    whole = standard_normal_host(key, 0, 5000)
+    pieces = np.concatenate([standard_normal_host(key, 0, 1), standard_normal_host(key, 1, 1999), standard_normal_host(key, 2000, 3000)])
+    assert whole.dtype == np.float32 and np.array_equal(whole.view(np.int32), pieces.view(np.int32))
+    assert not np.array_equal(whole, standard_normal_host(key + 1, 0, 5000))
+    z = standard_normal_host(key, 0, 400000).astype(np.float64)
+    assert np.isfinite(z).all() and np.abs(z).max() < 5.78
+    assert abs(z.mean()) < 0.006 and abs(z.std() - 1) < 0.005 and abs((z ** 3).mean()) < 0.02 and abs((z ** 4).mean() - 3) < 0.05
+    from scipy import stats
+    assert stats.kstest(z, "norm").statistic < 0.003
+
+
 def test_model_lists_tensors_by_the_reference_names():
     names = set(Model.from_config_dict(TINY_A, "float32", "cpu").tensor_specs())
     want = {"model.embed_tokens.weight", "model.norm.weight"}

@@ -18,7 +18,7 @@ import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["host.cpp", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip",
-           "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip"]
+           "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip", "random_init.hip"]
 HEADERS = ["common.h", "tq_kernels.h"]
 ARCH = "gfx950"
 # Packed float32 instructions are switched off for all device code.

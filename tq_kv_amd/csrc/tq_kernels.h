@@ -25,6 +25,11 @@ int tqk_embed(const void* table, int table_dtype, const int32_t* ids, int n_toke
               int hidden, int vocab, float* out, void* copy_bf16, const void* copy_weight,
               float* ss_out, void* stream);
 
+/* out[i] = std_dev * z(key, i) (+ 1 if plus_one), i < n: standard normal values that are a
+ * function of the 64-bit key and the index alone, the same bits as the host's recipe gives
+ * (tq_kv_amd/weights/random_init.py).  out: float32 or bfloat16 (rounded to nearest even). */
+int tqk_random_normal(void* out, int dtype, long long n, uint64_t key, float std_dev, int plus_one, void* stream);
+
 /* Row r (row index rows[r], or r if rows is NULL):
  *   v = (h ? h[row] : 0) + (delta ? delta[row] : 0);  if write_back: h[row] = v;
  *   out[r] = v / sqrt(mean(v^2) + eps) * weight          (all in float32)

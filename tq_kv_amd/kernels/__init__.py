@@ -95,6 +95,15 @@ def embed(table, ids, out, copy=None, copy_weight=None, ss_out=None):
     return out
 
 
+def random_normal(out, key, std, plus_one=False):
+    """out (float32 or bfloat16, any shape) = std * z(key, i) (+ 1): the stream of
+    weights.random_init for the 64-bit key, element i in the tensor's row-major order."""
+    _check(library().tqk_random_normal(_dev(out, "out"), _code(out.dtype), ctypes.c_longlong(out.numel()),
+                                       ctypes.c_uint64(int(key) & 0xFFFFFFFFFFFFFFFF), ctypes.c_float(std),
+                                       1 if plus_one else 0, _stream()), "random_normal")
+    return out
+
+
 def add_rmsnorm(h, delta, weight, eps, out, rows=None, write_back=False):
     """out = rmsnorm(h + delta) * weight; with write_back h becomes h + delta.
 
