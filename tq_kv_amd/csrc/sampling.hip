@@ -93,6 +93,62 @@ extern "C" int tqk_argmax(const float* logits, int n_rows, int vocab, int32_t* o
     return tqk_check_launch("tqk_argmax final");
 }
 
+// ---- argmax without a caller's scratch -------------------------------------------------------
+// The same two kernels with the chunks' best values and indices in an array that is part of
+// the library's image on every GPU it runs on (the process holds it until it ends), so the
+// call needs no device memory beyond its input and output.  Host code reaches the array only
+// through the address that hipGetSymbolAddress gives on the GPU that is current; every GPU
+// has its own copy at its own address.
+#define AM_STATIC_MAX_PAIRS 16384        // rows * chunks of a call, at most (128 KiB)
+#define AM_STATIC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[AM_STATIC_MAX_PAIRS * 8];
+
+#include <mutex>
+static std::mutex g_static_mutex;
+static void* g_static_ptr[AM_STATIC_MAX_DEVICES];        // per GPU: where its copy of the array lies
+
+// The current GPU's address of the array, or null with the error recorded.
+static void* static_scratch_of_current_device(const char* who) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { tqk_fail("%s: hipGetDevice: %s", who, hipGetErrorString(e)); return nullptr; }
+    if (dev < 0 || dev >= AM_STATIC_MAX_DEVICES) { tqk_fail("%s: GPU %d is beyond the %d this library keeps scratch for", who, dev, AM_STATIC_MAX_DEVICES); return nullptr; }
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) { tqk_fail("%s: hipGetSymbolAddress on GPU %d: %s", who, dev, hipGetErrorString(e)); return nullptr; }
+        g_static_ptr[dev] = ptr;
+    }
+    return g_static_ptr[dev];
+}
+
+extern "C" int tqk_argmax_static_max_pairs(void) { return AM_STATIC_MAX_PAIRS; }
+
+extern "C" int tqk_argmax_static_prepare(void) {
+    return static_scratch_of_current_device("tqk_argmax_static_prepare") ? 0 : -1;
+}
+
+extern "C" int tqk_argmax_static(const float* logits, int n_rows, int vocab, int32_t* out, void* stream) {
+    TQK_REQUIRE(logits && out, "tqk_argmax_static: null pointer");
+    TQK_REQUIRE(n_rows >= 0 && vocab > 0, "tqk_argmax_static: bad sizes rows=%d vocab=%d", n_rows, vocab);
+    if (n_rows == 0) return 0;
+    const int n_chunks = (vocab + AM_CHUNK - 1) / AM_CHUNK;
+    TQK_REQUIRE((long long)n_rows * n_chunks <= AM_STATIC_MAX_PAIRS,
+                "tqk_argmax_static: %d rows of %d chunks of %d need %lld scratch entries, the library holds %d (use tqk_argmax with a scratch buffer of your own)",
+                n_rows, n_chunks, AM_CHUNK, (long long)n_rows * n_chunks, AM_STATIC_MAX_PAIRS);
+    void* ptr = static_scratch_of_current_device("tqk_argmax_static");
+    if (!ptr) return -1;
+    // every entry the second kernel reads is written by the first: nothing has to start at zero
+    float* best_v = reinterpret_cast<float*>(ptr);
+    int32_t* best_i = reinterpret_cast<int32_t*>(best_v + (size_t)n_rows * n_chunks);
+    hipStream_t s = (hipStream_t)stream;
+    argmax_chunk_kernel<<<dim3(n_chunks, n_rows), AM_THREADS, 0, s>>>(logits, vocab, n_chunks, best_v, best_i);
+    if (tqk_check_launch("tqk_argmax_static")) return -1;
+    argmax_final_kernel<<<n_rows, AM_THREADS, 0, s>>>(best_v, best_i, n_chunks, out);
+    return tqk_check_launch("tqk_argmax_static final");
+}
+
 // ---- helpers for one-block-per-row passes ---------------------------------------
 // Order-preserving map from float to unsigned: a < b  <=>  key(a) < key(b).
 __device__ __forceinline__ uint32_t float_key(float f) {

@@ -149,6 +149,20 @@ int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int 
 int tqk_argmax_scratch_floats(int n_rows, int vocab);
 int tqk_argmax(const float* logits, int n_rows, int vocab, int32_t* out, float* scratch, void* stream);
 
+/* tqk_argmax for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
+ * chunks' results go to an array inside the library's image on the current GPU (128 KiB per GPU,
+ * held until the process ends) in place of a caller's scratch; n_rows * ceil(vocab / 4096) must
+ * not exceed tqk_argmax_static_max_pairs() (16384), more is refused with an error.  It calls no
+ * hipMalloc, hipFree or allocating library routine.  Every call on a GPU shares that GPU's array:
+ * calls that overlap in time on one GPU (different streams or threads) race; calls on one stream
+ * are ordered.  The GPU whose stream is given must be the current one.  The array's address is
+ * looked up at the first call on each GPU; tqk_argmax_static_prepare() does that lookup for the
+ * current GPU ahead of time (call it before a graph capture that will hold tqk_argmax_static). */
+int tqk_argmax_static_max_pairs(void);
+int tqk_argmax_static_prepare(void);
+int tqk_argmax_static(const float* logits, int n_rows, int vocab, int32_t* out, void* stream);
+
 /* In place: for every token in the history of the row's request, once per occurrence,
  * l > 0 ? l / penalty : l * penalty.  hist, times [n_req, hist_cap], hist_len [n_req]: the
  * history as tqk_append_history keeps it (times: for each entry how often the penalty is
