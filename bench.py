@@ -4,7 +4,13 @@ one MI355X: `python bench.py [--gpus 1] [--steps K] [--warmup W]` prints one JSO
 A step is one decode step of the whole batch through the generation loop (step
 function, sampling, host round trip for the stop check).  The reference measures
 tokens per second of one chat request including its prompt (src/main.rs:1123-1143);
-here decoding is timed alone and the prompt pass is reported beside it.
+here decoding is timed alone, the prompt pass is reported beside it, and the reference's
+prompt-inclusive figure goes into `end_to_end_tok_per_s`.
+
+Other workloads of the same bench, each one command and one line:
+  --workload 1.5b-mixed   Qwen2.5-1.5B shape, 32 prompts of 16..1024 tokens, 128 sampled steps
+  --workload 32b          Qwen2.5-32B shape, 16 prompts of 512 tokens, 256 greedy steps
+  --prompt-len N          other contexts of the default workload (8192, 16384, ...)
 """
 import argparse
 import json
@@ -12,24 +18,35 @@ import sys
 import time
 
 PEAK = {"hbm_gbs": 8000.0, "bf16_flops": 2.5e15}     # MI355X: HBM3E 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s
-SHAPE = "qwen2.5:7b"
+# shape, batch, prompt length, steps, warm-up steps; mixed: unequal prompts, sampled; no_points: headline only
+WORKLOADS = {
+    "7b": dict(shape="qwen2.5:7b", batch=8, prompt_len=2048, steps=128, warmup=16),
+    "1.5b-mixed": dict(shape="qwen2.5:1.5b", batch=32, prompt_len=1024, steps=128, warmup=16, mixed=True),
+    "32b": dict(shape="qwen2.5:32b", batch=16, prompt_len=512, steps=256, warmup=8, no_points=True),
+}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
-    ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--prompt-len", type=int, default=2048)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--batch", type=int, default=None)
+    ap.add_argument("--prompt-len", type=int, default=None)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="7b",
+                    help="a preset of shape, batch, prompt length, steps and sampling; the other options override it")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
-    ap.add_argument("--shape", default=SHAPE)
+    ap.add_argument("--shape", default=None)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--no-tune", action="store_true", help="do not let the library pick its fastest kernel per product shape")
     ap.add_argument("--mixed", action="store_true",
                     help="another workload instead: --batch prompts of unequal lengths (uniform in 16..--prompt-len), sampled with "
                          "the default parameters (temperature 0.7, top-k 40, top-p 0.9, repeat penalty 1.1); prints its own line")
     args = ap.parse_args()
+    preset = WORKLOADS[args.workload]
+    for key, value in preset.items():
+        if getattr(args, key) in (None, False):
+            setattr(args, key, value)
     if args.gpus != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not supported" % args.gpus)
         return 2
@@ -105,25 +122,37 @@ def main():
                 marks[calls[0]] = time.perf_counter()
             calls[0] += 1
         params = GenerationParams(max_tokens=warmup + steps + 2, temperature=0.0, repeat_penalty=1.0)
-        out = generate(engine, prompts(batch), params, on_tokens=on_tokens, max_batch=batch)
+        ps = prompts(batch)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = generate(engine, ps, params, on_tokens=on_tokens, max_batch=batch)
+        torch.cuda.synchronize()
+        whole = time.perf_counter() - t0
         assert all(len(o) == warmup + steps + 2 for o in out)
         seconds = marks[warmup + steps] - marks[warmup]
-        return batch * steps / seconds, seconds / steps
-
-    note("decode at batch %d" % args.batch)
-    tps, sec_per_step = decode(args.batch, args.steps, args.warmup)
-    points = {}
-    if not args.no_points:
-        note("decode at batch 1")
-        points["decode_b1"] = round(decode(1, min(args.steps, 64), 8)[0], 1)
-        note("decode at batch 64")
-        points["decode_b64"] = round(decode(64, min(args.steps, 32), 4)[0], 1)
-    note("done")
+        return batch * steps / seconds, seconds / steps, sum(len(o) for o in out) / whole
 
     weight_bytes = 2.0 * (linear_params + H * V)                      # every weight the step uses, once
-    mean_ctx = args.prompt_len + args.warmup + args.steps / 2.0
-    kv_bytes = args.batch * mean_ctx * layers * 2 * nkv * d * 2.0        # keys and values of the live requests
-    achieved = (weight_bytes + kv_bytes) / sec_per_step / 1e9
+
+    def hbm(batch, steps, warmup, sec_per_step):
+        """GB/s of a decode step: the weights once and the cache of the live requests, over its time."""
+        mean_ctx = args.prompt_len + warmup + steps / 2.0
+        kv_bytes = batch * mean_ctx * layers * 2 * nkv * d * 2.0
+        return (weight_bytes + kv_bytes) / sec_per_step / 1e9
+
+    note("decode at batch %d" % args.batch)
+    tps, sec_per_step, end_to_end = decode(args.batch, args.steps, args.warmup)
+    points = {}
+    if not args.no_points:
+        for batch, steps, warmup in ((1, min(args.steps, 64), 8), (64, min(args.steps, 32), 4)):
+            note("decode at batch %d" % batch)
+            b_tps, b_sec, _ = decode(batch, steps, warmup)
+            gbs = hbm(batch, steps, warmup, b_sec)
+            name = "decode_b%d" % batch
+            points.update({name: round(b_tps, 1), name + "_ms": round(b_sec * 1e3, 4), name + "_gbs": round(gbs, 1),
+                           name + "_frac": round(gbs / PEAK["hbm_gbs"], 4)})
+    note("done")
+    achieved = hbm(args.batch, args.steps, args.warmup, sec_per_step)
     line = {
         "metric": "decode tok/s @ batch %d, %s shape" % (args.batch, args.shape), "value": round(tps, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 4),
@@ -137,6 +166,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK["hbm_gbs"], "unit": "GB/s",
                      "frac": round(achieved / PEAK["hbm_gbs"], 4)},
         "points": points,
+        # the reference's figure: generated tokens over the whole run, prompt pass included (src/main.rs:1139-1143)
+        "end_to_end_tok_per_s": round(end_to_end, 1),
     }
     print(json.dumps(line))
     return 0

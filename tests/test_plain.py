@@ -197,6 +197,22 @@ def test_swiglu():
     torch.testing.assert_close(plain.swiglu_mlp(x, w, ""), want, rtol=1e-5, atol=1e-6)
 
 
+def test_silu_acts_on_the_gate_projection_not_on_up():
+    # src/models/turbo_generic.rs:105-111: down(silu(gate(x)) * up(x)).  A gate that is large and
+    # negative everywhere closes the feed-forward whatever up gives; with the roles swapped
+    # (silu on up, times gate) the same weights would give something huge instead.
+    x = rand(4, 8, seed=27).abs() + 0.5
+    w = {"gate_proj.weight": -10.0 * torch.ones(6, 8), "up_proj.weight": rand(6, 8, seed=28),
+         "down_proj.weight": rand(8, 6, seed=29)}
+    assert plain.swiglu_mlp(x, w, "").abs().max().item() < 1e-10
+    swapped = F.linear(F.silu(F.linear(x, w["up_proj.weight"])) * F.linear(x, w["gate_proj.weight"]), w["down_proj.weight"])
+    assert swapped.abs().max().item() > 1.0
+    # and the other way round: a wide-open gate passes up(x) times gate(x)
+    w["gate_proj.weight"] = 10.0 * torch.ones(6, 8)
+    g, u = F.linear(x, w["gate_proj.weight"]), F.linear(x, w["up_proj.weight"])
+    torch.testing.assert_close(plain.swiglu_mlp(x, w, ""), F.linear(g * u, w["down_proj.weight"]), rtol=1e-5, atol=1e-5)
+
+
 # ---- the whole model -----------------------------------------------------------------------
 def test_norms_sit_before_mixer_and_feed_forward():
     # with o_proj and down_proj zero every layer adds nothing: logits = head(norm(embedding)).
@@ -210,6 +226,78 @@ def test_norms_sit_before_mixer_and_feed_forward():
     e = w["model.embed_tokens.weight"][toks]
     want = plain.linear(plain.rms_norm(e, w["model.norm.weight"], cfg["rms_norm_eps"]), w["lm_head.weight"])
     torch.testing.assert_close(plain.forward(w, cfg, toks), want, rtol=1e-5, atol=1e-6)
+
+
+def test_each_norm_weight_acts_at_its_own_site():
+    # src/models/turbo_generic.rs:1959-1981: input_layernorm feeds the mixer, post_attention_layernorm
+    # the feed-forward.  One layer, one token (attention over a single key returns its value), norm
+    # weights that are distinct constants: the logits show which weight sat where.
+    cfg = dict(TINY_A, num_hidden_layers=1)
+    w = tiny_weights(cfg, seed=31, std=0.3)
+    p = "model.layers.0."
+    a, b = 3.0, 0.25
+    w[p + "input_layernorm.weight"] = torch.full((cfg["hidden_size"],), a)
+    w[p + "post_attention_layernorm.weight"] = torch.full((cfg["hidden_size"],), b)
+    eps, tok = cfg["rms_norm_eps"], [17]
+    x0 = w["model.embed_tokens.weight"][tok]
+    unit = lambda x: x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+    head = lambda x: F.linear(unit(x) * w["model.norm.weight"], w["model.embed_tokens.weight"])
+    n_rep = cfg["num_attention_heads"] // cfg["num_key_value_heads"]
+
+    def mixer(scale):
+        v = F.linear(unit(x0) * scale, w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"])
+        v = v.reshape(1, cfg["num_key_value_heads"], cfg["head_dim"]).repeat_interleave(n_rep, dim=1).reshape(1, -1)
+        return F.linear(v, w[p + "self_attn.o_proj.weight"])
+
+    def ff(x, scale):
+        h = unit(x) * scale
+        return F.linear(F.silu(F.linear(h, w[p + "mlp.gate_proj.weight"])) * F.linear(h, w[p + "mlp.up_proj.weight"]),
+                        w[p + "mlp.down_proj.weight"])
+    x1 = x0 + mixer(a)
+    want = head(x1 + ff(x1, b))
+    got = plain.forward(w, cfg, tok)
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5)
+    x1s = x0 + mixer(b)
+    swapped = head(x1s + ff(x1s, a))
+    assert (swapped - want).abs().max().item() > 0.05              # the other placing is far away
+
+
+def test_qkv_have_biases_and_the_output_projection_has_none():
+    # src/models/turbo_generic.rs:2103-2105 (q, k, v biases), :2094 and :2139 (o_proj: weight only).
+    # With zero projection weights every key is equal, every value is the v bias: the mixer's
+    # output is o_proj(v bias repeated over the heads of its group) for every token, and nothing
+    # is added after o_proj.
+    cfg = dict(TINY_B)
+    w = tiny_weights(cfg, seed=32)
+    p = "model.layers.0.self_attn."
+    for name in ("q_proj.weight", "k_proj.weight", "v_proj.weight"):
+        w[p + name].zero_()
+    x = rand(7, cfg["hidden_size"], seed=33)
+    n_rep = cfg["num_attention_heads"] // cfg["num_key_value_heads"]
+    bias = w[p + "v_proj.bias"].reshape(cfg["num_key_value_heads"], cfg["head_dim"]).repeat_interleave(n_rep, dim=0).reshape(-1)
+    want = F.linear(bias, w[p + "o_proj.weight"]).expand(7, -1)
+    torch.testing.assert_close(plain.attention(x, w, p, cfg, None), want, rtol=1e-5, atol=1e-6)
+    assert want.abs().max().item() > 1e-3
+    # without the biases the same weights would give exactly nothing
+    w[p + "v_proj.bias"].zero_()
+    assert plain.attention(x, w, p, cfg, None).abs().max().item() == 0.0
+    # an o_proj.bias is not looked up: planting one changes nothing
+    w[p + "o_proj.bias"] = torch.ones(cfg["hidden_size"])
+    assert plain.attention(x, w, p, cfg, None).abs().max().item() == 0.0
+
+
+def test_max_window_layers_decides_which_layers_are_windowed():
+    # layer l is windowed iff l >= max_window_layers: 0, 1 and 3 of tiny B's three layers give
+    # three different models at a position beyond the window, and the same model inside it
+    cfg = dict(TINY_B)
+    w = tiny_weights(cfg, seed=34, std=0.2)
+    toks = [(7 * i + 3) % cfg["vocab_size"] for i in range(41)]
+    outs = [plain.forward(w, dict(cfg, max_window_layers=m), toks) for m in (0, 1, 3)]
+    for i in range(3):
+        for j in range(i + 1, 3):
+            assert (outs[i][40] - outs[j][40]).abs().max().item() > 1e-4
+            torch.testing.assert_close(outs[i][:cfg["sliding_window"]], outs[j][:cfg["sliding_window"]])
+    torch.testing.assert_close(outs[2], plain.forward(w, dict(cfg, use_sliding_window=False), toks))
 
 
 def test_tied_and_untied_head():
