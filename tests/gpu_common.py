@@ -13,10 +13,15 @@ _FOLDERS = {}
 _PLAIN = {}
 _ENGINES = {}
 
-# Largest allowed |engine - plain| on logits whose own size is about 1.  The float32
-# path differs from the plain implementation only by the order of float32 additions;
-# the bfloat16 path rounds weights' products of bfloat16 activations at every layer.
+# Largest allowed |engine - plain|.  The float32 path differs from the plain implementation
+# only by the order of float32 additions.  The bfloat16 path rounds activations at every
+# kernel boundary; its allowance is tied to the logits' own spread (their standard deviation,
+# 0.16 to 0.25 for the tiny models): measured, a clean run stays below 0.06 of it on every
+# configuration, while one cache page taken from another sequence moves the logits by 0.17 of
+# it or more (test_a_foreign_page_in_the_cache_is_noticed asserts that such a fault fails).
 TOL = {"float32": dict(atol=2e-5, rtol=2e-5), "bfloat16": dict(atol=3e-2, rtol=3e-2)}
+BF16_SPREAD = 0.1        # bfloat16: atol = BF16_SPREAD * std(reference), rtol = BF16_RTOL
+BF16_RTOL = 0.02
 
 
 def tmp():
@@ -80,7 +85,12 @@ def prompts(name, lens, seed=100):
 
 
 def close(a, b, dtype, what=""):
-    torch.testing.assert_close(a.cpu().float(), b.cpu().float(), msg=lambda m: "%s: %s" % (what, m), **TOL[dtype])
+    """a: the engine's logits, b: the reference's."""
+    a, b = a.cpu().float(), b.cpu().float()
+    tol = TOL[dtype]
+    if dtype == "bfloat16" and b.numel() > 1:
+        tol = dict(atol=BF16_SPREAD * b.std().item(), rtol=BF16_RTOL)
+    torch.testing.assert_close(a, b, msg=lambda m: "%s: %s" % (what, m), **tol)
 
 
 def poison_free_pages(eng):

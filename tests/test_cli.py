@@ -48,3 +48,38 @@ def test_tq_generate_runs_and_is_greedy_reproducible():
     assert json.loads(b.stdout.strip().splitlines()[-1])["outputs"] == res["outputs"]
     c = subprocess.run(cmd[:-1] + ["--eos", str(res["outputs"][0][2])], capture_output=True, text=True)
     assert c.returncode == 0 and c.stdout.splitlines()[0].split(": ")[1].split() == [str(t) for t in res["outputs"][0][:2]]
+
+
+@pytest.mark.gpu
+def test_tq_generate_on_a_folder_written_by_tq_random_weights_emits_the_plain_tokens(tmp_path):
+    """`tq random-weights` writes a folder, `tq generate <folder>` loads it and generates; the
+    tokens it prints are the plain implementation's greedy tokens for the same folder, and a stop
+    id that only generation_config.json names ends a request without being printed."""
+    import helpers
+    import plain_qwen2 as plain
+    tq = [sys.executable, os.path.join(ROOT, "bin", "tq")]
+    cfg_path = tmp_path / "shape.json"
+    cfg_path.write_text(json.dumps(helpers.TINY_B))
+    folder = str(tmp_path / "model")
+    w = subprocess.run(tq + ["random-weights", str(cfg_path), folder, "--seed", "5", "--store", "float32"],
+                       capture_output=True, text=True)
+    assert w.returncode == 0 and os.path.exists(os.path.join(folder, "model.safetensors")), w.stderr
+    cfg, weights = helpers.read_folder(folder)
+    prompts = [[1, 2, 3], [9, 8, 7, 6, 5, 300, 12]]
+    want = [plain.generate_greedy(weights, cfg, p, 7) for p in prompts]
+    cmd = tq + ["--fp32", "generate", folder, "--prompt-ids", "1,2,3", "--prompt-ids", "9 8 7 6 5 300 12", "-n", "7", "-t", "0",
+                "--repeat-penalty", "1.0", "--json"]
+    a = subprocess.run(cmd, capture_output=True, text=True)
+    assert a.returncode == 0, a.stderr
+    assert json.loads(a.stdout.strip().splitlines()[-1])["outputs"] == want
+    # the same through the text output, one line per request
+    b = subprocess.run(cmd[:-1], capture_output=True, text=True)
+    assert [line.split(": ")[1].split() for line in b.stdout.strip().splitlines()] == [[str(t) for t in o] for o in want]
+    # a stop token named by generation_config.json alone
+    stop = want[1][3]
+    with open(os.path.join(folder, "generation_config.json"), "w") as f:
+        json.dump({"eos_token_id": [stop]}, f)
+    c = subprocess.run(cmd, capture_output=True, text=True)
+    assert c.returncode == 0, c.stderr
+    got = json.loads(c.stdout.strip().splitlines()[-1])["outputs"]
+    assert got == [plain.generate_greedy(weights, cfg, p, 7, eos_ids=(stop,)) for p in prompts] and len(got[1]) <= 3

@@ -11,7 +11,7 @@ import plain_qwen2 as plain
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-CASES = [("A", False), ("B", False), ("B", True), ("C", False), ("C", True)]
+CASES = [("A", False), ("A", True), ("B", False), ("B", True), ("C", False), ("C", True)]
 LENS = {"A": [5, 11, 17, 64, 65, 100], "B": [1, 7, 20, 33, 64, 90], "C": [70, 129, 333, 600]}
 
 
@@ -117,6 +117,86 @@ def test_batches_of_random_sizes_shrink_through_every_kind_of_step(name, seed, d
                     % (name, seed, round_, i, len(r), tails[i]))
         eng.cache.check()
         assert eng.cache.slots.n_held == 0
+
+
+PIECES = {"B": [2, 7, 31, 33], "C": [2, 7, 63, 64, 65, 129]}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_prompts_fed_in_pieces(name, dtype):
+    """A prompt fed in pieces of 2, 7, 63, 64, 65, ... tokens (each piece a step of several tokens
+    behind what the cache already holds, the window crossing piece edges), beside a second
+    request that takes part in some steps only and a third that is decoded one token at a time
+    meanwhile; every place of every request against the plain implementation."""
+    eng = G.engine(name, dtype, True)
+    top = {"B": 96, "C": 640}[name]
+    for piece in PIECES[name]:
+        long, other, slow = G.prompts(name, [top - 6, min(top, 3 * piece + 1), top // 3], seed=1300 + piece)
+        s_long, s_other, s_slow = eng.open(), eng.open(), eng.open()
+        got = {"long": [], "other": [], "slow": []}
+        at_long = at_other = at_slow = 0
+        step = 0
+        while at_long < len(long) or at_other < len(other) or at_slow < len(slow):
+            items, names = [], []
+            if at_long < len(long):
+                toks = long[at_long:at_long + piece]
+                items.append((s_long, toks, all_places(toks))), names.append(("long", len(toks)))
+                at_long += len(toks)
+            if at_other < len(other) and step % 2 == 1:                  # left out of every other step
+                toks = other[at_other:at_other + piece + 1]
+                items.append((s_other, toks, all_places(toks))), names.append(("other", len(toks)))
+                at_other += len(toks)
+            if at_slow < len(slow):
+                items.append((s_slow, [slow[at_slow]], [0])), names.append(("slow", 1))
+                at_slow += 1
+            if items:
+                out = eng.step(items)
+                off = 0
+                for who, n in names:
+                    got[who].append(out[off:off + n])
+                    off += n
+            step += 1
+        for s in (s_long, s_other, s_slow):
+            eng.close(s)
+        for who, toks in (("long", long), ("other", other), ("slow", slow)):
+            G.close(torch.cat(got[who]), G.plain_logits(name, toks, True), dtype, "%s pieces of %d, request %s" % (name, piece, who))
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("name,sharp", CASES)
+@pytest.mark.parametrize("mode", ["decode", "piece"])
+def test_a_foreign_page_in_the_cache_is_noticed(name, sharp, mode):
+    """The comparisons above can fail: with one page of one sequence's cache (keys and values of
+    its first 64 positions, in the layers that see everything) replaced by another sequence's,
+    the bfloat16 comparison with the plain implementation raises, for the sharpened and the
+    plain random model alike, in one-token steps and in a prompt piece; the other sequence of
+    the batch, whose cache is whole, still passes."""
+    eng = G.engine(name, "bfloat16", sharp)
+    n = {"A": 100, "B": 90, "C": 600}[name]
+    p, other = G.prompts(name, [n, n], seed=1400)
+    ref, ref_other = G.plain_logits(name, p, sharp), G.plain_logits(name, other, sharp)
+    k = n - 8
+    for spoil in (False, True):
+        s, s2 = eng.open(), eng.open()
+        eng.step([(s, p[:k], []), (s2, other[:k], [])])
+        if spoil:
+            g = next(g for g in eng.cache.kv_groups if g.need.window is None)
+            a, b = g.pages[s][0], g.pages[s2][0]
+            g.keys[:, a], g.values[:, a] = g.keys[:, b].clone(), g.values[:, b].clone()
+        if mode == "decode":
+            outs = [eng.step([(s, [p[t]], [0]), (s2, [other[t]], [0])]) for t in range(k, n)]
+            got, got_other = torch.cat([o[:1] for o in outs]), torch.cat([o[1:] for o in outs])
+        else:
+            out = eng.step([(s, p[k:], list(range(8))), (s2, other[k:], list(range(8)))])
+            got, got_other = out[:8], out[8:]
+        eng.close(s), eng.close(s2)
+        G.close(got_other, ref_other[k:], "bfloat16", "the untouched sequence")
+        if spoil:
+            with pytest.raises(AssertionError):
+                G.close(got, ref[k:], "bfloat16")
+        else:
+            G.close(got, ref[k:], "bfloat16", "the clean run")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -308,7 +388,7 @@ def test_greedy_generation_bfloat16_picks_a_best_token_each_time(name):
         ref = G.plain_logits(name, p + o, True)
         for i, tok in enumerate(o):
             row = ref[len(p) - 1 + i]
-            assert row[tok] >= row.max() - 2 * G.TOL["bfloat16"]["atol"]
+            assert row[tok] >= row.max() - 2 * G.BF16_SPREAD * row.std().item()
 
 
 @pytest.mark.parametrize("name", ["A", "B"])

@@ -854,3 +854,126 @@ def test_a_random_model_on_the_gpu_equals_the_folder_the_host_writes(tmp_path):
             assert set(made) == set(stored)
             for k in stored:
                 assert torch.equal(made[k].cpu(), stored[k]), k
+
+
+# ---- the attention kernels at the lengths that are benchmarked ------------------------------------
+def scrambled_pages(n_pages_needed, n_pages, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randperm(n_pages, generator=g)[:n_pages_needed].tolist()
+
+
+def long_sequence(nkv, n, d, seed, window, last):
+    """Keys and values [nkv, n, d] (bfloat16 values, as float32) of a sequence whose first element
+    is nearly silent, with loud keys planted where a mistake shows: in the first page, in the
+    middle of the sequence, at the edge of the window of query `last` and just outside it."""
+    k, v = rand(nkv, n, d, seed=seed).cpu(), rand(nkv, n, d, seed=seed + 1).cpu()
+    k[:, :, 0] *= 0.01
+    k[:, 3, 0], k[:, n // 2 + 5, 0] = 9.0, 8.8
+    if window and last - window + 1 > 0:
+        k[:, last - window + 1, 0], k[:, last - window, 0] = 8.0, 9.5       # the edge, and just outside
+    return k.to(torch.bfloat16).float(), v.to(torch.bfloat16).float()
+
+
+def padded_table(rows, multiple=8):
+    width = (max(len(r) for r in rows) + multiple - 1) // multiple * multiple
+    return [list(r) + [-1] * (width - len(r)) for r in rows]
+
+
+@pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64)])
+@pytest.mark.parametrize("n_keys", [2300, 8200])
+@pytest.mark.parametrize("window", [0, 1000])
+def test_attention_decode_over_thousands_of_keys(nh, nkv, d, n_keys, window):
+    """One long sequence and one short one: dozens of pages scrambled over the pool, the table
+    padded with -1 to a multiple of 8 pages as the graphed steps pad it, pages that have left the
+    window given back (-1, their places NaN), eight and more partitions whose waves take several
+    pages each."""
+    lens = [n_keys, 70]
+    n_pages = (n_keys + 63) // 64 + 40
+    ids = scrambled_pages((n_keys + 63) // 64 + 2, n_pages, seed=n_keys)
+    tables = [ids[:(n_keys + 63) // 64], ids[(n_keys + 63) // 64:]]
+    keys, values = make_cache(n_pages, nkv, d, torch.bfloat16)
+    ks, vs = [], []
+    for i, n in enumerate(lens):
+        k, v = long_sequence(nkv, n, d, 300 + 10 * i, window, n - 1)
+        kk, vv = paged(k, v, tables[i], n_pages, torch.bfloat16)
+        dead = (max(0, n - window) // 64) if window else 0              # pages wholly behind the window
+        for j, p in enumerate(tables[i]):
+            if j >= dead:
+                keys[p], values[p] = kk[p], vv[p]
+        tables[i] = [-1] * dead + tables[i][dead:]
+        ks.append(k), vs.append(v)
+    q = rand(2, nh, d, seed=61).cpu()
+    q[0] = 0.0
+    q[0, :, 0] = 30.0
+    q = q.to(torch.bfloat16)
+    pos = torch.tensor([n - 1 for n in lens])
+    table = ints(padded_table(tables))
+    assert table.shape[1] % 8 == 0 and table.shape[1] >= (n_keys + 63) // 64
+    out = torch.empty(2, nh * d, dtype=torch.bfloat16, device=DEV)
+    scale = 1 / math.sqrt(d)
+    K.attention_decode(q.to(DEV), keys, values, pos.to(torch.int32).to(DEV), table, window, scale, out, target_blocks=256)
+    for i in range(2):
+        want = attention_reference(q[i:i + 1].float(), ks[i], vs[i], pos[i:i + 1], window, scale)
+        torch.testing.assert_close(out[i:i + 1].float().cpu(), want, atol=2e-2, rtol=2e-2)
+    # the planted keys matter: without the window (or with it) the sharp query's answer is another
+    other = attention_reference(q[:1].float(), ks[0], vs[0], pos[:1], 0 if window else 1000, scale)
+    assert (other - out[:1].float().cpu()).abs().max() > 0.1
+    out2 = torch.empty_like(out)
+    K.attention(q.to(DEV), keys, values, ints([0, 1]), pos.to(torch.int32).to(DEV), table, window, scale, out2)
+    torch.testing.assert_close(out.float(), out2.float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("nh,nkv,d,spans,tile", [
+    (28, 4, 128, [(0, 2048)], 64),                    # the benchmarked prompt
+    (28, 4, 128, [(0, 3200)], 128),                   # the wider tile that long steps use
+    (28, 4, 128, [(1100, 2100), (0, 70)], 64),        # a piece of a prompt behind 1100 cached positions
+    (6, 2, 64, [(0, 2048), (500, 1300)], 128),
+    (3, 1, 96, [(0, 2500)], 64),
+])
+@pytest.mark.parametrize("window", [0, 1000])
+def test_attention_prefill_over_thousands_of_keys(nh, nkv, d, spans, tile, window):
+    scale = 1 / math.sqrt(d)
+    need = [(b + 63) // 64 for _, b in spans]
+    n_pages = sum(need) + 30
+    ids = scrambled_pages(sum(need), n_pages, seed=spans[0][1])
+    tables, at = [], 0
+    for n in need:
+        tables.append(ids[at:at + n])
+        at += n
+    keys, values = make_cache(n_pages, nkv, d, torch.bfloat16)
+    ks, vs, qs = [], [], []
+    for i, (a, b) in enumerate(spans):
+        k, v = long_sequence(nkv, b, d, 400 + 10 * i, window, b - 1)
+        qq = rand(b - a, nh, d, seed=420 + i).cpu()
+        for row in (b - a - 1, (b - a) // 2):               # sharp queries: the last one and one in the middle
+            qq[row] = 0.0
+            qq[row, :, 0] = 30.0
+        kk, vv = paged(k, v, tables[i], n_pages, torch.bfloat16)
+        for p in tables[i]:
+            keys[p], values[p] = kk[p], vv[p]
+        ks.append(k), vs.append(v), qs.append(qq.to(torch.bfloat16))
+    q = torch.cat(qs).to(DEV)
+    pos = torch.cat([torch.arange(a, b) for a, b in spans])
+    tile_seq, tile_tok0, tile_count, off = [], [], [], 0
+    for i, (a, b) in enumerate(spans):
+        for s0 in range(0, b - a, tile):
+            tile_seq.append(i), tile_tok0.append(off + s0), tile_count.append(min(tile, b - a - s0))
+        off += b - a
+    order = sorted(range(len(tile_seq)), key=lambda t: -(int(pos[tile_tok0[t]]) + tile_count[t]))      # as the engine orders them
+    tile_seq, tile_tok0, tile_count = ([x[t] for t in order] for x in (tile_seq, tile_tok0, tile_count))
+    out = torch.full((q.shape[0], nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    K.attention_prefill(q, keys, values, pos.to(torch.int32).to(DEV), ints(padded_table(tables)), ints(tile_seq), ints(tile_tok0),
+                        ints(tile_count), ints([a for a, _ in spans]), ints([b - a for a, b in spans]), window, scale, out,
+                        tile_queries=tile)
+    assert not torch.isnan(out.float()).any()
+    off = 0
+    for i, (a, b) in enumerate(spans):
+        n = b - a
+        rows = sorted(set(list(range(0, n, 53)) + [r for r in (0, 1, 62, 63, 64, 65, 127, 128, 129, n // 2, n - 2, n - 1) if r < n]))
+        want = attention_reference(qs[i][rows].float(), ks[i], vs[i], torch.tensor(rows) + a, window, scale)
+        torch.testing.assert_close(out[off:off + n][rows].float().cpu(), want, atol=2e-2, rtol=2e-2,
+                                   msg=lambda m: "sequence %d: %s" % (i, m))
+        if i == 0:
+            other = attention_reference(qs[0][-1:].float(), ks[0], vs[0], torch.tensor([b - 1]), 0 if window else 1000, scale)
+            assert (other - out[off + n - 1:off + n].float().cpu()).abs().max() > 0.1
+        off += n

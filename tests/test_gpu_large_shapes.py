@@ -82,8 +82,9 @@ def test_bfloat16_tracks_float32_in_steps_of_17_to_64_rows_at_large_sizes(shape,
     torch.testing.assert_close(outs["bfloat16"], outs["float32"], atol=0.03 * max(1.0, scale), rtol=0.03)
 
 
-def test_float32_path_equals_plain_at_7b_sizes():
-    raw = two_layer("qwen2.5:7b")
+@pytest.mark.parametrize("shape", ["qwen2.5:7b", "qwen2.5:1.5b", "qwen2.5:32b"])
+def test_float32_path_equals_plain_at_large_sizes(shape):
+    raw = two_layer(shape)
     tensors = tensors_for(raw, 4)
     prompt = helpers.random_tokens(40, raw["vocab_size"], 60)
     eng = Engine(build(raw, "float32", tensors), max_tokens=256)
@@ -119,3 +120,119 @@ def test_generation_through_graphs_and_running_ahead_equals_plain_stepping_at_7b
         for o, t in zip(slow, toks):
             o.append(t)
     assert fast == slow
+
+
+# ---- the lengths that are benchmarked ---------------------------------------------------------------
+def sharpened(tensors):
+    """q and k projections doubled, so that attention picks out few keys among thousands and a
+    key that is missed or wrongly seen moves the logits."""
+    return {k: (v.float() * 2.0).to(v.dtype) if ("q_proj" in k or "k_proj" in k) else v for k, v in tensors.items()}
+
+
+def plain_rows(tensors, cfg, tokens, rows):
+    """The plain implementation's logits at chosen places (the head on all of 2100 places of a
+    vocabulary of 152064 would only cost time)."""
+    w = {k: v.float().cpu() for k, v in tensors.items()}
+    x = w["model.embed_tokens.weight"][torch.as_tensor(tokens)]
+    for layer in range(cfg["num_hidden_layers"]):
+        x = plain.decoder_layer(x, w, layer, cfg)
+    x = plain.rms_norm(x[rows], w["model.norm.weight"], cfg["rms_norm_eps"])
+    return plain.linear(x, w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"])
+
+
+def row_errors(got, want):
+    """For every row the rms and the largest difference, in units of the reference's spread."""
+    sigma = want.std().item()
+    err = (got - want).float()
+    return err.pow(2).mean(dim=1).sqrt() / sigma, err.abs().amax(dim=1) / sigma
+
+
+def test_prompts_of_two_thousand_tokens_and_graphed_decoding_at_7b_sizes():
+    """What bench.py times, checked: eight prompts of up to 2111 tokens in one step (33 pages a
+    sequence, the prompt kernel's long tile lists), then eight decoding steps of the batch through
+    captured graphs (page tables padded to 40, eight and more partitions per sequence).
+
+    Three runs: float32; bfloat16; bfloat16 with the plain attention kernel in place of the two
+    matrix-core attention kernels.  The float32 run equals the plain implementation (longest
+    sequence, prompt places and decoded ones).  The two bfloat16 runs differ by the rounding of
+    the probabilities alone, so they agree far more closely than bfloat16 and float32 do (whose
+    difference at these sizes is rounding noise of 2 to 4 % of the logits' spread in every row):
+    close enough that one foreign page among a sequence's 33 shows, which the last part asserts."""
+    from tq_kv_amd.parts import attention as A
+    raw = two_layer("qwen2.5:7b")
+    tensors = sharpened(tensors_for(raw, 6))
+    lens = [2100, 1990, 2048, 1500, 2111, 64, 1, 700]
+    prompts = [helpers.random_tokens(n, raw["vocab_size"], 150 + i) for i, n in enumerate(lens)]
+    tails = [helpers.random_tokens(8, raw["vocab_size"], 170 + i) for i in range(len(lens))]
+    wants = [sorted({0, n // 2, n - 1}) for n in lens]
+    n_first = sum(len(w) for w in wants)
+
+    def run(dtype, spoil=False):
+        eng = Engine(build(raw, dtype, tensors), max_tokens=len(lens) * 2240)
+        slots = [eng.open() for _ in prompts]
+        got = [eng.step([(s, p, w) for s, p, w in zip(slots, prompts, wants)])]
+        if spoil:          # sequence 0's page 10 (positions 640..703) becomes sequence 2's, in every layer
+            g = eng.cache.kv_groups[0]
+            a, b = g.pages[slots[0]][10], g.pages[slots[2]][10]
+            g.keys[:, a], g.values[:, a] = g.keys[:, b].clone(), g.values[:, b].clone()
+        for step in range(8):
+            got.append(eng.step([(s, [t[step]], [0]) for s, t in zip(slots, tails)]))
+        n_graphs = len(eng.graphs)
+        for s in slots:
+            eng.close(s)
+        del eng
+        torch.cuda.empty_cache()
+        return torch.cat(got).cpu(), n_graphs
+
+    f32, _ = run("float32")
+    bf16, n_graphs = run("bfloat16")
+    assert n_graphs >= 1                                   # the one-token steps went through captured graphs
+    old = dict(A.POLICY)
+    A.POLICY.update(decode_mfma=False, prefill_mfma=False)
+    try:
+        bf16_plain_kernel, _ = run("bfloat16")
+    finally:
+        A.POLICY.update(old)
+    rms, worst = row_errors(bf16, f32)
+    assert rms.max().item() < 0.07 and worst.max().item() < 0.35, (rms.max().item(), worst.max().item())
+    rms, worst = row_errors(bf16, bf16_plain_kernel)
+    assert rms.max().item() < 0.02 and worst.max().item() < 0.1, (rms.max().item(), worst.max().item())
+    # the float32 path itself, for the first sequence: its three prompt places and its eight decoded ones
+    seq = prompts[0] + tails[0]
+    rows = wants[0] + [lens[0] + i for i in range(8)]
+    want = plain_rows(tensors, dict(raw), seq, rows)
+    got = torch.cat([f32[:len(wants[0])]] + [f32[n_first + len(lens) * i][None] for i in range(8)])
+    torch.testing.assert_close(got, want, atol=2e-5 * max(1.0, want.abs().max().item()), rtol=2e-5)
+    # a foreign page is noticed, in the sequence it belongs to and nowhere else
+    spoiled, _ = run("bfloat16", spoil=True)
+    rms, _ = row_errors(spoiled, bf16_plain_kernel)
+    decoded_0 = [n_first + len(lens) * i for i in range(8)]
+    others = [r for r in range(spoiled.shape[0]) if r not in decoded_0]
+    assert rms[decoded_0].min().item() > 0.03, rms[decoded_0]
+    assert rms[others].max().item() < 0.02, rms[others].max()
+    print("rms of the spoiled sequence's rows", rms[decoded_0], "largest of the others", rms[others].max())
+
+
+def test_a_step_of_more_than_three_thousand_tokens_takes_the_wide_tiles():
+    """A step of 3300 tokens (one prompt of 3200 and one of 100) runs the prompt kernel with
+    tiles of 128 queries; 1.5B sizes (12 heads in groups of 6), bfloat16 against the float32 path."""
+    raw = two_layer("qwen2.5:1.5b")
+    tensors = sharpened(tensors_for(raw, 7))
+    prompts = [helpers.random_tokens(n, raw["vocab_size"], 190 + i) for i, n in enumerate([3200, 100])]
+    wants = [[0, 1599, 3199], [0, 99]]
+    outs = {}
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine(build(raw, dtype, tensors), max_tokens=3328 + 128)
+        slots = [eng.open() for _ in prompts]
+        a = eng.step([(s, p, w) for s, p, w in zip(slots, prompts, wants)])
+        b = eng.step([(s, [5], [0]) for s in slots])
+        outs[dtype] = torch.cat([a, b]).cpu()
+        for s in slots:
+            eng.close(s)
+        del eng
+        torch.cuda.empty_cache()
+    rms, worst = row_errors(outs["bfloat16"], outs["float32"])
+    assert rms.max().item() < 0.07 and worst.max().item() < 0.35, (rms.max().item(), worst.max().item())
+    want = plain_rows(tensors, dict(raw), prompts[1] + [5], [0, 99, 100])
+    got = torch.cat([outs["float32"][3:5], outs["float32"][6:7]])
+    torch.testing.assert_close(got, want, atol=2e-5 * max(1.0, want.abs().max().item()), rtol=2e-5)
