@@ -171,3 +171,23 @@ def test_sizes():
         make([FULL], max_tokens=10)
     c = make([FULL], max_tokens=PAGE * 3 + 5, max_slots=100)
     assert c.n_pages == 3 and c.max_slots == 3        # never more slots than pages
+
+
+def test_a_cache_of_state_alone_holds_no_pages_and_is_bounded_by_slots():
+    from tq_kv_amd.engine.generate import plan_batches
+    cache = Cache([StateNeed((4,)), None, StateNeed((4,), "int32")], [None, None, None], 10, 7, torch.float32, "cpu")
+    assert not cache.holds_pages and cache.max_slots == 7 and cache.kv_groups == [] and len(cache.state_groups) == 2
+    assert cache.state_groups[1].state.dtype == torch.int32
+    slots = [cache.acquire() for _ in range(7)]
+    cache.reserve([(s, 100000) for s in slots])           # no pages to run out of
+    cache.commit([(s, 100000) for s in slots])
+    assert cache.length(slots[3]) == 100000
+    with pytest.raises(CacheFull):
+        cache.acquire()
+    for s in slots:
+        cache.release(s)
+    cache.check()
+    # the loop plans such a model by slots alone
+    assert plan_batches([500] * 5, 10, 64, 2, holds_pages=False) == [[0, 1], [2, 3], [4]]
+    with pytest.raises(Exception, match="cache positions"):
+        plan_batches([500] * 5, 10, 64, 2)

@@ -28,7 +28,7 @@ def ints(values):
 
 
 def test_library_is_built_and_loaded():
-    assert K.library().tqk_abi_version() == 9
+    assert K.library().tqk_abi_version() == 10
     assert K.library_path().endswith(".so")
     with pytest.raises(K.KernelError, match="GPU only"):
         K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))

@@ -226,9 +226,12 @@ class ToyDecay(Part):
         for b in range(ctx.n_seqs):
             a, e = int(ctx.host.cu[b]), int(ctx.host.cu[b + 1])
             s = entry.state[int(ctx.host.seq_slot[b])]
-            for t in range(a, e):
-                s.mul_(self.decay).add_(x[t].float())
-                out[t] = (self.w.float() @ s).to(x.dtype)
+            # all states of the piece at once: s_t = decay^(t+1) s_before + sum_j decay^(t-j) x_j
+            t = torch.arange(e - a, device=x.device, dtype=torch.float32)
+            powers = torch.tril(self.decay ** (t[:, None] - t[None, :]).clamp(min=0))
+            states = powers @ x[a:e].float() + (self.decay ** (t + 1))[:, None] * s[None, :]
+            out[a:e] = (states @ self.w.float().t()).to(x.dtype)
+            s.copy_(states[-1])
         return out
 
 
@@ -486,3 +489,105 @@ def test_toy_norm_between_the_frameworks_products_in_steps_of_every_size(dtype):
     tol = dict(atol=2e-5, rtol=2e-5) if dtype == "float32" else G.TOL["bfloat16"]
     for i, r in enumerate(reqs):
         torch.testing.assert_close(torch.cat(got[i]).cpu(), plain_forward(r), msg=lambda m: "request %d: %s" % (i, m), **tol)
+
+
+# ---- what an architecture may do around the blocks -----------------------------------------------
+@register("position", "toy_learned")
+class ToyLearned(Part):
+    """Learned absolute positions: the stream of the token at position p gets row p of a table
+    added.  It acts on the stream after the gather (add_to_stream), not on q and k."""
+    graph_safe = True
+
+    def __init__(self, params, env):
+        self.hidden, self.max_positions = params["hidden"], params["max_positions"]
+
+    def tensors(self):
+        return {"weight": TensorSpec((self.max_positions, self.hidden))}
+
+    def load(self, tensors):
+        self.table = tensors["weight"].float()
+
+    def add_to_stream(self, h, ctx):
+        h += self.table.index_select(0, ctx.dev.tok_pos.long())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embedding_scale_positions_on_the_stream_head_bias_and_logit_scale_and_cap(dtype):
+    """The model spec's optional fields, none of which the reference's decoder uses: the stream
+    starts as embedding * scale plus a learned position row, the logits get a bias, a scale and
+    a soft cap.  Prompt step, then small decoding steps (whose gather would otherwise prepare the
+    first norm), through captured graphs."""
+    import dataclasses
+    cfg = dict(helpers.TINY_A)
+    h = cfg["hidden_size"]
+    spec = dataclasses.replace(
+        tiny_spec(cfg, position=PartSpec("none", {})), embedding_scale=float(h) ** 0.5,
+        stream_position=PartSpec("toy_learned", {"hidden": h, "max_positions": cfg["max_position_embeddings"]}),
+        stream_position_prefix="model.positions.", head_bias_name="lm_head.bias", logit_scale=0.5, logit_cap=0.75)
+    model = Model(spec, dtype, DEV)
+    assert {"model.positions.weight", "lm_head.bias"} <= set(model.tensor_specs()) and model.graph_safe
+    std = {"model.positions.weight": 0.5, "lm_head.bias": 1.0, "model.embed_tokens.weight": 0.1}
+    specs = {n: TensorSpec(s.shape, s.init, std.get(n, 0.08) if s.init == "normal" else 0.1) for n, s in model.tensor_specs().items()}
+    w = random_tensors(specs, 12, DT[dtype], "cpu")
+    model.load({k: v.to(DEV) for k, v in w.items()})
+    w = {k: v.float() for k, v in w.items()}
+    eps = cfg["rms_norm_eps"]
+
+    def plain_forward(tokens):
+        t = len(tokens)
+        x = w["model.embed_tokens.weight"][tokens] * (float(h) ** 0.5) + w["model.positions.weight"][:t]
+        nh, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+        for l in range(cfg["num_hidden_layers"]):
+            p = "model.layers.%d." % l
+            hn = plain.rms_norm(x, w[p + "input_layernorm.weight"], eps)
+            q, k, v = (plain.linear(hn, w[p + "self_attn.%s_proj.weight" % n], w[p + "self_attn.%s_proj.bias" % n])
+                       .reshape(t, heads, d).transpose(0, 1) for n, heads in (("q", nh), ("k", nkv), ("v", nkv)))
+            y = plain.attention_core(q, k, v, plain.visibility(t)).transpose(0, 1).reshape(t, nh * d)     # no rotation
+            x = x + plain.linear(y, w[p + "self_attn.o_proj.weight"])
+            x = x + plain.swiglu_mlp(plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], eps), w, p + "mlp.")
+        logits = (plain.linear(plain.rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"]) + w["lm_head.bias"]) * 0.5
+        return 0.75 * torch.tanh(logits / 0.75)
+
+    eng = Engine(model, max_tokens=1024)
+    a, b = helpers.random_tokens(30, 256, 14), helpers.random_tokens(12, 256, 15)
+    for round_ in range(2):                               # the second round replays the graphs of the first
+        sa, sb = eng.open(), eng.open()
+        out = eng.step([(sa, a[:20], list(range(20))), (sb, b[:5], list(range(5)))])
+        got_a, got_b = [out[:20]], [out[20:]]
+        for t in range(7):
+            out = eng.step([(sa, [a[20 + t]], [0]), (sb, [b[5 + t]], [0])])
+            got_a.append(out[:1].clone()), got_b.append(out[1:].clone())
+        eng.close(sb)
+        for t in range(27, 30):
+            got_a.append(eng.step([(sa, [a[t]], [0])]))
+        eng.close(sa)
+        want_a, want_b = plain_forward(a), plain_forward(b)
+        assert want_a.abs().max() > 0.6 and want_a.abs().max() < 0.75          # the cap bites, and holds
+        tol = dict(atol=2e-5, rtol=2e-5) if dtype == "float32" else dict(atol=0.1 * want_a.std().item(), rtol=0.02)
+        torch.testing.assert_close(torch.cat(got_a).cpu(), want_a, **tol)
+        torch.testing.assert_close(torch.cat(got_b).cpu(), want_b, **tol)
+    assert len(eng.graphs) >= 1
+    with pytest.raises(ValueError, match="cannot act on the stream"):
+        Model(dataclasses.replace(spec, stream_position=PartSpec("none", {})), dtype, DEV)
+
+
+def test_a_model_of_state_alone_is_not_bounded_by_cache_positions():
+    """Every run keeps a fixed-size state and none keeps keys: the cache holds no pages, so
+    max_tokens bounds nothing and the generation loop plans by slots alone.  300 requests of 500
+    tokens through an engine made with max_tokens=64."""
+    from tq_kv_amd import GenerationParams, generate
+    cfg = dict(helpers.TINY_A, num_hidden_layers=2, max_position_embeddings=600)
+    toy = PartSpec("toy_decay", {"hidden": cfg["hidden_size"], "decay": 0.5})
+    model = Model(tiny_spec(cfg, mixers={0: toy, 1: toy}), "float32", DEV)
+    specs = {n: TensorSpec(s.shape, s.init, 0.2 if s.init == "normal" else 0.1) for n, s in model.tensor_specs().items()}
+    model.load({k: v.to(DEV) for k, v in random_tensors(specs, 13, torch.float32, "cpu").items()})
+    eng = Engine(model, max_tokens=64, max_slots=64)
+    assert not eng.holds_pages and eng.cache.kv_groups == [] and eng.max_slots == 64
+    prompts = [helpers.random_tokens(500, 256, 1000 + i % 7) for i in range(300)]
+    out = generate(eng, prompts, GenerationParams(max_tokens=2, temperature=0.0, repeat_penalty=1.0), max_batch=64)
+    assert len(out) == 300 and all(len(o) == 2 for o in out)
+    for i in range(7, 300):
+        assert out[i] == out[i % 7]                       # equal prompts, equal tokens, whatever the batch and the slot
+    assert len({tuple(o) for o in out[:7]}) > 1
+    eng.cache.check()
+    assert eng.cache.slots.n_held == 0

@@ -94,12 +94,17 @@ class KVGroup:
         self.pool.give_back([p for p in have if p >= 0])
 
 
+STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
+
+
 class StateGroup:
     def __init__(self, need, runs, n_slots, device):
         self.need = need
         self.runs = list(runs)
+        if need.dtype not in STATE_DTYPES:
+            raise TypeError("state of kind %r (known: %s)" % (need.dtype, ", ".join(sorted(STATE_DTYPES))))
         self.state = torch.zeros((len(self.runs), n_slots) + tuple(need.shape),
-                                 dtype=torch.float32, device=device)
+                                 dtype=STATE_DTYPES[need.dtype], device=device)
 
     def reset(self, slot):
         self.state[:, slot].zero_()
@@ -115,10 +120,13 @@ class Cache:
     """
 
     def __init__(self, needs, cache_of, max_tokens, max_slots, dtype, device):
-        if max_tokens < PAGE:
+        # pages bound the cache only where some run keeps keys and values: a model whose runs all
+        # keep fixed-size state (or nothing) is bounded by its slots alone
+        self.holds_pages = any(isinstance(need, KVNeed) and cache_of[run] is None for run, need in enumerate(needs))
+        if self.holds_pages and max_tokens < PAGE:
             raise ValueError("max_tokens must be at least %d, got %d" % (PAGE, max_tokens))
-        self.n_pages = max_tokens // PAGE
-        self.max_slots = max(1, min(int(max_slots), self.n_pages))
+        self.n_pages = max_tokens // PAGE if self.holds_pages else 0
+        self.max_slots = max(1, min(int(max_slots), self.n_pages)) if self.holds_pages else max(1, int(max_slots))
         self.device = device
         self.slots = FreeList(self.max_slots, "slot")
         self.lengths = [0] * self.max_slots
@@ -201,7 +209,7 @@ class Cache:
 
     def page_table(self, group, slots):
         """[len(slots), width] int32 of page ids (-1: none) for the sequences of a step."""
-        width = max(1, max(len(group.pages.get(s, ())) for s in slots))
+        width = max(1, max(len(group.pages.get(s, ())) for s in slots))     # (a group exists only with pages)
         table = np.full((len(slots), width), -1, dtype=np.int32)
         for i, s in enumerate(slots):
             have = group.pages.get(s, ())

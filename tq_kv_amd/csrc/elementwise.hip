@@ -7,7 +7,7 @@
 // The reference looks rows up with candle's embedding op (src/models/turbo_generic.rs:1958).
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
-                             int hidden, int vocab, float* __restrict__ out, bf16_t* __restrict__ copy,
+                             int hidden, int vocab, float scale, float* __restrict__ out, bf16_t* __restrict__ copy,
                              const bf16_t* __restrict__ copy_weight, float* __restrict__ ss_out) {
     __shared__ float scratch[16];
     const int t = blockIdx.x;
@@ -18,7 +18,7 @@ __global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restr
     const T* row = table + (size_t)(ok ? id : 0) * hidden;
     float ss = 0.f;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-        const float v = ok ? to_float(row[i]) : 0.f;
+        const float v = ok ? to_float(row[i]) * scale : 0.f;
         o[i] = v;
         ss = fmaf(v, v, ss);
         if (c) c[i] = from_float<bf16_t>(copy_weight ? v * to_float(copy_weight[i]) : v);
@@ -31,7 +31,7 @@ __global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restr
 
 // bfloat16 table, hidden a multiple of 8: 16 bytes per thread and load, one pass.
 __global__ void embed_bf16x8_kernel(const bf16_t* __restrict__ table, const int32_t* __restrict__ ids,
-                                    int hidden, int vocab, float* __restrict__ out, bf16_t* __restrict__ copy,
+                                    int hidden, int vocab, float scale, float* __restrict__ out, bf16_t* __restrict__ copy,
                                     const bf16_t* __restrict__ copy_weight, float* __restrict__ ss_out) {
     __shared__ float scratch[16];
     const int t = blockIdx.x;
@@ -45,8 +45,8 @@ __global__ void embed_bf16x8_kernel(const bf16_t* __restrict__ table, const int3
         float v[8];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            v[2 * j] = __uint_as_float(words[j] << 16);
-            v[2 * j + 1] = __uint_as_float(words[j] & 0xffff0000u);
+            v[2 * j] = __uint_as_float(words[j] << 16) * scale;
+            v[2 * j + 1] = __uint_as_float(words[j] & 0xffff0000u) * scale;
         }
         float4* o = reinterpret_cast<float4*>(out + (size_t)t * hidden + (size_t)i * 8);
         o[0] = make_float4(v[0], v[1], v[2], v[3]);
@@ -55,8 +55,9 @@ __global__ void embed_bf16x8_kernel(const bf16_t* __restrict__ table, const int3
         for (int j = 0; j < 8; ++j) ss = fmaf(v[j], v[j], ss);
         if (copy) {
             uint4 packed = raw;
-            if (copy_weight) {
-                const uint4 wraw = reinterpret_cast<const uint4*>(copy_weight)[i];
+            if (copy_weight || scale != 1.0f) {
+                const uint4 wraw = copy_weight ? reinterpret_cast<const uint4*>(copy_weight)[i]
+                                               : make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);      // ones
                 const uint32_t ww[4] = {wraw.x, wraw.y, wraw.z, wraw.w};
                 uint32_t pw[4];
 #pragma unroll
@@ -77,7 +78,7 @@ __global__ void embed_bf16x8_kernel(const bf16_t* __restrict__ table, const int3
 }
 
 extern "C" int tqk_embed(const void* table, int table_dtype, const int32_t* ids, int n_tokens,
-                         int hidden, int vocab, float* out, void* copy_bf16, const void* copy_weight,
+                         int hidden, int vocab, float scale, float* out, void* copy_bf16, const void* copy_weight,
                          float* ss_out, void* stream) {
     TQK_REQUIRE(table && ids && out, "tqk_embed: null pointer");
     TQK_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "tqk_embed: bad sizes tokens=%d hidden=%d vocab=%d", n_tokens, hidden, vocab);
@@ -85,18 +86,41 @@ extern "C" int tqk_embed(const void* table, int table_dtype, const int32_t* ids,
     if (n_tokens == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (table_dtype == TQK_F32)
-        embed_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)table, ids, hidden, vocab, out, (bf16_t*)copy_bf16,
+        embed_kernel<float><<<n_tokens, 256, 0, s>>>((const float*)table, ids, hidden, vocab, scale, out, (bf16_t*)copy_bf16,
                                                      (const bf16_t*)copy_weight, ss_out);
     else if (table_dtype == TQK_BF16 && hidden % 8 == 0 && (((uintptr_t)table | (uintptr_t)out | (uintptr_t)copy_bf16 | (uintptr_t)copy_weight) & 15) == 0) {
         const int threads = ((hidden / 8 + TQK_WAVE - 1) / TQK_WAVE) * TQK_WAVE;
-        embed_bf16x8_kernel<<<n_tokens, threads > 1024 ? 1024 : threads, 0, s>>>((const bf16_t*)table, ids, hidden, vocab, out, (bf16_t*)copy_bf16,
+        embed_bf16x8_kernel<<<n_tokens, threads > 1024 ? 1024 : threads, 0, s>>>((const bf16_t*)table, ids, hidden, vocab, scale, out, (bf16_t*)copy_bf16,
                                                                                (const bf16_t*)copy_weight, ss_out);
     } else if (table_dtype == TQK_BF16)
-        embed_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)table, ids, hidden, vocab, out, (bf16_t*)copy_bf16,
+        embed_kernel<bf16_t><<<n_tokens, 256, 0, s>>>((const bf16_t*)table, ids, hidden, vocab, scale, out, (bf16_t*)copy_bf16,
                                                       (const bf16_t*)copy_weight, ss_out);
     else
         return tqk_fail("tqk_embed: unknown dtype %d", table_dtype);
     return tqk_check_launch("tqk_embed");
+}
+
+// ---- what an architecture may do to its logits after the head ------------------------------------
+__global__ void finish_logits_kernel(float* __restrict__ logits, long long n, int vocab, const float* __restrict__ bias,
+                                     float scale, float cap) {
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        float l = logits[i];
+        if (bias) l += bias[i % vocab];
+        l *= scale;
+        if (cap > 0.f) l = cap * tanhf(l / cap);
+        logits[i] = l;
+    }
+}
+
+extern "C" int tqk_finish_logits(float* logits, int n_rows, int vocab, const float* bias, float scale, float cap, void* stream) {
+    TQK_REQUIRE(logits, "tqk_finish_logits: null pointer");
+    TQK_REQUIRE(n_rows >= 0 && vocab > 0, "tqk_finish_logits: bad sizes rows=%d vocab=%d", n_rows, vocab);
+    if (n_rows == 0) return 0;
+    const long long n = (long long)n_rows * vocab;
+    const long long want = (n + 255) / 256;
+    finish_logits_kernel<<<(int)(want < 8192 ? want : 8192), 256, 0, (hipStream_t)stream>>>(logits, n, vocab, bias, scale, cap);
+    return tqk_check_launch("tqk_finish_logits");
 }
 
 // ---- residual add + RMSNorm -----------------------------------------------------

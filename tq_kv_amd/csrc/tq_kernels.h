@@ -18,12 +18,16 @@ extern "C" {
 const char* tqk_last_error(void);
 int tqk_abi_version(void);
 
-/* out[t, :] = float(table[ids[t], :]); ids outside [0, vocab) give zeros.  copy_bf16
+/* out[t, :] = scale * float(table[ids[t], :]); ids outside [0, vocab) give zeros.  copy_bf16
  * (optional): the same values as bfloat16 [tokens, hidden], times copy_weight [hidden]
  * (bfloat16) if given.  ss_out (optional, at most 16 tokens): ss_out[t] = sum of out[t]^2. */
 int tqk_embed(const void* table, int table_dtype, const int32_t* ids, int n_tokens,
-              int hidden, int vocab, float* out, void* copy_bf16, const void* copy_weight,
+              int hidden, int vocab, float scale, float* out, void* copy_bf16, const void* copy_weight,
               float* ss_out, void* stream);
+
+/* In place on float32 logits [rows, vocab]: l = (l + bias[v]) * scale, then, if cap > 0,
+ * l = cap * tanh(l / cap).  bias (float32 [vocab]) may be null. */
+int tqk_finish_logits(float* logits, int n_rows, int vocab, const float* bias, float scale, float cap, void* stream);
 
 /* out[i] = std_dev * z(key, i) (+ 1 if plus_one), i < n: standard normal values that are a
  * function of the 64-bit key and the index alone, the same bits as the host's recipe gives

@@ -11,14 +11,6 @@ import numpy as np
 import torch
 
 
-def tile_queries(n_tokens):
-    """Queries per tile of the prompt attention kernel: 128 where there is work for many
-    blocks anyway (a query then costs less LDS traffic), 64 for smaller steps (more blocks to
-    share out, fewer idle lanes).  Measured at 28 heads of 128: 2048 tokens 75 us with tiles of
-    64 against 84 us with 128, 4096 tokens 239 against 211."""
-    return 128 if n_tokens >= 3072 else 64
-
-
 class _Arrays:
     pass
 
@@ -90,39 +82,14 @@ class StepContext:
         host.last_rows = np.unique(host.want_rows).astype(np.int32)
         host.want_in_last = np.searchsorted(host.last_rows, host.want_rows).astype(np.int32)
         self.n_last = int(host.last_rows.shape[0])
-        # tiles of consecutive queries of one sequence, for the prompt attention kernel
-        self.tile_queries = tile = tile_queries(self.n_tokens)
-        t_seq, t_tok0, t_count = [], [], []
-        for i, n in enumerate(lens):
-            for a in range(0, n, tile):
-                t_seq.append(i)
-                t_tok0.append(int(host.cu[i]) + a)
-                t_count.append(min(tile, n - a))
-        # longest first (a tile's work grows with the position of its last query)
-        order = sorted(range(len(t_seq)), key=lambda k: -(int(host.tok_pos[t_tok0[k]]) + t_count[k]))
-        host.tile_seq = np.asarray([t_seq[k] for k in order], dtype=np.int32)
-        host.tile_tok0 = np.asarray([t_tok0[k] for k in order], dtype=np.int32)
-        host.tile_count = np.asarray([t_count[k] for k in order], dtype=np.int32)
         self.all_decode = all(n == 1 for n in lens)
         self.prune_last = not self.all_decode and self.n_last < self.n_tokens
-        # the same for the last run's rows, in their own numbering: runs of neighbouring rows of a sequence
-        l_seq, l_tok0, l_count = [], [], []
         if self.prune_last:
             host.last_seq, host.last_pos = host.tok_seq[host.last_rows], host.tok_pos[host.last_rows]
-            k = 0
-            while k < self.n_last:
-                j = k + 1
-                while (j < self.n_last and j - k < tile and host.last_rows[j] == host.last_rows[j - 1] + 1
-                       and host.last_seq[j] == host.last_seq[k]):
-                    j += 1
-                l_seq.append(int(host.last_seq[k])), l_tok0.append(k), l_count.append(j - k)
-                k = j
         else:
             host.last_rows = host.want_in_last = host.last_seq = host.last_pos = np.zeros(0, dtype=np.int32)
-        order = sorted(range(len(l_seq)), key=lambda t: -(int(host.last_pos[l_tok0[t]]) + l_count[t]))
-        host.last_tile_seq = np.asarray([l_seq[t] for t in order], dtype=np.int32)
-        host.last_tile_tok0 = np.asarray([l_tok0[t] for t in order], dtype=np.int32)
-        host.last_tile_count = np.asarray([l_count[t] for t in order], dtype=np.int32)
+        self._lens = lens
+        self._tiles = {}              # (which rows, queries per tile) -> device arrays, built when a mixer asks
         self.host = host
         self.fuse_small = False      # set by the model for small decoding steps in bfloat16
         self.max_new = max(lens)
@@ -139,8 +106,7 @@ class StepContext:
                 self.host_tables[i] = wide
 
         names = ["tokens", "tok_seq", "tok_pos", "seq_slot", "seq_start", "seq_new", "cu", "want_rows",
-                 "tile_seq", "tile_tok0", "tile_count", "last_rows", "want_in_last", "last_seq", "last_pos",
-                 "last_tile_seq", "last_tile_tok0", "last_tile_count"]
+                 "last_rows", "want_in_last", "last_seq", "last_pos"]
         parts = [getattr(host, n) for n in names] + [t.reshape(-1) for t in self.host_tables]
         offsets, total = [], 0
         for p in parts:
@@ -150,6 +116,7 @@ class StepContext:
         for off, p in zip(offsets, parts):
             packed[off:off + p.shape[0]] = p
         self.packed = packed
+        self._device, self._staging = device, staging
         if into is not None and not isinstance(into, torch.Tensor):
             return                                   # host arrays only
         if staging is not None:
@@ -166,6 +133,52 @@ class StepContext:
         self._tables = {}
         for g, off, t in zip(self.groups, offsets[len(names):], self.host_tables):
             self._tables[id(g)] = flat[off:off + t.size].view(t.shape)
+
+    # -- tiles of consecutive queries, for mixers that work on them -----------------------------
+    def _upload_tiles(self, key, seq, tok0, count, order_key):
+        order = sorted(range(len(seq)), key=order_key)          # longest first: a tile's work grows with its last position
+        packed = np.asarray([seq[k] for k in order] + [tok0[k] for k in order] + [count[k] for k in order], dtype=np.int32)
+        n = len(order)
+        if n == 0:
+            flat = torch.zeros(0, dtype=torch.int32, device=self._device)
+        elif self._staging is not None:
+            flat = self._staging.upload(packed)
+        else:
+            flat = torch.from_numpy(packed).to(self._device)
+        self._tiles[key] = (flat[:n], flat[n:2 * n], flat[2 * n:3 * n])
+        return self._tiles[key]
+
+    def query_tiles(self, tile):
+        """The step's tokens cut into tiles of up to `tile` consecutive queries of one sequence:
+        (sequence of the step, first packed token, number of queries) per tile, int32 on the
+        device, longest reach first.  Built and uploaded when a mixer first asks for this size."""
+        key = ("all", int(tile))
+        if key in self._tiles:
+            return self._tiles[key]
+        cu, pos = self.host.cu, self.host.tok_pos
+        seq, tok0, count = [], [], []
+        for i, n in enumerate(self._lens):
+            for a in range(0, n, tile):
+                seq.append(i), tok0.append(int(cu[i]) + a), count.append(min(tile, n - a))
+        return self._upload_tiles(key, seq, tok0, count, lambda k: -(int(pos[tok0[k]]) + count[k]))
+
+    def last_tiles(self, tile):
+        """The same for the step's last_rows, in their own numbering: runs of neighbouring rows of
+        one sequence, up to `tile` each."""
+        key = ("last", int(tile))
+        if key in self._tiles:
+            return self._tiles[key]
+        h = self.host
+        seq, tok0, count = [], [], []
+        k = 0
+        while self.prune_last and k < self.n_last:
+            j = k + 1
+            while (j < self.n_last and j - k < tile and h.last_rows[j] == h.last_rows[j - 1] + 1
+                   and h.last_seq[j] == h.last_seq[k]):
+                j += 1
+            seq.append(int(h.last_seq[k])), tok0.append(k), count.append(j - k)
+            k = j
+        return self._upload_tiles(key, seq, tok0, count, lambda t: -(int(h.last_pos[tok0[t]]) + count[t]))
 
     def shape_key(self):
         """What fixes the layout of the device arrays (and so what a captured graph of the

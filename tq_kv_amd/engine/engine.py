@@ -33,6 +33,8 @@ class Engine:
         self.max_tokens = int(max_tokens)
         self.cache = Cache(model.needs, model.cache_of, self.max_tokens, max_slots, model.dtype, model.device)
         self.staging = HostStaging(model.device) if model.device.type == "cuda" else None
+        self.holds_pages = self.cache.holds_pages       # False: no run keeps keys and values, max_tokens bounds nothing
+        self.max_slots = self.cache.max_slots
         self.vocab_size = model.spec.vocab_size
         self.max_positions = model.spec.max_positions
         # Steps of one token per sequence are captured as HIP graphs and replayed: the step

@@ -26,13 +26,13 @@ def _room(prompt_len, max_new):
     return (longest + PAGE - 1) // PAGE * PAGE
 
 
-def plan_batches(prompt_lens, max_new, max_tokens, max_batch):
+def plan_batches(prompt_lens, max_new, max_tokens, max_batch, holds_pages=True):
     """Cut the requests, in order, into batches that fit the cache: at most max_batch
-    requests and at most max_tokens positions (whole pages each).  Returns lists of
-    request indices."""
+    requests and at most max_tokens positions (whole pages each; not counted where the
+    engine's cache holds no pages: holds_pages False).  Returns lists of request indices."""
     batches, cur, used = [], [], 0
     for i, n in enumerate(prompt_lens):
-        need = _room(n, max_new)
+        need = _room(n, max_new) if holds_pages else 0
         if need > max_tokens:
             raise GenerationError("request %d needs %d cache positions, the engine has %d" % (i, need, max_tokens))
         if cur and (len(cur) >= max_batch or used + need > max_tokens):
@@ -73,7 +73,9 @@ def generate(engine, prompts, params=None, eos_ids=None, on_tokens=None, max_bat
             return Sampler(p, request_ids, engine.model.device)
 
     emitted = [[] for _ in prompts]
-    for batch in plan_batches([len(p) for p in prompts], params.max_tokens, engine.max_tokens, max_batch):
+    max_batch = min(max_batch, getattr(engine, "max_slots", max_batch))
+    for batch in plan_batches([len(p) for p in prompts], params.max_tokens, engine.max_tokens, max_batch,
+                              holds_pages=getattr(engine, "holds_pages", True)):
         _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, make_sampler(params, batch),
                    max(1, int(max_step_tokens)))
     return emitted

@@ -37,6 +37,11 @@ class Model:
         self.env = BuildEnv(self.device, self.dtype)
         self.blocks = [self.env.build("block", layer.block) for layer in spec.layers]
         self.final_norm = self.env.build("norm", spec.final_norm)
+        self.stream_position = (self.env.build("position", spec.stream_position)
+                                if spec.stream_position is not None else None)
+        if self.stream_position is not None and not hasattr(self.stream_position, "add_to_stream"):
+            raise ValueError("position kind '%s' cannot act on the stream (it has no add_to_stream)" % spec.stream_position.kind)
+        self.head_bias = None
         for i, run in enumerate(spec.order):
             if not 0 <= run.layer < len(self.blocks):
                 raise ValueError("run %d names layer %d, the model has %d" % (i, run.layer, len(self.blocks)))
@@ -55,7 +60,8 @@ class Model:
         # a step can be captured as a graph if every part's forward launches the same kernels
         # whatever the step's data are; up to 64 rows (the hand-written products; where a weight
         # has no packed copy the library's, which capture as they are)
-        self.graph_safe = all(getattr(b, "graph_safe", False) for b in self.blocks) and getattr(self.final_norm, "graph_safe", False)
+        self.graph_safe = (all(getattr(b, "graph_safe", False) for b in self.blocks) and getattr(self.final_norm, "graph_safe", False)
+                           and (self.stream_position is None or getattr(self.stream_position, "graph_safe", False)))
         self.graph_max_rows = 64
 
     # -- tensors ----------------------------------------------------------
@@ -70,6 +76,11 @@ class Model:
             out[s.final_norm_prefix + name] = spec
         if s.head_name is not None:
             out[s.head_name] = TensorSpec((s.vocab_size, s.hidden_size))
+        if self.stream_position is not None:
+            for name, spec in self.stream_position.tensors().items():
+                out[s.stream_position_prefix + name] = spec
+        if s.head_bias_name is not None:
+            out[s.head_bias_name] = TensorSpec((s.vocab_size,))
         return out
 
     def load(self, tensors):
@@ -80,6 +91,10 @@ class Model:
             block.load({name: tensors[layer.prefix + name] for name in block.tensors()})
         self.final_norm.load({name: tensors[s.final_norm_prefix + name] for name in self.final_norm.tensors()})
         self.head = self.embedding if s.head_name is None else tensors[s.head_name]
+        if self.stream_position is not None:
+            self.stream_position.load({name: tensors[s.stream_position_prefix + name] for name in self.stream_position.tensors()})
+        if s.head_bias_name is not None:
+            self.head_bias = tensors[s.head_bias_name].to(torch.float32)
         self.few_head = L.few_rows_form(self.head)      # the head's copy for the few-row kernel
         self.loaded = True
         return self
@@ -155,22 +170,39 @@ class Model:
                         and L.POLICY["skinny_max_rows"] < ctx.n_tokens <= K.MID_MAX_ROWS)
         # the norm that reads the stream first in every run, and after the last one
         firsts = [self.blocks[run.layer].first_norm() for run in s.order] + [self.final_norm]
+        scale = 1.0 if s.embedding_scale is None else float(s.embedding_scale)
         if ctx.fuse_small:
             xw = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.bfloat16, device=self.device)
             ss = torch.empty(((s.hidden_size + 15) // 16, 16), dtype=torch.float32, device=self.device)      # the most pieces a product gives
             stream = L.Stream(h, xw, ss)
             norm = firsts[0] if getattr(firsts[0], "foldable", False) else None
-            K.embed(self.embedding, ctx.dev.tokens, h, copy=xw, copy_weight=norm.weight if norm is not None else None, ss_out=ss)
+            K.embed(self.embedding, ctx.dev.tokens, h, copy=xw, copy_weight=norm.weight if norm is not None else None, ss_out=ss,
+                    scale=scale)
             stream.xw_for, stream.n_ss = norm, 1
         else:
             stream = L.Stream(h)
-            K.embed(self.embedding, ctx.dev.tokens, h)
+            K.embed(self.embedding, ctx.dev.tokens, h, scale=scale)
+        if self.stream_position is not None:
+            self.stream_position.add_to_stream(h, ctx)
+            stream.invalidate()              # what the gather prepared for the first norm is of the stream before this
         for i, run in enumerate(s.order):
             stream = self.blocks[run.layer].forward(stream, ctx, cache.entry(i), next_norm=firsts[i + 1],
                                                     last=i + 1 == len(s.order)) or stream
         n_rows = ctx.dev.want_rows.shape[0]
         if n_rows == 0:
             return torch.empty((0, s.vocab_size), dtype=torch.float32, device=self.device)
+        return self._finish(self._head(stream, ctx, n_rows))
+
+    def _finish(self, logits):
+        """Bias, scale and cap of the logits, where the architecture has them."""
+        s = self.spec
+        if self.head_bias is not None or s.logit_scale is not None or s.logit_cap is not None:
+            K.finish_logits(logits, self.head_bias, 1.0 if s.logit_scale is None else float(s.logit_scale),
+                            0.0 if s.logit_cap is None else float(s.logit_cap))
+        return logits
+
+    def _head(self, stream, ctx, n_rows):
+        s = self.spec
         # the last block may have gone on with the wanted rows alone, numbered among themselves
         want_rows = ctx.dev.want_in_last if getattr(stream, "of_last_rows", False) else ctx.dev.want_rows
         lazy = self.final_norm.lazy(stream) if ctx.fuse_small and hasattr(self.final_norm, "lazy") else None

@@ -78,8 +78,8 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def embed(table, ids, out, copy=None, copy_weight=None, ss_out=None):
-    """out[t] = float32(table[ids[t]]);  table [V,H], ids [T] int32, out [T,H] float32.
+def embed(table, ids, out, copy=None, copy_weight=None, ss_out=None, scale=1.0):
+    """out[t] = scale * float32(table[ids[t]]);  table [V,H], ids [T] int32, out [T,H] float32.
     copy (optional): the same as bfloat16 [T,H], times copy_weight [H] if given; ss_out
     (optional, float32, at least T values, T <= 16): sums of squares of the rows."""
     vocab, hidden = table.shape
@@ -87,7 +87,7 @@ def embed(table, ids, out, copy=None, copy_weight=None, ss_out=None):
     if ss_out is not None and ss_out.numel() < max(n, 1):
         raise KernelError("embed: ss_out holds %d values for %d tokens" % (ss_out.numel(), n))
     _check(library().tqk_embed(_dev(table, "table"), _code(table.dtype), _dev(ids, "ids", torch.int32, (n,)),
-                               n, hidden, vocab, _dev(out, "out", torch.float32, (n, hidden)),
+                               n, hidden, vocab, ctypes.c_float(scale), _dev(out, "out", torch.float32, (n, hidden)),
                                _opt(copy, "copy", torch.bfloat16, (n, hidden)),
                                _opt(copy_weight, "copy_weight", torch.bfloat16, (hidden,)),
                                _opt(ss_out, "ss_out", torch.float32), _stream()),
@@ -102,6 +102,15 @@ def random_normal(out, key, std, plus_one=False):
                                        ctypes.c_uint64(int(key) & 0xFFFFFFFFFFFFFFFF), ctypes.c_float(std),
                                        1 if plus_one else 0, _stream()), "random_normal")
     return out
+
+
+def finish_logits(logits, bias=None, scale=1.0, cap=0.0):
+    """In place: logits = (logits + bias) * scale, then cap * tanh(logits / cap) if cap > 0."""
+    rows, vocab = logits.shape
+    _check(library().tqk_finish_logits(_dev(logits, "logits", torch.float32), rows, vocab,
+                                       _opt(bias, "bias", torch.float32, (vocab,)), ctypes.c_float(scale),
+                                       ctypes.c_float(cap), _stream()), "finish_logits")
+    return logits
 
 
 def add_rmsnorm(h, delta, weight, eps, out, rows=None, write_back=False):

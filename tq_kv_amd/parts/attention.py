@@ -20,7 +20,12 @@ from .spec import KVNeed, TensorSpec
 class Attention(Part):
     """params: hidden, n_heads, n_kv_heads, head_dim, qkv_bias (bool), out_bias (bool),
     window (None or positions a query sees, itself included), scale (None: 1/sqrt(head_dim)),
-    position (PartSpec)."""
+    position (PartSpec); optional prompt_tiles = (queries per tile of the prompt kernel, the wider
+    tile, the step size in tokens from which the wider one is used)."""
+
+    # Measured with 28 heads of 128: 2048 tokens run faster in tiles of 64 queries (more blocks to
+    # share out), 4096 and more in tiles of 128 (less staging per query).
+    PROMPT_TILES = (64, 128, 3072)
 
     def __init__(self, params, env):
         self.env = env
@@ -38,6 +43,9 @@ class Attention(Part):
             raise ValueError("attention: window must be at least 1, got %r" % (self.window,))
         scale = params.get("scale")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.prompt_tiles = tuple(int(v) for v in params.get("prompt_tiles", self.PROMPT_TILES))
+        if len(self.prompt_tiles) != 3 or any(t not in (64, 128) for t in self.prompt_tiles[:2]):
+            raise ValueError("attention: prompt_tiles must be (64 or 128, 64 or 128, tokens), got %r" % (self.prompt_tiles,))
         spec = params["position"]
         key = ("position", spec.kind, tuple(sorted(spec.params.items())))
         if key not in env.shared:
@@ -119,14 +127,19 @@ class Attention(Part):
             if ctx.n_last == 0:
                 return torch.empty((0, self.hidden), dtype=dtype, device=q.device)
             y = torch.empty((ctx.n_last, self.n_heads * self.head_dim), dtype=dtype, device=q.device)
-            attend_rows(q.index_select(0, d.last_rows), entry, table, ctx, self.window, self.scale, y)
+            attend_rows(q.index_select(0, d.last_rows), entry, table, ctx, self.window, self.scale, y, self.tile_for(ctx))
             return linear(y, self.w_o, self.b_o, few=self.few_o)
         y = torch.empty((n, self.n_heads * self.head_dim), dtype=dtype, device=q.device)
-        attend(q, entry, table, ctx, self.window, self.scale, y)
+        attend(q, entry, table, ctx, self.window, self.scale, y, self.tile_for(ctx))
         if stream is not None:
             stream.add_product(y, self.few_o or self.w_o)
             return None
         return linear(y, self.w_o, self.b_o, few=self.few_o)
+
+    def tile_for(self, ctx):
+        """Queries per tile of the prompt kernel for this step."""
+        small, wide, wide_from = self.prompt_tiles
+        return wide if ctx.n_tokens >= wide_from else small
 
     def _qkv(self, x, ctx, entry, table, q):
         """Product, then bias, position encoding and cache write in their own kernel."""
@@ -158,7 +171,7 @@ class Attention(Part):
 POLICY = {"decode_mfma": True, "prefill_mfma": True}
 
 
-def attend(q, entry, table, ctx, window, scale, out):
+def attend(q, entry, table, ctx, window, scale, out, tile=64):
     """Softmax attention of q over the cache entry: picks the kernel for the step.
 
     float32, or a head size the MFMA kernels do not take: the plain kernel, one wave per
@@ -169,15 +182,16 @@ def attend(q, entry, table, ctx, window, scale, out):
         return K.attention_decode(q, entry.keys, entry.values, ctx.dev.tok_pos, table, window, scale, out)
     if q.dtype == torch.bfloat16 and POLICY["prefill_mfma"] and K.attention_prefill_supported(head_dim):
         d = ctx.dev
-        return K.attention_prefill(q, entry.keys, entry.values, d.tok_pos, table, d.tile_seq, d.tile_tok0, d.tile_count,
-                                   d.seq_start, d.seq_new, window, scale, out, tile_queries=ctx.tile_queries)
+        tile_seq, tile_tok0, tile_count = ctx.query_tiles(tile)
+        return K.attention_prefill(q, entry.keys, entry.values, d.tok_pos, table, tile_seq, tile_tok0, tile_count,
+                                   d.seq_start, d.seq_new, window, scale, out, tile_queries=tile)
     return K.attention(q, entry.keys, entry.values, ctx.dev.tok_seq, ctx.dev.tok_pos, table, window, scale, out)
 
 
 DECODE_KERNEL_ROWS = 32     # up to so many rows of a prompt step go through the decoding kernel
 
 
-def attend_rows(q, entry, table, ctx, window, scale, out):
+def attend_rows(q, entry, table, ctx, window, scale, out, tile=64):
     """The same for the step's last_rows alone (q holds their queries): the cache already holds
     the keys and values of all the step's tokens."""
     head_dim = q.shape[2]
@@ -188,7 +202,7 @@ def attend_rows(q, entry, table, ctx, window, scale, out):
         # kernel would walk them in one; a row is a sequence of its own to it
         return K.attention_decode(q, entry.keys, entry.values, d.last_pos, table.index_select(0, d.last_seq), window, scale, out)
     if q.dtype == torch.bfloat16 and POLICY["prefill_mfma"] and K.attention_prefill_supported(head_dim):
-        return K.attention_prefill(q, entry.keys, entry.values, d.last_pos, table, d.last_tile_seq, d.last_tile_tok0,
-                                   d.last_tile_count, d.seq_start, d.seq_new, window, scale, out,
-                                   tile_queries=ctx.tile_queries)
+        tile_seq, tile_tok0, tile_count = ctx.last_tiles(tile)
+        return K.attention_prefill(q, entry.keys, entry.values, d.last_pos, table, tile_seq, tile_tok0,
+                                   tile_count, d.seq_start, d.seq_new, window, scale, out, tile_queries=tile)
     return K.attention(q, entry.keys, entry.values, d.last_seq, d.last_pos, table, window, scale, out)

@@ -40,8 +40,10 @@ class KVNeed:
 
 @dataclass(frozen=True)
 class StateNeed:
-    """A mixer that keeps a fixed-size state per sequence (float32, zero at start)."""
+    """A mixer that keeps a fixed-size state per sequence (zero at start).  dtype: "float32",
+    "bfloat16" or "int32"."""
     shape: Tuple[int, ...]
+    dtype: str = "float32"
 
 
 @dataclass(frozen=True)
@@ -73,3 +75,10 @@ class ModelSpec:
     final_norm_prefix: str
     head_name: Optional[str]      # None: the head is the embedding matrix (tied)
     eos_token_ids: Tuple[int, ...] = ()
+    # What an architecture may do around the blocks; all off for the reference's decoder.
+    embedding_scale: Optional[float] = None        # the stream starts as embedding * scale
+    stream_position: Optional[PartSpec] = None     # a position part that acts on the stream after the
+    stream_position_prefix: str = ""               #   gather (add_to_stream), and where its tensors live
+    head_bias_name: Optional[str] = None           # logits += this tensor [vocab]
+    logit_scale: Optional[float] = None            # logits *= scale
+    logit_cap: Optional[float] = None              # logits = cap * tanh(logits / cap)
