@@ -621,9 +621,9 @@ def test_attention_decode_refuses_other_head_sizes():
                            torch.empty(1, 48, dtype=torch.bfloat16, device=DEV))
 
 
-@pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (3, 1, 96)])
+@pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (3, 1, 96), (40, 2, 64), (12, 2, 128)])
 @pytest.mark.parametrize("window", [0, 70, 12])
-@pytest.mark.parametrize("tile", [64, 128])
+@pytest.mark.parametrize("tile", [16, 32, 64, 128])
 def test_attention_prefill(nh, nkv, d, window, tile):
     # sequence 0: 150 new queries at positions 150..299 behind 150 cached ones; sequence 1: a
     # whole prompt of 70; sequence 2: one token at position 0.  Pages scrambled, unread places NaN.
@@ -924,11 +924,15 @@ def test_attention_decode_over_thousands_of_keys(nh, nkv, d, n_keys, window):
 
 
 @pytest.mark.parametrize("nh,nkv,d,spans,tile", [
-    (28, 4, 128, [(0, 2048)], 64),                    # the benchmarked prompt
-    (28, 4, 128, [(0, 3200)], 128),                   # the wider tile that long steps use
-    (28, 4, 128, [(1100, 2100), (0, 70)], 64),        # a piece of a prompt behind 1100 cached positions
+    (28, 4, 128, [(0, 2048)], 16),                    # the benchmarked prompt: two heads a wave, all blocks resident
+    (28, 4, 128, [(0, 2048)], 64),
+    (28, 4, 128, [(0, 3200)], 32),                    # a head a wave, blocks of seven waves shared out as they finish
+    (28, 4, 128, [(0, 3200)], 128),
+    (28, 4, 128, [(1100, 2100), (0, 70)], 32),        # a piece of a prompt behind 1100 cached positions
     (6, 2, 64, [(0, 2048), (500, 1300)], 128),
+    (40, 2, 64, [(0, 1500), (300, 900)], 32),         # groups of 20 heads: three blocks a group
     (3, 1, 96, [(0, 2500)], 64),
+    (5, 5, 32, [(0, 2100)], 128),
 ])
 @pytest.mark.parametrize("window", [0, 1000])
 def test_attention_prefill_over_thousands_of_keys(nh, nkv, d, spans, tile, window):

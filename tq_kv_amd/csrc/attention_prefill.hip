@@ -1,251 +1,402 @@
 // Attention for prompts (and any step with many tokens per sequence): causal softmax
-// attention of a tile of consecutive queries of one sequence and one head over the
-// sequence's pages of the cache, flash style: one pass over the keys, running maximum
-// and sum, float32 softmax, bfloat16 MFMA products.  Formulas as
-// src/models/turbo_generic.rs:1620-1631 and :56-62; the mask is right for queries that
-// start at any position (the reference's is only for position 0, :1937-1956), with an
-// optional window.
+// attention of a tile of consecutive queries of one sequence over the sequence's pages of
+// the cache, flash style: one pass over the keys, running maximum and sum, float32 softmax,
+// bfloat16 MFMA products.  Formulas as src/models/turbo_generic.rs:1620-1631 and :56-62; the
+// mask is right for queries that start at any position (the reference's is only for
+// position 0, :1937-1956), with an optional window.
 //
-// A block of 4 waves owns a tile of 64 or 128 queries; wave w owns 16 or 32 consecutive
-// ones.  Tiles late in a sequence see more keys than early ones: the host lists the tiles
-// longest first, and blocks are numbered heads-fastest, so that the blocks that share a
-// compute unit have different lengths and the long ones start first.  The pages of keys
-// (64 positions x head_dim) and of values (head_dim x 64 positions, stored transposed)
-// are staged in LDS once per block and read by all four waves; the next page is on
-// its way from global memory into registers while the current one is computed on.
+// Work of a block: one tile of queries, one kv head, and the query heads that share it (up
+// to 256 / tile of them; more are split over blocks): a page of keys and values is staged
+// in LDS once and serves all those heads, where the reference expands keys and values per
+// query head (src/models/turbo_generic.rs:195-204).  The columns (head, query) of the block
+// are dealt out 32 to a wave.  LDS holds two pages: the next page travels from global
+// memory into registers while this one is computed on and is written to the other buffer
+// afterwards, so a page costs one barrier.
 //
-// Matrix-core mapping as in the decoding kernel: scores^T = K Q^T puts a query in a
-// lane's column and 4 keys of each group of 16 in its registers, which is exactly the
-// operand layout that out^T = V^T P^T needs, so the probabilities never move.
-// LDS rows are padded (keys by 8 elements, values by 8 places) so that the lanes of a
-// read phase fall into different banks.
+// Matrix-core mapping, v_mfma_f32_32x32x16_bf16 (D[32x32] += A[32x16] B[16x32]; a lane
+// holds of A row l%32 and the 8 k starting at 8*(l/32), of B the same k of column l%32, of
+// D column l%32 and the rows 8*(i/4) + 4*(l/32) + i%4, i = 0..15):
+//   scores^T[key][column] = K[key][:] . Q^T[:][column]   A = keys from LDS, B = the queries, kept in registers
+//   out^T[element][column] = V^T[element][key] . P^T[key][column]
+// The probabilities never move: the lane's registers 8s..8s+7 of a score tile are the B
+// operand of step s of the second product, if the keys are dealt to the rows of the first
+// product so that those registers hold the 8 keys whose values lie together in the cache
+// (the cache keeps values transposed with the positions of a page in the order
+// value_place of common.h): row r = 8a + 4h + j of a tile of 32 keys is key
+// 4*(2*(a/2) + h) + 16*(a%2) + j.
+//
+// In LDS a row of keys takes 64, 128 or 256 bytes (head sizes 32, 64, 96 and 128; 96 is
+// padded), a row of values 128; the 16-byte pieces of a row are XOR-swizzled so that the lanes
+// of a read phase meet different banks.
+//
+// Softmax in base 2 (c = scale * log2 e): p = 2^(s*c - m).  The running maximum m is
+// raised only when a score exceeds it by more than 2^8 (then out and sum are rescaled);
+// until then p may be up to 2^8, which float32 sums and bfloat16 products carry as well.
 #include "common.h"
 #include "tq_kernels.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));      // a native vector: copies of it stay in registers
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+// pointers into LDS, typed as such: the compiler then tells the page being read from the page
+// under way (restrict) and does not make the reads wait for the loads
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+typedef __attribute__((address_space(3))) bf16x8_t lds_bf16x8;
+typedef __attribute__((address_space(3))) uint16_t lds_u16;
+typedef __attribute__((address_space(3))) u32x4_t lds_u32x4;
 
-#define PF_THREADS 256
-#define PF_WAVES (PF_THREADS / TQK_WAVE)
-#define PF_VPAD 8
+#define PF_MAX_WAVES 8
+#define PF_LAZY 8.0f            // how far (in powers of two) a score may exceed the running maximum before it is raised
 
-// QB: blocks of 16 queries per wave.  A wave reads every key and value operand from LDS once
-// and uses it for all its query blocks, so with QB = 2 (tiles of 128 queries) a query costs
-// half the LDS reads and half the staging of QB = 1 (tiles of 64), and a wave has two
-// independent chains of work; tiles of 64 leave fewer lanes idle on short prompts.
-template <int D, int QB>
-__global__ __launch_bounds__(PF_THREADS, 2)
-void attention_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ keys,
-                              const bf16_t* __restrict__ values, const int32_t* __restrict__ tok_pos,
-                              const int32_t* __restrict__ page_table, int table_width,
-                              const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_tok0,
-                              const int32_t* __restrict__ tile_count, const int32_t* __restrict__ seq_start,
-                              const int32_t* __restrict__ seq_new, int window, float scale,
-                              bf16_t* __restrict__ out, int n_heads, int n_kv_heads, int n_tiles, int snake_width) {
-    constexpr int KB = D / 32, DB = D / 16;
-    constexpr int KSTRIDE = D + 8;                   // elements per key row in LDS
-    constexpr int VSTRIDE = TQK_PAGE + PF_VPAD;      // elements per value row in LDS
-    constexpr int CHUNKS = D / 32;                   // 16-byte chunks per thread, per operand
-    constexpr int WQ = 16 * QB;                      // queries per wave
-    __shared__ __attribute__((aligned(16))) uint16_t k_lds[TQK_PAGE * KSTRIDE];
-    __shared__ __attribute__((aligned(16))) uint16_t v_lds[D * VSTRIDE];
+namespace {
 
-    const int tid = threadIdx.x;
-    const int wave = tid / TQK_WAVE, lane = tid % TQK_WAVE;
-    const int col = lane % 16, g = lane / 16;
-    // Blocks in the order of their work, heads fastest (the host lists the tiles longest first).
-    // With snake_width > 0 every other run of snake_width blocks is taken backwards: when all
-    // blocks are resident at once, the compute units that got the longest get the shortest next.
-    int order = blockIdx.x;
-    if (snake_width > 0) {
-        const int total = n_tiles * n_heads;
-        const int round = order / snake_width, first = round * snake_width;
-        const int size = min(snake_width, total - first);
-        if (round & 1) order = first + size - 1 - (order - first);
+// the key (0..31) that row r of a score tile holds
+__device__ __forceinline__ int tile_key(int r) {
+    const int a = r >> 3, h = (r >> 2) & 1, j = r & 3;
+    return 4 * (2 * (a >> 1) + h) + 16 * (a & 1) + j;
+}
+
+template <int D>
+struct Layout {
+    static constexpr int KROW = D <= 32 ? 64 : (D <= 64 ? 128 : 256);    // bytes of a key row in LDS
+    static constexpr int K_BYTES = 64 * KROW;
+    static constexpr int V_BYTES = D * 128;
+    // Where piece c of key row `key` lies, and where the 8 places pc*8.. of value row d (byte offsets
+    // inside a buffer).  Rows lie one after the other; the pieces of a row are XOR-swizzled with
+    // bits of the row's number, chosen so that the lanes that read together (8 or 16 lanes with
+    // consecutive rows of one tile of 32, see tile_key) meet different banks, whether a read phase
+    // covers 128 or 256 bytes of banks.
+    __device__ static __forceinline__ int k_at(int key, int c) {
+        const int f = KROW == 256 ? ((key & 7) | (((key >> 4) & 1) << 3))
+                    : KROW == 128 ? ((key & 7) ^ ((key >> 4) & 1))
+                                  : (((key >> 1) & 3) ^ ((key >> 4) & 1));
+        return key * KROW + ((c ^ f) << 4);
     }
-    const int tile = order / n_heads, head = order % n_heads;
-    const int kvh = head / (n_heads / n_kv_heads);
-    const int seq = tile_seq[tile], tok0 = tile_tok0[tile], count = tile_count[tile];
-    const int pos0 = tok_pos[tok0];
-    const int seq_end = seq_start[seq] + seq_new[seq];   // positions the cache holds after this step
-
-    // this lane's queries, one per query block
-    int qi[QB], my_pos[QB], my_lo[QB];
-    bool q_live[QB];
-#pragma unroll
-    for (int b = 0; b < QB; ++b) {
-        qi[b] = wave * WQ + b * 16 + col;
-        q_live[b] = qi[b] < count;
-        my_pos[b] = q_live[b] ? pos0 + qi[b] : -1;
-        my_lo[b] = window > 0 ? max(0, my_pos[b] - window + 1) : 0;
+    __device__ static __forceinline__ int v_at(int d, int pc) {
+        return d * 128 + ((pc ^ ((d & 7) ^ ((d >> 3) & 1))) << 4);
     }
-    // the wave's and the tile's ranges of positions
-    const bool wave_live = wave * WQ < count;
-    const int wave_last = min(pos0 + wave * WQ + WQ - 1, pos0 + count - 1);
-    const int wave_first = pos0 + wave * WQ;                  // the wave's first query: it sees the fewest late keys
-    const int wave_lo = window > 0 ? max(0, wave_first - window + 1) : 0;
-    const int wave_lo_last = window > 0 ? max(0, wave_last - window + 1) : 0;   // the wave's last query sees the fewest early keys
-    const float c2 = scale * 1.44269504088896340736f;
-    const int tile_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
-    const int first_page = tile_lo / TQK_PAGE, last_page = (pos0 + count - 1) / TQK_PAGE;
+};
 
-    const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    bf16x8_t bq[QB][KB];
+struct PrefillArgs {
+    const bf16_t* q;
+    const bf16_t* keys;
+    const bf16_t* values;
+    const int32_t* tok_pos;
+    const int32_t* page_table;
+    int table_width;
+    const int32_t* tile_seq;
+    const int32_t* tile_tok0;
+    const int32_t* tile_count;
+    const int32_t* seq_start;
+    const int32_t* seq_new;
+    int window;
+    float scale;
+    bf16_t* out;
+    int n_heads, n_kv_heads, n_tiles;
+    int tq_shift;            // log2 of the queries per tile
+    int heads_per_block, head_chunks;
+    int snake_width;
+};
+
+// What a wave knows about its place in the block's tile, and what it carries from page to page.
+template <int D>
+struct Wave {
+    static constexpr int KS = D / 16;           // k steps of the score product
+    static constexpr int DT = D / 32;           // tiles of 32 elements of the output
+    int tid, n_threads, wave, n_waves, lane, c32, h;
+    int kvh;
+    int my_pos, my_lo;                           // this lane's query and the first key it sees
+    bool wave_live;
+    int wave_first, wave_last, wave_lo, wave_lo_last;
+    int seq_end, last_page;
+    float c2;
+    const bf16_t* keys;
+    const bf16_t* values;
+    size_t page_stride;
+    bf16x8_t bq[KS];                             // the queries: B operand of the score product
+    float m, l;
+    floatx16_t o[DT];
+};
+
+// A page travels in two legs: from global memory into registers (fetch_page: 16 bytes a lane and
+// load, asked for before the work on the page before it and waited for after), and from there into
+// LDS (stage_page), each piece to its swizzled place.  Piece i of the keys is piece i % (D/8) of
+// key row i / (D/8); piece i of the values holds places 8 (i % 8) .. of element row i / 8.
+template <int D>
+__device__ __forceinline__ void fetch_page(const Wave<D>& w, int page, u32x4_t (&kr)[D / 32], u32x4_t (&vr)[D / 32]) {
+    const size_t base = (size_t)(page < 0 ? 0 : page) * w.page_stride + (size_t)w.kvh * TQK_PAGE * D;
+    const u32x4_t* kg = reinterpret_cast<const u32x4_t*>(w.keys + base);
+    const u32x4_t* vg = reinterpret_cast<const u32x4_t*>(w.values + base);
 #pragma unroll
-    for (int b = 0; b < QB; ++b) {
-        const bf16_t* qrow = q + ((size_t)(tok0 + (q_live[b] ? qi[b] : 0)) * n_heads + head) * D + g * 8;
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
-            bq[b][kb] = q_live[b] ? *reinterpret_cast<const bf16x8_t*>(qrow + kb * 32) : zero;
+    for (int c = 0; c < D / 32; ++c) {
+        const int i = min(w.tid + c * w.n_threads, 8 * D - 1);      // (beyond the page: its last piece again, not stored)
+        kr[c] = kg[i];
+        vr[c] = vg[i];
     }
+}
 
-    float m[QB], l[QB];
-    floatx4_t o[QB][DB];
+template <int D>
+__device__ __forceinline__ void stage_page(const Wave<D>& w, const u32x4_t (&kr)[D / 32], const u32x4_t (&vr)[D / 32],
+                                           lds_byte* __restrict__ kd, lds_byte* __restrict__ vd) {
+    using L = Layout<D>;
 #pragma unroll
-    for (int b = 0; b < QB; ++b) {
-        m[b] = -INFINITY;
-        l[b] = 0.f;
-#pragma unroll
-        for (int i = 0; i < DB; ++i) o[b][i] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-    }
-
-    const int32_t* pages = page_table + (size_t)seq * table_width;
-    const size_t page_stride = (size_t)n_kv_heads * TQK_PAGE * D;
-    u32x4_t kreg[CHUNKS], vreg[CHUNKS];
-
-    // the next page's keys and values travel from global memory into registers while the
-    // current page is computed on, and from there into LDS
-    auto fetch = [&](int pg, u32x4_t (&kr)[CHUNKS], u32x4_t (&vr)[CHUNKS]) {
-        const int page = pages[pg];
-        const size_t base = (size_t)(page < 0 ? 0 : page) * page_stride + (size_t)kvh * TQK_PAGE * D;
-        const u32x4_t* kp = reinterpret_cast<const u32x4_t*>(keys + base);
-        const u32x4_t* vp = reinterpret_cast<const u32x4_t*>(values + base);
-#pragma unroll
-        for (int c = 0; c < CHUNKS; ++c) {
-            kr[c] = kp[tid + c * PF_THREADS];
-            vr[c] = vp[tid + c * PF_THREADS];
-        }
-    };
-    auto stage = [&](int pg, const u32x4_t (&kr)[CHUNKS], const u32x4_t (&vr)[CHUNKS]) {
-        const int key0 = pg * TQK_PAGE;
-        const bool tail = key0 + TQK_PAGE > seq_end;       // the page holds places beyond the sequence
-#pragma unroll
-        for (int c = 0; c < CHUNKS; ++c) {
-            const int idx = tid + c * PF_THREADS;
-            // keys: chunk idx is elements 8*(idx % (D/8)).. of key row idx / (D/8)
-            const int krow = idx / (D / 8), kpart = idx % (D / 8);
-            *reinterpret_cast<u32x4_t*>(&k_lds[krow * KSTRIDE + kpart * 8]) = kr[c];
-            // values: chunk idx is positions 8*(idx % 8).. of element row idx / 8
-            const int vrow = idx / 8, vpart = idx % 8;
-            uint32_t vw[4] = {vr[c].x, vr[c].y, vr[c].z, vr[c].w};
-            if (tail) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i)     // nothing stored beyond the sequence may count
-                    if (key0 + value_position(vpart * 8 + i) >= seq_end) vw[i / 2] &= (i & 1) ? 0x0000ffffu : 0xffff0000u;
-            }
-            *reinterpret_cast<u32x4_t*>(&v_lds[vrow * VSTRIDE + vpart * 8]) = u32x4_t{vw[0], vw[1], vw[2], vw[3]};
-        }
-    };
-
-    fetch(first_page, kreg, vreg);
-    for (int pg = first_page; pg <= last_page; ++pg) {
-        __syncthreads();                       // everyone is done with the page in LDS
-        stage(pg, kreg, vreg);
-        __syncthreads();
-        fetch(min(pg + 1, last_page), kreg, vreg);           // (the last page again rather than a branch)
-        const int key0 = pg * TQK_PAGE;
-        if (!wave_live || key0 > wave_last || key0 + TQK_PAGE - 1 < wave_lo) continue;
-
-        // independent chains of products (one per group of 16 keys and query block), interleaved
-        floatx4_t s[QB][4];
-#pragma unroll
-        for (int b = 0; b < QB; ++b)
-#pragma unroll
-            for (int t = 0; t < 4; ++t) s[b][t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(&k_lds[(t * 16 + col) * KSTRIDE + kb * 32 + g * 8]);
-#pragma unroll
-                for (int b = 0; b < QB; ++b) s[b][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq[b][kb], s[b][t], 0, 0, 0);
-            }
-        // Softmax in base 2: with c = scale * log2(e), p = 2^(s*c - m) where m is the running
-        // maximum of s*c.  Only pages that cross a query's causal or window edge need the mask.
-        const bool need_mask = key0 + TQK_PAGE - 1 > wave_first || key0 < wave_lo_last;
-        bf16x8_t pb[QB][2];
-#pragma unroll
-        for (int b = 0; b < QB; ++b) {
-            float mx = -INFINITY;
-            if (need_mask) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int j = key0 + t * 16 + g * 4 + r;
-                        if (j < my_lo[b] || j > my_pos[b]) s[b][t][r] = -INFINITY;
-                        mx = fmaxf(mx, s[b][t][r]);
-                    }
-            } else {
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[b][t][r]);
-            }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, TQK_WAVE));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));
-            const float m_new = fmaxf(m[b], mx * c2);        // c2 > 0, so the maximum of s*c2 is c2 times the maximum of s
-            // a query may have no key in this page yet (window, or a lane without a query)
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m[b] - m_use);  // 2^(-inf) = 0 on a query's first keys
-            m[b] = m_new;
-            float psum = 0.f;
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float p = __builtin_amdgcn_exp2f(fmaf(s[b][t][r], c2, -m_use));
-                    // the probability enters the product as bfloat16; the sum uses the same rounded value
-                    const __bf16 pr16 = (__bf16)p;
-                    psum += (float)pr16;
-                    pb[b][t / 2][(t % 2) * 4 + r] = pr16;
-                }
-            l[b] = l[b] * alpha + psum;
-            if (__any(alpha != 1.f)) {
-#pragma unroll
-                for (int db = 0; db < DB; ++db) { o[b][db][0] *= alpha; o[b][db][1] *= alpha; o[b][db][2] *= alpha; o[b][db][3] *= alpha; }
-            }
-        }
-        // the lane's 8 keys of each half page lie together (value_place); independent chains
-#pragma unroll
-        for (int pr = 0; pr < 2; ++pr)
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(&v_lds[(db * 16 + col) * VSTRIDE + g * 8 + pr * 32]);
-#pragma unroll
-                for (int b = 0; b < QB; ++b) o[b][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pb[b][pr], o[b][db], 0, 0, 0);
-            }
-    }
-#pragma unroll
-    for (int b = 0; b < QB; ++b) {
-        float lb = l[b];
-        lb += __shfl_xor(lb, 16, TQK_WAVE);
-        lb += __shfl_xor(lb, 32, TQK_WAVE);
-        if (q_live[b]) {
-            // out^T[element db*16 + 4g + r][query col]
-            bf16_t* orow = out + ((size_t)(tok0 + qi[b]) * n_heads + head) * D;
-            const float inv = 1.f / lb;
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) orow[db * 16 + g * 4 + r] = from_float<bf16_t>(o[b][db][r] * inv);
+    for (int c = 0; c < D / 32; ++c) {
+        const int i = w.tid + c * w.n_threads;
+        if (i < 8 * D) {
+            *(lds_u32x4*)(kd + L::k_at(i / (D / 8), i % (D / 8))) = kr[c];
+            *(lds_u32x4*)(vd + L::v_at(i >> 3, i & 7)) = vr[c];
         }
     }
 }
 
+// The work on one page, held in kc, vc.
+template <int D>
+__device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_byte* __restrict__ kc, lds_byte* __restrict__ vc) {
+    using L = Layout<D>;
+    constexpr int KS = Wave<D>::KS, DT = Wave<D>::DT;
+    const int key0 = pg * TQK_PAGE;
+    const int c32 = w.c32, h = w.h;
+    if (key0 + TQK_PAGE > w.seq_end) {
+        // the page holds places beyond the sequence: whatever is stored there must not count,
+        // not even with probability 0 (0 * NaN); their values become zeros
+        const int valid = w.seq_end - key0;
+        for (int e = w.tid; e < D * 8; e += w.n_threads) {
+            const int d = e >> 3, pc = e & 7;
+            lds_u16* at = (lds_u16*)(vc + L::v_at(d, pc));
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (value_position(pc * 8 + i) >= valid) at[i] = 0;
+        }
+        __syncthreads();
+    }
+    if (!w.wave_live || page_now < 0) return;
+    const int krow = tile_key(c32);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        // a tile of 32 keys at a time
+        const int k0 = key0 + 32 * t;
+        if (k0 > w.wave_last || k0 + 31 < w.wave_lo) continue;
+        // all operands of the tile's score product first, so that their reads are under way together
+        bf16x8_t ka[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) ka[ks] = *(lds_bf16x8*)(kc + L::k_at(32 * t + krow, 2 * ks + h));
+        __builtin_amdgcn_sched_barrier(0);
+        floatx16_t s;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], w.bq[ks], s, 0, 0, 0);
+        // and the values of the second product, which arrive during the softmax
+        bf16x8_t va[2][DT];
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) va[st][dt] = *(lds_bf16x8*)(vc + L::v_at(32 * dt + c32, 4 * t + 2 * st + h));
+        __builtin_amdgcn_sched_barrier(0);
+        // the mask is needed only on tiles that cross a query's causal or window edge
+        const bool need_mask = k0 + 31 > w.wave_first || k0 < w.wave_lo_last;
+        if (need_mask) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int a = i >> 2;
+                const int j = k0 + 4 * (2 * (a >> 1) + h) + 16 * (a & 1) + (i & 3);
+                if (j < w.my_lo || j > w.my_pos) s[i] = -INFINITY;
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) mx = fmaxf(mx, fmaxf(s[i], s[i + 1]));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));         // the column's other 16 keys
+        const float top = mx * w.c2;                           // c2 > 0
+        if (__any(top > w.m + PF_LAZY)) {
+            // raise the running maximum (on a query's first keys m is -inf and alpha 0)
+            const float m_new = top > w.m + PF_LAZY ? top : w.m;
+            const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(w.m - m_new);
+            w.m = m_new;
+            w.l *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) w.o[dt][i] *= alpha;
+        }
+        const float m_use = w.m == -INFINITY ? 0.f : w.m;      // a column without a key so far: every p is 2^(-inf) = 0
+        bf16x8_t pb[2];
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float pr = __builtin_amdgcn_exp2f(fmaf(s[i], w.c2, -m_use));
+            psum += pr;
+            pb[i >> 3][i & 7] = (__bf16)pr;
+        }
+        w.l += psum;
+        // out^T += V^T P^T: step st takes the lane's registers 8 st .. 8 st + 7 and the 16 bytes of
+        // values that hold the same keys
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) w.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[st][dt], pb[st], w.o[dt], 0, 0, 0);
+    }
+}
+
+template <int D>
+__global__ __launch_bounds__(PF_MAX_WAVES * TQK_WAVE)
+void attention_prefill_kernel(const PrefillArgs p) {
+    using L = Layout<D>;
+    constexpr int KS = Wave<D>::KS, DT = Wave<D>::DT;
+    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * L::K_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * L::V_BYTES];
+    lds_byte* const kb = (lds_byte*)k_lds;
+    lds_byte* const vb = (lds_byte*)v_lds;
+
+    Wave<D> w;
+    w.tid = threadIdx.x;
+    w.n_threads = blockDim.x;
+    w.wave = w.tid / TQK_WAVE;
+    w.lane = w.tid % TQK_WAVE;
+    w.n_waves = blockDim.x / TQK_WAVE;
+    w.c32 = w.lane & 31;
+    w.h = w.lane >> 5;
+
+    // Blocks in the order of their work (the host lists the tiles longest first), kv heads and
+    // head chunks fastest.  With snake_width > 0 every other run of snake_width blocks is taken
+    // backwards: when all blocks are resident at once, the compute units that got the longest
+    // get the shortest next.
+    const int per_tile = p.n_kv_heads * p.head_chunks;
+    int order = blockIdx.x;
+    if (p.snake_width > 0) {
+        const int total = p.n_tiles * per_tile;
+        const int round = order / p.snake_width, first = round * p.snake_width;
+        const int size = min(p.snake_width, total - first);
+        if (round & 1) order = first + size - 1 - (order - first);
+    }
+    const int tile = order / per_tile, chunk = order % p.head_chunks;
+    w.kvh = (order % per_tile) / p.head_chunks;
+    const int n_rep = p.n_heads / p.n_kv_heads;
+    const int head0 = w.kvh * n_rep + chunk * p.heads_per_block;
+    const int heads_here = min(p.heads_per_block, n_rep - chunk * p.heads_per_block);
+    const int seq = p.tile_seq[tile], tok0 = p.tile_tok0[tile], count = p.tile_count[tile];
+    const int pos0 = p.tok_pos[tok0];
+    w.seq_end = p.seq_start[seq] + p.seq_new[seq];       // positions the cache holds after this step
+    const int tq = 1 << p.tq_shift;
+
+    // this lane's column: a query of a head
+    const int col = w.wave * 32 + w.c32;
+    const int head_local = col >> p.tq_shift, qi = col & (tq - 1);
+    const bool live = head_local < heads_here && qi < count;
+    const int head = head0 + (live ? head_local : 0);
+    w.my_pos = live ? pos0 + qi : -1;
+    w.my_lo = p.window > 0 ? max(0, w.my_pos - p.window + 1) : 0;
+    // the wave's range of queries (the same for all its heads)
+    const int wq_first = (w.wave * 32) & (tq - 1);
+    const int wq_last = min(tq >= 32 ? wq_first + 31 : tq - 1, count - 1);
+    w.wave_live = (w.wave * 32 >> p.tq_shift) < heads_here && wq_first < count;
+    w.wave_first = pos0 + wq_first;
+    w.wave_last = pos0 + wq_last;
+    w.wave_lo = p.window > 0 ? max(0, w.wave_first - p.window + 1) : 0;            // first key any of its queries sees
+    w.wave_lo_last = p.window > 0 ? max(0, w.wave_last - p.window + 1) : 0;        // first key all of them see
+    w.c2 = p.scale * 1.44269504088896340736f;
+    const int tile_lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
+    const int first_page = tile_lo / TQK_PAGE;
+    w.last_page = (pos0 + count - 1) / TQK_PAGE;
+    w.keys = p.keys;
+    w.values = p.values;
+    w.page_stride = (size_t)p.n_kv_heads * TQK_PAGE * D;
+
+    const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    {
+        const bf16_t* qrow = p.q + ((size_t)(tok0 + (live ? qi : 0)) * p.n_heads + head) * D + w.h * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) w.bq[ks] = live ? *reinterpret_cast<const bf16x8_t*>(qrow + ks * 16) : zero8;
+    }
+    w.m = -INFINITY;
+    w.l = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) w.o[dt][i] = 0.f;
+
+    // Two buffers: while a page is worked on, the next one is on its way into registers, and goes
+    // into the other buffer afterwards; one barrier per page.
+    const int32_t* pages = p.page_table + (size_t)seq * p.table_width;
+    u32x4_t kr[D / 32], vr[D / 32];
+    int page_now = pages[first_page];
+    fetch_page<D>(w, page_now, kr, vr);
+    stage_page<D>(w, kr, vr, kb + (first_page & 1) * L::K_BYTES, vb + (first_page & 1) * L::V_BYTES);
+    for (int pg = first_page; pg <= w.last_page; ++pg) {
+        const int cur = pg & 1;
+        __syncthreads();                      // the page is whole; all are done with the other buffer
+        int page_next = -1;
+        if (pg < w.last_page) {
+            page_next = pages[pg + 1];
+            fetch_page<D>(w, page_next, kr, vr);
+        }
+        page_step<D>(w, pg, page_now, kb + cur * L::K_BYTES, vb + cur * L::V_BYTES);
+        if (pg < w.last_page) stage_page<D>(w, kr, vr, kb + (cur ^ 1) * L::K_BYTES, vb + (cur ^ 1) * L::V_BYTES);
+        page_now = page_next;
+    }
+    float l = w.l;
+    l += __shfl_xor(l, 32, TQK_WAVE);
+    if (live) {
+        // out^T[element 32 dt + 8 (i/4) + 4 h + i%4][this column]
+        bf16_t* orow = p.out + ((size_t)(tok0 + qi) * p.n_heads + head) * D;
+        const float inv = 1.f / l;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                uint16_t w4[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) w4[j] = float_to_bf16_bits(w.o[dt][4 * a + j] * inv);
+                *reinterpret_cast<uint2*>(orow + 32 * dt + 8 * a + 4 * w.h) =
+                    make_uint2((uint32_t)w4[0] | ((uint32_t)w4[1] << 16), (uint32_t)w4[2] | ((uint32_t)w4[3] << 16));
+            }
+    }
+}
+
+}  // namespace
+
 extern "C" int tqk_attention_prefill_supported(int head_dim) {
     return head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128;
+}
+
+// Heads of a group that one block takes for tiles of tile_queries, and in how many chunks the
+// group is then cut: as many heads as 8 waves of 32 columns hold, dealt out evenly.
+static void prefill_heads(int n_rep, int tile_queries, int* heads_per_block, int* chunks) {
+    const int most = 32 * PF_MAX_WAVES / tile_queries;
+    *chunks = (n_rep + most - 1) / most;
+    *heads_per_block = (n_rep + *chunks - 1) / *chunks;
+}
+
+static int prefill_compute_units(void) {
+    static int n_cus = 0;
+    if (n_cus == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+            return 0;
+        n_cus = v;
+    }
+    return n_cus;
+}
+
+/* Queries per tile that suit a step of n_tokens: tiles of 64 (a wave holds 32 queries of one
+ * head, a block four heads) where that gives several blocks per compute unit to share out,
+ * tiles of 16 (two heads a wave) for shorter steps; groups of few heads take longer tiles, so
+ * that a block has at least four waves. */
+extern "C" int tqk_attention_prefill_tile(int n_tokens, int n_heads, int n_kv_heads, int head_dim) {
+    (void)head_dim;
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads) return 64;
+    const int n_rep = n_heads / n_kv_heads;
+    if (n_rep == 1) return 128;
+    if (n_rep <= 3) return 64;
+    int n_cus = prefill_compute_units();
+    if (n_cus <= 0) n_cus = 256;
+    int hb, chunks;
+    prefill_heads(n_rep, 32, &hb, &chunks);
+    const long long blocks32 = (long long)((n_tokens + 31) / 32) * n_kv_heads * chunks;
+    // measured with groups of 7 heads of 128: 2048 tokens run fastest in tiles of 16 (512 blocks of
+    // four waves), 8192 and more in tiles of 64 (blocks of 8 and 6 waves)
+    if (blocks32 >= 2LL * n_cus) return 64;
+    return n_rep == 4 ? 32 : 16;
 }
 
 extern "C" int tqk_attention_prefill(const void* q, const void* keys, const void* values, const int32_t* tok_pos,
@@ -261,32 +412,38 @@ extern "C" int tqk_attention_prefill(const void* q, const void* keys, const void
     TQK_REQUIRE(tqk_attention_prefill_supported(head_dim), "tqk_attention_prefill: head_dim %d is not one of 32, 64, 96, 128", head_dim);
     TQK_REQUIRE(table_width > 0 && n_pages > 0 && n_seqs > 0, "tqk_attention_prefill: empty page table");
     TQK_REQUIRE(window >= 0, "tqk_attention_prefill: negative window");
-    TQK_REQUIRE(tile_queries == 64 || tile_queries == 128, "tqk_attention_prefill: tiles hold 64 or 128 queries, not %d", tile_queries);
-    TQK_REQUIRE((long long)n_tiles * n_heads <= 0x7fffffffLL, "tqk_attention_prefill: %d tiles are more than the grid takes", n_tiles);
+    TQK_REQUIRE(tile_queries == 16 || tile_queries == 32 || tile_queries == 64 || tile_queries == 128,
+                "tqk_attention_prefill: tiles hold 16, 32, 64 or 128 queries, not %d", tile_queries);
+    TQK_REQUIRE((((uintptr_t)q | (uintptr_t)keys | (uintptr_t)values | (uintptr_t)out) & 15) == 0,
+                "tqk_attention_prefill: q, keys, values and out must be 16-byte aligned");
     if (n_tiles == 0) return 0;
+    PrefillArgs a;
+    a.q = (const bf16_t*)q; a.keys = (const bf16_t*)keys; a.values = (const bf16_t*)values;
+    a.tok_pos = tok_pos; a.page_table = page_table; a.table_width = table_width;
+    a.tile_seq = tile_seq; a.tile_tok0 = tile_tok0; a.tile_count = tile_count;
+    a.seq_start = seq_start; a.seq_new = seq_new; a.window = window; a.scale = scale;
+    a.out = (bf16_t*)out; a.n_heads = n_heads; a.n_kv_heads = n_kv_heads; a.n_tiles = n_tiles;
+    a.tq_shift = tile_queries == 16 ? 4 : (tile_queries == 32 ? 5 : (tile_queries == 64 ? 6 : 7));
+    prefill_heads(n_heads / n_kv_heads, tile_queries, &a.heads_per_block, &a.head_chunks);
+    // at least four waves: the page's journey through registers is dealt out to 256 threads or more
+    const int waves = max(4, (a.heads_per_block * tile_queries + 31) / 32);
+    const long long total = (long long)n_tiles * n_kv_heads * a.head_chunks;
+    TQK_REQUIRE(total <= 0x7fffffffLL, "tqk_attention_prefill: %d tiles are more than the grid takes", n_tiles);
+    const int n_cus = prefill_compute_units();
+    TQK_REQUIRE(n_cus > 0, "tqk_attention_prefill: cannot read the number of compute units");
+    // Blocks that are all resident at once (a compute unit holds 8 such waves) are not shared out
+    // as they finish: then the runs of one block per compute unit alternate their direction.
+    const int per_cu = waves <= 4 ? 2 : 1;
+    a.snake_width = (total > n_cus && total <= (long long)per_cu * n_cus) ? n_cus : 0;
     hipStream_t s = (hipStream_t)stream;
-    // all blocks resident at once (two per compute unit): alternate the direction of the runs
-    static int n_cus = 0;
-    if (n_cus == 0) {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
-            return tqk_fail("tqk_attention_prefill: cannot read the number of compute units");
-        n_cus = v;
-    }
-    const long long total = (long long)n_tiles * n_heads;
-    const int snake = total <= 2LL * n_cus ? n_cus : 0;
     dim3 grid((unsigned)total);
-#define LAUNCH(DD, QQ) attention_prefill_kernel<DD, QQ><<<grid, PF_THREADS, 0, s>>>( \
-        (const bf16_t*)q, (const bf16_t*)keys, (const bf16_t*)values, tok_pos, page_table, table_width, tile_seq, tile_tok0, \
-        tile_count, seq_start, seq_new, window, scale, (bf16_t*)out, n_heads, n_kv_heads, n_tiles, snake)
-#define LAUNCH_D(DD) do { if (tile_queries == 128) LAUNCH(DD, 2); else LAUNCH(DD, 1); } while (0)
+#define LAUNCH(DD) attention_prefill_kernel<DD><<<grid, waves * TQK_WAVE, 0, s>>>(a)
     switch (head_dim) {
-        case 32: LAUNCH_D(32); break;
-        case 64: LAUNCH_D(64); break;
-        case 96: LAUNCH_D(96); break;
-        case 128: LAUNCH_D(128); break;
+        case 32: LAUNCH(32); break;
+        case 64: LAUNCH(64); break;
+        case 96: LAUNCH(96); break;
+        case 128: LAUNCH(128); break;
     }
-#undef LAUNCH_D
 #undef LAUNCH
     return tqk_check_launch("tqk_attention_prefill");
 }

@@ -133,11 +133,14 @@ int tqk_attention_decode(const void* q, const void* keys, const void* values, co
                          float scale, int n_parts, void* part_out, void* part_ml,
                          void* out, int n_heads, int n_kv_heads, int head_dim, void* stream);
 
-/* Prompts: tiles of up to 64 consecutive queries of one sequence (tile i: sequence
- * tile_seq[i], first packed token tile_tok0[i], tile_count[i] queries) over the sequence's
- * pages, causal with optional window, bfloat16, MFMA.  seq_start + seq_new is the number
- * of positions a sequence's cache holds after this step. */
+/* Prompts: tiles of up to tile_queries (16, 32, 64 or 128) consecutive queries of one sequence
+ * (tile i: sequence tile_seq[i], first packed token tile_tok0[i], tile_count[i] queries, none more
+ * than tile_queries) over the sequence's pages, causal with optional window, bfloat16, MFMA; the
+ * tiles are best listed longest reach first.  seq_start + seq_new is the number of positions a
+ * sequence's cache holds after this step.  tqk_attention_prefill_tile: the tile size that suits
+ * a step of n_tokens. */
 int tqk_attention_prefill_supported(int head_dim);
+int tqk_attention_prefill_tile(int n_tokens, int n_heads, int n_kv_heads, int head_dim);
 int tqk_attention_prefill(const void* q, const void* keys, const void* values, const int32_t* tok_pos,
                           const int32_t* page_table, int table_width, int n_seqs, int n_pages,
                           const int32_t* tile_seq, const int32_t* tile_tok0, const int32_t* tile_count,

@@ -309,9 +309,14 @@ def attention_prefill_supported(head_dim):
     return bool(library().tqk_attention_prefill_supported(int(head_dim)))
 
 
+def attention_prefill_tile(n_tokens, n_heads, n_kv_heads, head_dim):
+    """Queries per tile (16, 32, 64 or 128) that suit a step of n_tokens for these head counts."""
+    return int(library().tqk_attention_prefill_tile(int(n_tokens), int(n_heads), int(n_kv_heads), int(head_dim)))
+
+
 def attention_prefill(q, keys, values, tok_pos, page_table, tile_seq, tile_tok0, tile_count, seq_start, seq_new,
                       window, scale, out, tile_queries=64):
-    """Causal attention of tiles of up to tile_queries (64 or 128) consecutive queries
+    """Causal attention of tiles of up to tile_queries (16, 32, 64 or 128) consecutive queries
     (q [T, heads, d] bfloat16) over the paged cache; out [T, heads*d].  tile_count must not
     exceed tile_queries (the caller built the tiles; the kernel covers no more)."""
     n, n_heads, head_dim = q.shape

@@ -20,12 +20,8 @@ from .spec import KVNeed, TensorSpec
 class Attention(Part):
     """params: hidden, n_heads, n_kv_heads, head_dim, qkv_bias (bool), out_bias (bool),
     window (None or positions a query sees, itself included), scale (None: 1/sqrt(head_dim)),
-    position (PartSpec); optional prompt_tiles = (queries per tile of the prompt kernel, the wider
-    tile, the step size in tokens from which the wider one is used)."""
-
-    # Measured with 28 heads of 128: 2048 tokens run faster in tiles of 64 queries (more blocks to
-    # share out), 4096 and more in tiles of 128 (less staging per query).
-    PROMPT_TILES = (64, 128, 3072)
+    position (PartSpec); optional prompt_tile: queries per tile of the prompt kernel (16, 32, 64 or
+    128; default: what the kernel library finds fitting for the step's size and these head counts)."""
 
     def __init__(self, params, env):
         self.env = env
@@ -43,9 +39,9 @@ class Attention(Part):
             raise ValueError("attention: window must be at least 1, got %r" % (self.window,))
         scale = params.get("scale")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
-        self.prompt_tiles = tuple(int(v) for v in params.get("prompt_tiles", self.PROMPT_TILES))
-        if len(self.prompt_tiles) != 3 or any(t not in (64, 128) for t in self.prompt_tiles[:2]):
-            raise ValueError("attention: prompt_tiles must be (64 or 128, 64 or 128, tokens), got %r" % (self.prompt_tiles,))
+        self.prompt_tile = params.get("prompt_tile")
+        if self.prompt_tile is not None and self.prompt_tile not in (16, 32, 64, 128):
+            raise ValueError("attention: prompt_tile must be 16, 32, 64 or 128, got %r" % (self.prompt_tile,))
         spec = params["position"]
         key = ("position", spec.kind, tuple(sorted(spec.params.items())))
         if key not in env.shared:
@@ -127,10 +123,10 @@ class Attention(Part):
             if ctx.n_last == 0:
                 return torch.empty((0, self.hidden), dtype=dtype, device=q.device)
             y = torch.empty((ctx.n_last, self.n_heads * self.head_dim), dtype=dtype, device=q.device)
-            attend_rows(q.index_select(0, d.last_rows), entry, table, ctx, self.window, self.scale, y, self.tile_for(ctx))
+            attend_rows(q.index_select(0, d.last_rows), entry, table, ctx, self.window, self.scale, y, self.tile_for)
             return linear(y, self.w_o, self.b_o, few=self.few_o)
         y = torch.empty((n, self.n_heads * self.head_dim), dtype=dtype, device=q.device)
-        attend(q, entry, table, ctx, self.window, self.scale, y, self.tile_for(ctx))
+        attend(q, entry, table, ctx, self.window, self.scale, y, self.tile_for)
         if stream is not None:
             stream.add_product(y, self.few_o or self.w_o)
             return None
@@ -138,8 +134,14 @@ class Attention(Part):
 
     def tile_for(self, ctx):
         """Queries per tile of the prompt kernel for this step."""
-        small, wide, wide_from = self.prompt_tiles
-        return wide if ctx.n_tokens >= wide_from else small
+        if self.prompt_tile is not None:
+            return self.prompt_tile
+        if not hasattr(ctx, "_prompt_tile"):
+            ctx._prompt_tile = {}
+        key = (self.n_heads, self.n_kv_heads, self.head_dim)
+        if key not in ctx._prompt_tile:
+            ctx._prompt_tile[key] = K.attention_prefill_tile(ctx.n_tokens, *key)
+        return ctx._prompt_tile[key]
 
     def _qkv(self, x, ctx, entry, table, q):
         """Product, then bias, position encoding and cache write in their own kernel."""
@@ -171,7 +173,7 @@ class Attention(Part):
 POLICY = {"decode_mfma": True, "prefill_mfma": True}
 
 
-def attend(q, entry, table, ctx, window, scale, out, tile=64):
+def attend(q, entry, table, ctx, window, scale, out, tile_for=None):
     """Softmax attention of q over the cache entry: picks the kernel for the step.
 
     float32, or a head size the MFMA kernels do not take: the plain kernel, one wave per
@@ -182,6 +184,7 @@ def attend(q, entry, table, ctx, window, scale, out, tile=64):
         return K.attention_decode(q, entry.keys, entry.values, ctx.dev.tok_pos, table, window, scale, out)
     if q.dtype == torch.bfloat16 and POLICY["prefill_mfma"] and K.attention_prefill_supported(head_dim):
         d = ctx.dev
+        tile = tile_for(ctx) if tile_for is not None else 64
         tile_seq, tile_tok0, tile_count = ctx.query_tiles(tile)
         return K.attention_prefill(q, entry.keys, entry.values, d.tok_pos, table, tile_seq, tile_tok0, tile_count,
                                    d.seq_start, d.seq_new, window, scale, out, tile_queries=tile)
@@ -191,7 +194,7 @@ def attend(q, entry, table, ctx, window, scale, out, tile=64):
 DECODE_KERNEL_ROWS = 32     # up to so many rows of a prompt step go through the decoding kernel
 
 
-def attend_rows(q, entry, table, ctx, window, scale, out, tile=64):
+def attend_rows(q, entry, table, ctx, window, scale, out, tile_for=None):
     """The same for the step's last_rows alone (q holds their queries): the cache already holds
     the keys and values of all the step's tokens."""
     head_dim = q.shape[2]
@@ -202,6 +205,7 @@ def attend_rows(q, entry, table, ctx, window, scale, out, tile=64):
         # kernel would walk them in one; a row is a sequence of its own to it
         return K.attention_decode(q, entry.keys, entry.values, d.last_pos, table.index_select(0, d.last_seq), window, scale, out)
     if q.dtype == torch.bfloat16 and POLICY["prefill_mfma"] and K.attention_prefill_supported(head_dim):
+        tile = tile_for(ctx) if tile_for is not None else 64
         tile_seq, tile_tok0, tile_count = ctx.last_tiles(tile)
         return K.attention_prefill(q, entry.keys, entry.values, d.last_pos, table, tile_seq, tile_tok0,
                                    tile_count, d.seq_start, d.seq_new, window, scale, out, tile_queries=tile)
