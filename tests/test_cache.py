@@ -5,7 +5,7 @@ import random
 import pytest
 import torch
 
-from tq_kv_amd.cache import PAGE, Cache, CacheFull, FreeList
+from tq_kv_amd.cache import PAGE, Cache, CacheFull
 from tq_kv_amd.parts.spec import KVNeed, StateNeed
 
 FULL = KVNeed(2, 16, None)
@@ -14,21 +14,6 @@ WIN = KVNeed(2, 16, 100)
 
 def make(needs, cache_of=None, max_tokens=PAGE * 8, max_slots=4):
     return Cache(needs, cache_of or [None] * len(needs), max_tokens, max_slots, torch.float32, "cpu")
-
-
-def test_free_list():
-    f = FreeList(3, "page")
-    a = f.take(2)
-    assert sorted(a) == [0, 1] and f.n_free == 1
-    with pytest.raises(CacheFull):
-        f.take(2)
-    assert f.n_free == 1                        # a refused request takes nothing
-    f.give_back([a[0]])
-    with pytest.raises(AssertionError):
-        f.give_back([a[0]])                     # freed twice
-    with pytest.raises(AssertionError):
-        f.give_back([7])
-    f.check()
 
 
 def test_lengths_after_prompt_and_single_tokens():

@@ -1,0 +1,89 @@
+"""The arrays of a step as the engine's host library lays them out (tqe_plan_step), without a
+GPU: against a plain construction of the same arrays, for random batches."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from tq_kv_amd import native
+from tq_kv_amd.cache import PAGE, Cache, CacheFull
+from tq_kv_amd.engine.context import StepContext
+from tq_kv_amd.parts.spec import KVNeed
+
+
+def plain_arrays(items, want):
+    lens = [len(t) for _, _, t in items]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    tok_seq = np.repeat(np.arange(len(items)), lens)
+    tok_pos = np.concatenate([np.arange(start, start + n) for (_, start, _), n in zip(items, lens)])
+    rows = [int(cu[i]) + j for i, w in enumerate(want) for j in w]
+    last = sorted(set(rows))
+    all_decode = all(n == 1 for n in lens)
+    prune = not all_decode and len(last) < sum(lens)
+    return dict(tokens=np.concatenate([t for _, _, t in items]), tok_seq=tok_seq, tok_pos=tok_pos,
+                seq_slot=[s for s, _, _ in items], seq_start=[s for _, s, _ in items], seq_new=lens, cu=cu, want_rows=rows,
+                last_rows=last if prune else [], want_in_last=[last.index(r) for r in rows] if prune else [],
+                last_seq=[int(tok_seq[r]) for r in last] if prune else [], last_pos=[int(tok_pos[r]) for r in last] if prune else []), \
+        dict(n_tokens=sum(lens), n_last=len(last), all_decode=all_decode, prune_last=prune, max_new=max(lens),
+             max_end=max(s + n for (_, s, _), n in zip(items, lens)))
+
+
+def test_step_arrays_equal_a_plain_construction():
+    rng = random.Random(3)
+    cache = Cache([KVNeed(2, 16, None), KVNeed(2, 16, 100)], [None, None], PAGE * 64, 8, torch.float32, "cpu")
+    slots = [cache.acquire() for _ in range(6)]
+    for round_ in range(40):
+        chosen = rng.sample(slots, rng.randint(1, len(slots)))
+        decode = rng.random() < 0.4
+        items, want = [], []
+        for s in chosen:
+            n = 1 if decode else rng.choice([1, 2, 7, 64, 65, 130])
+            if cache.length(s) + n > 1000:
+                cache.release(s)
+                slots[slots.index(s)] = s = cache.acquire()
+            items.append((s, cache.length(s), [rng.randrange(1000) for _ in range(n)]))
+            want.append([rng.randrange(n) for _ in range(rng.choice([0, 1, 1, 3]))] if rng.random() < 0.8 else list(range(n)))
+        sizes = [(s, len(t)) for s, _, t in items]
+        cache.reserve(sizes)
+        step = rng.choice([1, 8])
+        ctx = StepContext(items, want, cache, None, None, step, into=object())
+        arrays, facts = plain_arrays(items, want)
+        for name, value in arrays.items():
+            assert getattr(ctx.host, name).tolist() == [int(v) for v in value], (round_, name)
+        for name, value in facts.items():
+            assert getattr(ctx, name) == value, (round_, name)
+        for g, table in zip(cache.kv_groups, ctx.host_tables):
+            want_table = cache.page_table(g, [s for s, _, _ in items])
+            width = (want_table.shape[1] + step - 1) // step * step
+            assert table.shape == (len(items), width)
+            assert table[:, :want_table.shape[1]].tolist() == want_table.tolist() and (table[:, want_table.shape[1]:] == -1).all()
+        assert ctx.shape_key() == (facts["n_tokens"], len(items), len(arrays["want_rows"]), tuple(t.shape[1] for t in ctx.host_tables))
+        cache.commit(sizes)
+        cache.check()
+    with pytest.raises(IndexError, match="wanted place 2"):
+        StepContext([(slots[0], 0, [1, 2])], [[2]], cache, None, None, 1, into=object())
+
+
+def test_the_native_cache_reports_what_goes_wrong():
+    c = native.NativeCache(2, [(3, 0)])
+    a, b = c.acquire(), c.acquire()
+    assert (a, b) == (0, 1) and c.counts(-1) == (0, 2)
+    with pytest.raises(CacheFull, match="0 free of 2"):
+        c.acquire()
+    c.release(a)
+    with pytest.raises(AssertionError, match="slot 0 given back but not held"):
+        c.release(a)
+    with pytest.raises(AssertionError, match="slot 0 is not held"):
+        c.reserve([(a, 1)])
+    assert c.acquire() == a                       # what came back last goes out first
+    c.reserve([(a, PAGE + 1)])
+    assert c.pages(0, a) == [0, 1] and c.pages(0, b) is None and c.counts(0) == (1, 3)
+    with pytest.raises(CacheFull, match="2 more pages"):
+        c.reserve([(b, 2 * PAGE)])
+    assert c.pages(0, b) is None and c.counts(0) == (1, 3)        # nothing was taken
+    c.commit([(a, PAGE + 1)])
+    assert c.length(a) == PAGE + 1
+    c.check()
+    with pytest.raises(native.EngineLibraryError, match="no slot 7"):
+        c.length(7)

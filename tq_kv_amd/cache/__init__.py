@@ -1,4 +1,4 @@
-from .pages import CacheFull, FreeList
+from .pages import CacheFull
 from .store import PAGE, Cache, KVEntry, StateEntry
 
-__all__ = ["CacheFull", "FreeList", "PAGE", "Cache", "KVEntry", "StateEntry"]
+__all__ = ["CacheFull", "PAGE", "Cache", "KVEntry", "StateEntry"]

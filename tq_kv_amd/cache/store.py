@@ -13,6 +13,10 @@ window gives pages back as soon as every position in them has left the window; a
 group without keeps them until the slot is released.  Mixers with a fixed-size
 state get one float32 row per slot, zeroed when the slot is taken.
 
+The bookkeeping (free slots, lengths, page lists) is the engine's host library's
+(csrc/host_engine.cpp behind the C boundary csrc/tq_engine.h); the classes here own the
+storage tensors and show the bookkeeping to Python.
+
 The reference keeps one growing tensor pair per layer and one sequence
 (src/models/turbo_generic.rs:1606-1618) and resets by position
 (src/engine.rs:322-324); lengths after prompt(8), +1, +1 are 8, 9, 10 as in
@@ -21,8 +25,9 @@ tq-kv/src/candle_kv.rs:266-299.
 import numpy as np
 import torch
 
+from .. import native
 from ..parts.spec import KVNeed, StateNeed
-from .pages import CacheFull, FreeList
+from .pages import CacheFull
 
 PAGE = 64
 
@@ -54,44 +59,72 @@ class StateEntry:
         self.writes = writes
 
 
+class _PoolView:
+    """Free and held counts of a pool of the native cache (the slots, or a group's pages)."""
+
+    def __init__(self, cache, group):
+        self._cache, self._group = cache, group
+
+    @property
+    def n(self):
+        return self._cache.counts(self._group)[1]
+
+    @property
+    def n_free(self):
+        return self._cache.counts(self._group)[0]
+
+    @property
+    def n_held(self):
+        free, total = self._cache.counts(self._group)
+        return total - free
+
+    def is_held(self, i):
+        if self._group != -1:
+            raise TypeError("only slots can be asked for one by one")
+        return self._cache.is_held(i)
+
+
+class _PagesView:
+    """slot -> list of page ids (-1 where given back) of a group, read from the native cache."""
+
+    def __init__(self, cache, group):
+        self._cache, self._group = cache, group
+
+    def get(self, slot, default=None):
+        have = self._cache.pages(self._group, slot)
+        return default if have is None else have
+
+    def __getitem__(self, slot):
+        have = self._cache.pages(self._group, slot)
+        if have is None:
+            raise KeyError(slot)
+        return have
+
+    def __contains__(self, slot):
+        return self._cache.pages(self._group, slot) is not None
+
+    def __iter__(self):
+        return (s for s in range(self._cache.max_slots) if s in self)
+
+    def values(self):
+        return [self[s] for s in self]
+
+
 class KVGroup:
     def __init__(self, need, runs, n_pages, dtype, device):
         self.need = need
         self.runs = list(runs)
-        self.pool = FreeList(n_pages, "page")
+        self.n_pages = n_pages
         shape = (len(self.runs), n_pages, need.n_kv_heads, PAGE, need.head_dim)
         self.keys = torch.zeros(shape, dtype=dtype, device=device)
         self.values = torch.zeros(shape[:3] + (need.head_dim, PAGE), dtype=dtype, device=device)
-        self.pages = {}               # slot -> list of page ids, -1 where given back
+        self.pool = self.pages = None      # views of the native bookkeeping, set by the cache
 
     def first_needed(self, length):
         """First position a query at or after `length` can still see."""
         if self.need.window is None:
             return 0
         return max(0, length + 1 - self.need.window)
-
-    def missing(self, slot, new_length):
-        return max(0, pages_for(new_length) - len(self.pages.get(slot, ())))
-
-    def extend(self, slot, new_length):
-        have = self.pages.setdefault(slot, [])
-        have.extend(self.pool.take(pages_for(new_length) - len(have)))
-
-    def trim(self, slot, length):
-        """Give back the pages whose positions are all out of the window."""
-        if self.need.window is None:
-            return
-        have = self.pages.get(slot, [])
-        dead = min(self.first_needed(length) // PAGE, len(have))
-        gone = [p for p in have[:dead] if p >= 0]
-        if gone:
-            self.pool.give_back(gone)
-            for i in range(dead):
-                have[i] = -1
-
-    def release(self, slot):
-        have = self.pages.pop(slot, [])
-        self.pool.give_back([p for p in have if p >= 0])
 
 
 STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
@@ -128,8 +161,6 @@ class Cache:
         self.n_pages = max_tokens // PAGE if self.holds_pages else 0
         self.max_slots = max(1, min(int(max_slots), self.n_pages)) if self.holds_pages else max(1, int(max_slots))
         self.device = device
-        self.slots = FreeList(self.max_slots, "slot")
-        self.lengths = [0] * self.max_slots
         self.kv_groups = []
         self.state_groups = []
         self._entry = {}              # run index -> (group, index within group)
@@ -149,6 +180,15 @@ class Cache:
                 raise TypeError("unknown cache need %r" % (need,))
             for i, run in enumerate(runs):
                 self._entry[run] = (group, i)
+        if len(self.kv_groups) > native.MAX_GROUPS:
+            raise ValueError("%d groups of cached runs, the engine's library takes %d" % (len(self.kv_groups), native.MAX_GROUPS))
+        # the bookkeeping: free slots, lengths, page lists
+        self.native = native.NativeCache(self.max_slots, [(g.n_pages, g.need.window) for g in self.kv_groups])
+        self.slots = _PoolView(self.native, -1)
+        for i, g in enumerate(self.kv_groups):
+            g.index = i
+            g.pool = _PoolView(self.native, i)
+            g.pages = _PagesView(self.native, i)
         self._views = {}
         for run, need in enumerate(needs):
             src = cache_of[run]
@@ -167,52 +207,38 @@ class Cache:
     # -- slots ------------------------------------------------------------
     def acquire(self):
         """A free slot with length 0 and zeroed state."""
-        slot = self.slots.take(1)[0]
-        self.lengths[slot] = 0
+        slot = self.native.acquire()
         for g in self.state_groups:
             g.reset(slot)
         return slot
 
     def release(self, slot):
         """Give the slot and everything it holds back."""
-        self.slots.give_back([slot])
-        for g in self.kv_groups:
-            g.release(slot)
-        self.lengths[slot] = 0
+        self.native.release(slot)
 
     def length(self, slot):
-        return self.lengths[slot]
+        return self.native.length(slot)
+
+    @property
+    def lengths(self):
+        return [self.native.length(s) for s in range(self.max_slots)]
 
     # -- one step ---------------------------------------------------------
     def reserve(self, items):
         """items: [(slot, n_new)].  Make room for n_new more positions in every group,
         for all sequences or (CacheFull) for none."""
-        for g in self.kv_groups:
-            want = 0
-            for slot, n_new in items:
-                if not self.slots.is_held(slot):
-                    raise AssertionError("slot %d is not held" % slot)
-                want += g.missing(slot, self.lengths[slot] + n_new)
-            if want > g.pool.n_free:
-                raise CacheFull("step needs %d more pages of %d positions, %d free of %d"
-                                % (want, PAGE, g.pool.n_free, g.pool.n))
-        for g in self.kv_groups:
-            for slot, n_new in items:
-                g.extend(slot, self.lengths[slot] + n_new)
+        self.native.reserve(items)
 
     def commit(self, items):
         """The step has been launched: lengths grow, windows let go of old pages."""
-        for slot, n_new in items:
-            self.lengths[slot] += n_new
-            for g in self.kv_groups:
-                g.trim(slot, self.lengths[slot])
+        self.native.commit(items)
 
     def page_table(self, group, slots):
         """[len(slots), width] int32 of page ids (-1: none) for the sequences of a step."""
-        width = max(1, max(len(group.pages.get(s, ())) for s in slots))     # (a group exists only with pages)
+        lists = [group.pages.get(s, ()) for s in slots]
+        width = max(1, max(len(have) for have in lists))
         table = np.full((len(slots), width), -1, dtype=np.int32)
-        for i, s in enumerate(slots):
-            have = group.pages.get(s, ())
+        for i, have in enumerate(lists):
             table[i, :len(have)] = have
         return table
 
@@ -222,17 +248,8 @@ class Cache:
     # -- checks -----------------------------------------------------------
     def tokens_held(self):
         """Positions held by live sequences, each counted up to a multiple of PAGE."""
-        return sum(pages_for(self.lengths[s]) * PAGE for s in range(self.max_slots) if self.slots.is_held(s))
+        return sum(pages_for(self.native.length(s)) * PAGE for s in range(self.max_slots) if self.native.is_held(s))
 
     def check(self):
-        self.slots.check()
-        for g in self.kv_groups:
-            g.pool.check()
-            held = [p for have in g.pages.values() for p in have if p >= 0]
-            if len(held) != len(set(held)):
-                raise AssertionError("a page is held by two sequences")
-            if len(held) != g.pool.n_held:
-                raise AssertionError("%d pages held by sequences, pool says %d" % (len(held), g.pool.n_held))
-            for slot in g.pages:
-                if not self.slots.is_held(slot):
-                    raise AssertionError("free slot %d still holds pages" % slot)
+        """Nothing lost, held twice or freed twice (AssertionError with the finding)."""
+        self.native.check()

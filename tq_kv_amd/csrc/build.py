@@ -20,6 +20,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["host.cpp", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip",
            "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip", "random_init.hip"]
 HEADERS = ["common.h", "tq_kernels.h"]
+# the engine's host side: no GPU code, built with the host compiler into a library of its own
+HOST_SOURCES = ["host_engine.cpp"]
+HOST_HEADERS = ["tq_engine.h"]
+HOST_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-shared", "-Wall"]
 ARCH = "gfx950"
 # Packed float32 instructions are switched off for all device code.
 HIPCC_FLAGS = ["-O3", "-fPIC", "-std=c++17", "--offload-arch=" + ARCH,
@@ -52,6 +56,20 @@ def library_name():
     return "libtqkernels_%s.so" % source_hash()
 
 
+def host_source_hash():
+    h = hashlib.sha256()
+    for name in sorted(HOST_SOURCES + HOST_HEADERS):
+        with open(os.path.join(HERE, name), "rb") as f:
+            h.update(name.encode())
+            h.update(f.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return h.hexdigest()[:12]
+
+
+def host_library_name():
+    return "libtqengine_%s.so" % host_source_hash()
+
+
 def _writable(folder):
     try:
         os.makedirs(folder, exist_ok=True)
@@ -74,6 +92,52 @@ def find_library():
         if os.path.exists(path):
             return path
     return None
+
+
+def find_host_library():
+    name = host_library_name()
+    for folder in (HERE, _fallback_dir()):
+        path = os.path.join(folder, name)
+        if os.path.exists(path):
+            return path
+    return None
+
+
+def _host_compiler():
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"), "/opt/rocm/llvm/bin/clang++"):
+        if cand and (os.path.exists(cand) or shutil.which(cand)):
+            return cand
+    raise BuildError("no C++ compiler found for the engine's host library (looked in $CXX, g++, c++, clang++)")
+
+
+def build_host(force=True, verbose=True):
+    """Compile the engine's host library (seconds; needs no GPU toolchain).  Returns its path."""
+    existing = find_host_library()
+    if existing and not force:
+        return existing
+    out_dir = HERE if _writable(HERE) else _fallback_dir()
+    if not _writable(out_dir):
+        raise BuildError("cannot write the engine library to %s or %s" % (HERE, out_dir))
+    target = os.path.join(out_dir, host_library_name())
+    tmp = target + ".tmp%d" % os.getpid()
+    cmd = [_host_compiler()] + HOST_FLAGS + ["-I", HERE] + [os.path.join(HERE, n) for n in HOST_SOURCES] + ["-o", tmp]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise BuildError("the host compiler failed on %s:\n%s" % (", ".join(HOST_SOURCES), proc.stdout))
+    os.replace(tmp, target)
+    for name in os.listdir(out_dir):
+        if name.startswith("libtqengine_") and name.endswith(".so") and name != os.path.basename(target):
+            try:
+                os.remove(os.path.join(out_dir, name))
+            except OSError:
+                pass
+    if verbose:
+        print("[tq_kv_amd build] built %s" % target, file=sys.stderr, flush=True)
+    return target
+
+
+def ensure_host_built(verbose=False):
+    return find_host_library() or build_host(force=True, verbose=verbose)
 
 
 def _run_with_heartbeat(cmd, what, log):
@@ -103,6 +167,7 @@ def build(force=True, verbose=True):
     existing = find_library()
     if existing and not force:
         return existing
+    build_host(force=force, verbose=verbose)
     hipcc = _hipcc()
     out_dir = HERE if _writable(HERE) else _fallback_dir()
     if not _writable(out_dir):

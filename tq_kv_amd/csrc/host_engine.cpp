@@ -1,0 +1,369 @@
+// The engine's bookkeeping on the host, behind a C boundary in the manner of the
+// reference's (tq-kv/include/tq_kv.h:27-84, tq-kv/src/ffi.rs:89-108): opaque handles made
+// and freed by the library, plain C types, int32 status (0 ok, negative error) and a
+// message for the last error.  No GPU code here: this file is compiled with the host
+// compiler alone and works on a machine without a GPU.
+//
+// tqe_cache_t owns what the cache must never lose: which slots are free, how many
+// positions every sequence holds, and for every group of cached runs which pages of the
+// group's pool each slot holds (a group with a window gives pages back as soon as all
+// their positions have left the window).  The storage itself (the tensors of keys,
+// values and states) belongs to the caller and is indexed by the slot and page numbers
+// handed out here.
+//
+// tqe_plan_step turns one step's batch (sequences that bring unequal numbers of new
+// tokens) into the packed int32 array that the kernels read: tokens, per-token sequence
+// and position, per-sequence slot, start, count and offsets, the wanted rows, the rows the
+// last run has to compute, and one page table per group for the step's sequences.
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <algorithm>
+#include <new>
+#include <vector>
+
+#include "tq_engine.h"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+// A pool of n numbered things, each free or held; hands out the lowest numbers first and
+// reuses what came back last.
+struct Pool {
+    std::vector<int32_t> free;
+    std::vector<uint8_t> held;
+    int n = 0;
+    void init(int count) {
+        n = count;
+        free.resize(count);
+        for (int i = 0; i < count; ++i) free[i] = count - 1 - i;
+        held.assign(count, 0);
+    }
+    int n_free() const { return (int)free.size(); }
+    int take() {
+        const int i = free.back();
+        free.pop_back();
+        held[i] = 1;
+        return i;
+    }
+    bool give_back(int i) {
+        if (i < 0 || i >= n || !held[i]) return false;
+        held[i] = 0;
+        free.push_back(i);
+        return true;
+    }
+    // every item is on the free list once or held, never both
+    bool consistent(const char* what, char* msg, size_t cap) const {
+        std::vector<uint8_t> seen(n, 0);
+        for (int i : free) {
+            if (i < 0 || i >= n || seen[i]) { snprintf(msg, cap, "%s %d is on the free list twice", what, i); return false; }
+            seen[i] = 1;
+            if (held[i]) { snprintf(msg, cap, "%s %d is both free and held", what, i); return false; }
+        }
+        for (int i = 0; i < n; ++i)
+            if (!seen[i] && !held[i]) { snprintf(msg, cap, "%s %d is lost", what, i); return false; }
+        return true;
+    }
+};
+
+struct Group {
+    Pool pool;
+    int window = 0;                                   // 0: every position stays
+    std::vector<std::vector<int32_t>> pages;          // per slot: page of positions 64 i .. , -1 where given back
+    std::vector<uint8_t> known;                       // per slot: whether the slot has a list at all
+};
+
+int pages_for(long long positions) { return (int)((positions + TQE_PAGE - 1) / TQE_PAGE); }
+
+}  // namespace
+
+struct tqe_cache {
+    int max_slots = 0;
+    Pool slots;
+    std::vector<int32_t> lengths;
+    std::vector<Group> groups;
+};
+
+extern "C" {
+
+const char* tqe_last_error(void) { return g_error; }
+int tqe_abi_version(void) { return 1; }
+
+tqe_cache_t* tqe_cache_new(int max_slots, int n_groups, const int32_t* pages_per_group, const int32_t* window_per_group) {
+    if (max_slots < 1 || n_groups < 0 || n_groups > TQE_MAX_GROUPS || (n_groups > 0 && (!pages_per_group || !window_per_group))) {
+        fail(TQE_ERR_ARGUMENT, "tqe_cache_new: bad arguments (slots %d, groups %d)", max_slots, n_groups);
+        return nullptr;
+    }
+    tqe_cache_t* c = new (std::nothrow) tqe_cache();
+    if (!c) { fail(TQE_ERR_ARGUMENT, "tqe_cache_new: out of memory"); return nullptr; }
+    c->max_slots = max_slots;
+    c->slots.init(max_slots);
+    c->lengths.assign(max_slots, 0);
+    c->groups.resize(n_groups);
+    for (int g = 0; g < n_groups; ++g) {
+        if (pages_per_group[g] < 0 || window_per_group[g] < 0) {
+            fail(TQE_ERR_ARGUMENT, "tqe_cache_new: group %d with %d pages and window %d", g, pages_per_group[g], window_per_group[g]);
+            delete c;
+            return nullptr;
+        }
+        c->groups[g].pool.init(pages_per_group[g]);
+        c->groups[g].window = window_per_group[g];
+        c->groups[g].pages.resize(max_slots);
+        c->groups[g].known.assign(max_slots, 0);
+    }
+    return c;
+}
+
+void tqe_cache_free(tqe_cache_t* c) { delete c; }
+
+int tqe_cache_acquire(tqe_cache_t* c, int32_t* slot_out) {
+    if (!c || !slot_out) return fail(TQE_ERR_ARGUMENT, "tqe_cache_acquire: null pointer");
+    if (c->slots.n_free() < 1) return fail(TQE_ERR_FULL, "need 1 slot(s), 0 free of %d", c->max_slots);
+    const int s = c->slots.take();
+    c->lengths[s] = 0;
+    *slot_out = s;
+    return TQE_OK;
+}
+
+int tqe_cache_release(tqe_cache_t* c, int slot) {
+    if (!c) return fail(TQE_ERR_ARGUMENT, "tqe_cache_release: null pointer");
+    if (!c->slots.give_back(slot)) return fail(TQE_ERR_STATE, "slot %d given back but not held", slot);
+    for (Group& g : c->groups) {
+        for (int32_t p : g.pages[slot])
+            if (p >= 0) g.pool.give_back(p);
+        g.pages[slot].clear();
+        g.known[slot] = 0;
+    }
+    c->lengths[slot] = 0;
+    return TQE_OK;
+}
+
+int tqe_cache_length(const tqe_cache_t* c, int slot) {
+    if (!c || slot < 0 || slot >= c->max_slots) return fail(TQE_ERR_ARGUMENT, "tqe_cache_length: no slot %d", slot);
+    return c->lengths[slot];
+}
+
+int tqe_cache_is_held(const tqe_cache_t* c, int slot) {
+    return c && slot >= 0 && slot < c->max_slots && c->slots.held[slot];
+}
+
+int tqe_cache_counts(const tqe_cache_t* c, int group, int32_t* n_free, int32_t* n_total) {
+    if (!c || group < -1 || group >= (int)c->groups.size()) return fail(TQE_ERR_ARGUMENT, "tqe_cache_counts: no group %d", group);
+    const Pool& p = group < 0 ? c->slots : c->groups[group].pool;
+    if (n_free) *n_free = p.n_free();
+    if (n_total) *n_total = p.n;
+    return TQE_OK;
+}
+
+int tqe_cache_reserve(tqe_cache_t* c, int n, const int32_t* slots, const int32_t* n_new) {
+    if (!c || (n > 0 && (!slots || !n_new))) return fail(TQE_ERR_ARGUMENT, "tqe_cache_reserve: null pointer");
+    for (int i = 0; i < n; ++i)
+        if (slots[i] < 0 || slots[i] >= c->max_slots || !c->slots.held[slots[i]]) return fail(TQE_ERR_STATE, "slot %d is not held", slots[i]);
+    for (const Group& g : c->groups) {
+        long long want = 0;
+        for (int i = 0; i < n; ++i) {
+            const int need = pages_for((long long)c->lengths[slots[i]] + n_new[i]) - (int)g.pages[slots[i]].size();
+            if (need > 0) want += need;
+        }
+        if (want > g.pool.n_free())
+            return fail(TQE_ERR_FULL, "step needs %lld more pages of %d positions, %d free of %d", want, TQE_PAGE, g.pool.n_free(), g.pool.n);
+    }
+    for (Group& g : c->groups)
+        for (int i = 0; i < n; ++i) {
+            std::vector<int32_t>& have = g.pages[slots[i]];
+            const int need = pages_for((long long)c->lengths[slots[i]] + n_new[i]);
+            g.known[slots[i]] = 1;
+            while ((int)have.size() < need) have.push_back(g.pool.take());
+        }
+    return TQE_OK;
+}
+
+int tqe_cache_commit(tqe_cache_t* c, int n, const int32_t* slots, const int32_t* n_new) {
+    if (!c || (n > 0 && (!slots || !n_new))) return fail(TQE_ERR_ARGUMENT, "tqe_cache_commit: null pointer");
+    for (int i = 0; i < n; ++i) {
+        const int s = slots[i];
+        if (s < 0 || s >= c->max_slots || !c->slots.held[s]) return fail(TQE_ERR_STATE, "slot %d is not held", s);
+        c->lengths[s] += n_new[i];
+        for (Group& g : c->groups) {
+            if (g.window <= 0) continue;
+            // pages whose positions are all out of the window of the next query go back
+            std::vector<int32_t>& have = g.pages[s];
+            const int first_needed = std::max(0, c->lengths[s] + 1 - g.window);
+            const int dead = std::min(first_needed / TQE_PAGE, (int)have.size());
+            for (int k = 0; k < dead; ++k)
+                if (have[k] >= 0) { g.pool.give_back(have[k]); have[k] = -1; }
+        }
+    }
+    return TQE_OK;
+}
+
+int tqe_cache_pages(const tqe_cache_t* c, int group, int slot, int32_t* out, int cap) {
+    if (!c || group < 0 || group >= (int)c->groups.size() || slot < 0 || slot >= c->max_slots)
+        return fail(TQE_ERR_ARGUMENT, "tqe_cache_pages: no group %d or slot %d", group, slot);
+    const Group& g = c->groups[group];
+    if (!g.known[slot]) return TQE_NO_LIST;                    // (distinct from an empty list)
+    const std::vector<int32_t>& have = g.pages[slot];
+    if (out)
+        for (int i = 0; i < (int)have.size() && i < cap; ++i) out[i] = have[i];
+    return (int)have.size();
+}
+
+int tqe_cache_check(const tqe_cache_t* c) {
+    if (!c) return fail(TQE_ERR_ARGUMENT, "tqe_cache_check: null pointer");
+    char msg[256];
+    if (!c->slots.consistent("slot", msg, sizeof(msg))) return fail(TQE_ERR_STATE, "%s", msg);
+    for (const Group& g : c->groups) {
+        if (!g.pool.consistent("page", msg, sizeof(msg))) return fail(TQE_ERR_STATE, "%s", msg);
+        std::vector<uint8_t> seen(g.pool.n, 0);
+        int held = 0;
+        for (int s = 0; s < c->max_slots; ++s) {
+            if (!g.pages[s].empty() && !c->slots.held[s]) return fail(TQE_ERR_STATE, "free slot %d still holds pages", s);
+            for (int32_t p : g.pages[s]) {
+                if (p < 0) continue;
+                if (p >= g.pool.n || seen[p]) return fail(TQE_ERR_STATE, "a page is held by two sequences");
+                seen[p] = 1;
+                ++held;
+            }
+        }
+        if (held != g.pool.n - g.pool.n_free())
+            return fail(TQE_ERR_STATE, "%d pages held by sequences, pool says %d", held, g.pool.n - g.pool.n_free());
+    }
+    return TQE_OK;
+}
+
+// ---- the step's arrays ------------------------------------------------------------------------
+int tqe_plan_step(const tqe_cache_t* c, int n_seqs, const int32_t* slots, const int32_t* starts, const int32_t* n_new,
+                  const int32_t* tokens, const int32_t* want_counts, const int32_t* want_idx, int width_step,
+                  int32_t* out, int out_cap, int32_t* meta) {
+    if (n_seqs < 1 || !slots || !n_new || !want_counts || !meta) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: bad arguments");
+    if (!c && !starts) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: without a cache the sequences' starts must be given");
+    const int n_groups = c ? (int)c->groups.size() : 0;
+    long long n_tokens = 0, n_want = 0;
+    int max_new = 0;
+    bool all_decode = true;
+    for (int i = 0; i < n_seqs; ++i) {
+        if (n_new[i] < 1) return fail(TQE_ERR_ARGUMENT, "sequence %d of the step brings no token", i);
+        if (c && (slots[i] < 0 || slots[i] >= c->max_slots)) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: no slot %d", slots[i]);
+        n_tokens += n_new[i];
+        n_want += want_counts[i];
+        max_new = std::max(max_new, n_new[i]);
+        all_decode = all_decode && n_new[i] == 1;
+    }
+    if (n_tokens > 0x3fffffff) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: %lld tokens in one step", n_tokens);
+    if (n_want > 0 && !want_idx) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: wanted places without their list");
+    // the wanted rows, and those of them the last run computes: each once, in order
+    std::vector<int32_t> cu(n_seqs + 1, 0), want_rows((size_t)n_want);
+    for (int i = 0; i < n_seqs; ++i) cu[i + 1] = cu[i] + n_new[i];
+    {
+        size_t k = 0;
+        for (int i = 0; i < n_seqs; ++i)
+            for (int j = 0; j < want_counts[i]; ++j, ++k) {
+                const int at = want_idx[k];
+                if (at < 0 || at >= n_new[i])
+                    return fail(TQE_ERR_RANGE, "wanted place %d is outside the %d tokens of sequence %d", at, n_new[i], i);
+                want_rows[k] = cu[i] + at;
+            }
+    }
+    std::vector<int32_t> last_rows(want_rows);
+    std::sort(last_rows.begin(), last_rows.end());
+    last_rows.erase(std::unique(last_rows.begin(), last_rows.end()), last_rows.end());
+    const int n_last = (int)last_rows.size();
+    const bool prune_last = !all_decode && n_last < n_tokens;
+    const int n_last_kept = prune_last ? n_last : 0;
+    // page table widths
+    std::vector<int> width(n_groups, 1);
+    for (int g = 0; g < n_groups; ++g) {
+        int wmax = 1;
+        for (int i = 0; i < n_seqs; ++i) wmax = std::max(wmax, (int)c->groups[g].pages[slots[i]].size());
+        if (width_step > 1) wmax = (wmax + width_step - 1) / width_step * width_step;
+        width[g] = wmax;
+    }
+    // layout: every array starts at a multiple of 4 values
+    const long long sizes[12] = {n_tokens, n_tokens, n_tokens, n_seqs, n_seqs, n_seqs, n_seqs + 1, n_want,
+                                 n_last_kept, prune_last ? n_want : 0, n_last_kept, n_last_kept};
+    long long total = 0;
+    int32_t* offsets = meta + TQE_META_OFFSETS;
+    for (int a = 0; a < 12; ++a) {
+        offsets[a] = (int32_t)total;
+        total += (sizes[a] + 3) / 4 * 4;
+    }
+    for (int g = 0; g < n_groups; ++g) {
+        offsets[12 + g] = (int32_t)total;
+        total += ((long long)n_seqs * width[g] + 3) / 4 * 4;
+    }
+    if (total < 4) total = 4;
+    if (total > 0x7fffffff) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: the step's arrays are too large");
+    int max_end = 0;
+    for (int i = 0; i < n_seqs; ++i) max_end = std::max(max_end, (starts ? starts[i] : c->lengths[slots[i]]) + n_new[i]);
+    meta[TQE_META_TOTAL] = (int32_t)total;
+    meta[TQE_META_TOKENS] = (int32_t)n_tokens;
+    meta[TQE_META_WANT] = (int32_t)n_want;
+    meta[TQE_META_LAST] = n_last;
+    meta[TQE_META_ALL_DECODE] = all_decode ? 1 : 0;
+    meta[TQE_META_PRUNE_LAST] = prune_last ? 1 : 0;
+    meta[TQE_META_MAX_NEW] = max_new;
+    meta[TQE_META_MAX_END] = max_end;
+    meta[TQE_META_GROUPS] = n_groups;
+    for (int g = 0; g < n_groups; ++g) meta[TQE_META_OFFSETS + 12 + TQE_MAX_GROUPS + g] = width[g];
+    if (!out) return TQE_OK;                                   // sizes only
+    if (out_cap < total) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: %lld values do not fit the %d given", total, out_cap);
+    if (!tokens) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: no tokens");
+    memset(out, 0, sizeof(int32_t) * (size_t)total);
+    int32_t* o_tokens = out + offsets[0];
+    int32_t* o_tok_seq = out + offsets[1];
+    int32_t* o_tok_pos = out + offsets[2];
+    int32_t* o_slot = out + offsets[3];
+    int32_t* o_start = out + offsets[4];
+    int32_t* o_new = out + offsets[5];
+    int32_t* o_cu = out + offsets[6];
+    int32_t* o_want = out + offsets[7];
+    memcpy(o_tokens, tokens, sizeof(int32_t) * (size_t)n_tokens);
+    for (int i = 0; i < n_seqs; ++i) {
+        const int start = starts ? starts[i] : c->lengths[slots[i]];
+        o_slot[i] = slots[i];
+        o_start[i] = start;
+        o_new[i] = n_new[i];
+        o_cu[i] = cu[i];
+        for (int t = 0; t < n_new[i]; ++t) {
+            o_tok_seq[cu[i] + t] = i;
+            o_tok_pos[cu[i] + t] = start + t;
+        }
+    }
+    o_cu[n_seqs] = cu[n_seqs];
+    for (long long k = 0; k < n_want; ++k) o_want[k] = want_rows[(size_t)k];
+    if (prune_last) {
+        int32_t* o_last = out + offsets[8];
+        int32_t* o_in_last = out + offsets[9];
+        int32_t* o_last_seq = out + offsets[10];
+        int32_t* o_last_pos = out + offsets[11];
+        for (int k = 0; k < n_last; ++k) {
+            o_last[k] = last_rows[k];
+            o_last_seq[k] = o_tok_seq[last_rows[k]];
+            o_last_pos[k] = o_tok_pos[last_rows[k]];
+        }
+        for (long long k = 0; k < n_want; ++k)
+            o_in_last[k] = (int32_t)(std::lower_bound(last_rows.begin(), last_rows.end(), want_rows[(size_t)k]) - last_rows.begin());
+    }
+    for (int g = 0; g < n_groups; ++g) {
+        int32_t* table = out + offsets[12 + g];
+        for (long long k = 0; k < (long long)n_seqs * width[g]; ++k) table[k] = -1;
+        for (int i = 0; i < n_seqs; ++i) {
+            const std::vector<int32_t>& have = c->groups[g].pages[slots[i]];
+            for (size_t k = 0; k < have.size(); ++k) table[(size_t)i * width[g] + k] = have[k];
+        }
+    }
+    return TQE_OK;
+}
+
+}  // extern "C"

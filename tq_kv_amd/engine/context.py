@@ -10,6 +10,8 @@ host as one int32 array and uploaded in one copy.
 import numpy as np
 import torch
 
+from .. import native
+
 
 class _Arrays:
     pass
@@ -50,72 +52,59 @@ class HostStaging:
         return dev
 
 
+_NAMES = ["tokens", "tok_seq", "tok_pos", "seq_slot", "seq_start", "seq_new", "cu", "want_rows",
+          "last_rows", "want_in_last", "last_seq", "last_pos"]
+
+
 class StepContext:
     """items: [(slot, start, tokens)] with `start` the sequence's length before the step;
-    want: for each item the indices among its tokens whose logits are wanted."""
+    want: for each item the indices among its tokens whose logits are wanted.
+
+    The arrays are laid out by the engine's host library (tqe_plan_step): the wanted rows, the
+    rows that the last run of the order has to compute (the wanted ones, each once, in order:
+    where these are fewer than the step's tokens, a prompt of which the last place is wanted or a
+    piece of a prompt of which nothing is, the last run computes its queries, its output product
+    and its feed-forward for them alone), and the page tables of the step's sequences."""
 
     def __init__(self, items, want, cache, device, staging=None, width_step=1, into=None):
         self.n_seqs = len(items)
         lens = [len(toks) for _, _, toks in items]
-        self.n_tokens = int(sum(lens))
-        host = _Arrays()
-        host.tokens = np.concatenate([np.asarray(toks, dtype=np.int64) for _, _, toks in items]).astype(np.int32)
-        host.seq_slot = np.asarray([slot for slot, _, _ in items], dtype=np.int32)
-        host.seq_start = np.asarray([start for _, start, _ in items], dtype=np.int32)
-        host.seq_new = np.asarray(lens, dtype=np.int32)
-        host.cu = np.zeros(self.n_seqs + 1, dtype=np.int32)
-        np.cumsum(host.seq_new, out=host.cu[1:])
-        host.tok_seq = np.repeat(np.arange(self.n_seqs, dtype=np.int32), host.seq_new)
-        host.tok_pos = (np.arange(self.n_tokens, dtype=np.int32) - np.repeat(host.cu[:-1], host.seq_new)
-                        + np.repeat(host.seq_start, host.seq_new)).astype(np.int32)
-        rows = []
-        for i, w in enumerate(want):
-            for j in w:
-                if not 0 <= j < lens[i]:
-                    raise IndexError("wanted place %d is outside the %d tokens of sequence %d" % (j, lens[i], i))
-                rows.append(int(host.cu[i]) + int(j))
-        host.want_rows = np.asarray(rows, dtype=np.int32)
-        # The rows that the last run of the order has to compute: the wanted ones, each once, in
-        # order.  Where these are fewer than the step's tokens (a prompt of which the last place is
-        # wanted, a piece of a prompt of which nothing is), the last run computes its queries,
-        # its output product and its feed-forward for them alone.
-        host.last_rows = np.unique(host.want_rows).astype(np.int32)
-        host.want_in_last = np.searchsorted(host.last_rows, host.want_rows).astype(np.int32)
-        self.n_last = int(host.last_rows.shape[0])
-        self.all_decode = all(n == 1 for n in lens)
-        self.prune_last = not self.all_decode and self.n_last < self.n_tokens
-        if self.prune_last:
-            host.last_seq, host.last_pos = host.tok_seq[host.last_rows], host.tok_pos[host.last_rows]
+        slots = np.asarray([slot for slot, _, _ in items], dtype=np.int32)
+        starts = np.asarray([start for _, start, _ in items], dtype=np.int32)
+        n_new = np.asarray(lens, dtype=np.int32)
+        if len(items) == 1:
+            tokens = np.asarray(items[0][2], dtype=np.int64).astype(np.int32)
         else:
-            host.last_rows = host.want_in_last = host.last_seq = host.last_pos = np.zeros(0, dtype=np.int32)
+            tokens = np.concatenate([np.asarray(toks, dtype=np.int64) for _, _, toks in items]).astype(np.int32)
+        want_counts = np.asarray([len(w) for w in want], dtype=np.int32)
+        want_idx = np.asarray([j for w in want for j in w], dtype=np.int64).astype(np.int32)
+        self.groups = list(cache.kv_groups) if cache is not None else []
+        packed, meta = native.plan_step(cache.native if cache is not None else None, slots, starts, n_new, tokens,
+                                        want_counts, want_idx, width_step)
+        self.packed = packed
+        self.n_tokens = int(meta[native.META_TOKENS])
+        self.n_last = int(meta[native.META_LAST])
+        self.all_decode = bool(meta[native.META_ALL_DECODE])
+        self.prune_last = bool(meta[native.META_PRUNE_LAST])
+        self.max_new = int(meta[native.META_MAX_NEW])
+        self.max_end = int(meta[native.META_MAX_END])
+        offsets = [int(o) for o in meta[native.META_OFFSETS:native.META_OFFSETS + 12 + len(self.groups)]]
+        widths = [int(x) for x in meta[native.META_WIDTHS:native.META_WIDTHS + len(self.groups)]]
+        n_want = int(meta[native.META_WANT])
+        kept = self.n_last if self.prune_last else 0
+        sizes = [self.n_tokens] * 3 + [self.n_seqs] * 3 + [self.n_seqs + 1, n_want, kept, n_want if self.prune_last else 0, kept, kept]
+        self._table_shapes = [(self.n_seqs, w) for w in widths]
+
+        def carve(flat, make=lambda x: x):
+            out = _Arrays()
+            for name, off, size in zip(_NAMES, offsets, sizes):
+                setattr(out, name, make(flat[off:off + size]))
+            return out
+        self.host = carve(packed)
+        self.host_tables = [packed[off:off + n * w].reshape(n, w) for off, (n, w) in zip(offsets[12:], self._table_shapes)]
         self._lens = lens
         self._tiles = {}              # (which rows, queries per tile) -> device arrays, built when a mixer asks
-        self.host = host
-        self.fuse_small = False      # set by the model for small decoding steps in bfloat16
-        self.max_new = max(lens)
-        self.max_end = int((host.seq_start + host.seq_new).max())
-        self.groups = list(cache.kv_groups) if cache is not None else []
-        slots = [slot for slot, _, _ in items]
-        self.host_tables = [cache.page_table(g, slots) for g in self.groups]
-        if width_step > 1:
-            # widths in steps, so that a captured graph serves until a sequence outgrows them
-            for i, t in enumerate(self.host_tables):
-                width = (t.shape[1] + width_step - 1) // width_step * width_step
-                wide = np.full((t.shape[0], width), -1, dtype=np.int32)
-                wide[:, :t.shape[1]] = t
-                self.host_tables[i] = wide
-
-        names = ["tokens", "tok_seq", "tok_pos", "seq_slot", "seq_start", "seq_new", "cu", "want_rows",
-                 "last_rows", "want_in_last", "last_seq", "last_pos"]
-        parts = [getattr(host, n) for n in names] + [t.reshape(-1) for t in self.host_tables]
-        offsets, total = [], 0
-        for p in parts:
-            offsets.append(total)
-            total += (p.shape[0] + 3) // 4 * 4
-        packed = np.zeros(max(total, 4), dtype=np.int32)
-        for off, p in zip(offsets, parts):
-            packed[off:off + p.shape[0]] = p
-        self.packed = packed
+        self.fuse_small = False       # set by the model for small decoding steps in bfloat16
         self._device, self._staging = device, staging
         if into is not None and not isinstance(into, torch.Tensor):
             return                                   # host arrays only
@@ -126,13 +115,10 @@ class StepContext:
         else:
             flat = torch.from_numpy(packed).to(device)
         self.flat = flat
-        dev = _Arrays()
-        for name, off, p in zip(names, offsets, parts):
-            setattr(dev, name, flat[off:off + p.shape[0]])
-        self.dev = dev
+        self.dev = carve(flat)
         self._tables = {}
-        for g, off, t in zip(self.groups, offsets[len(names):], self.host_tables):
-            self._tables[id(g)] = flat[off:off + t.size].view(t.shape)
+        for g, off, (n, w) in zip(self.groups, offsets[12:], self._table_shapes):
+            self._tables[id(g)] = flat[off:off + n * w].view(n, w)
 
     # -- tiles of consecutive queries, for mixers that work on them -----------------------------
     def _upload_tiles(self, key, seq, tok0, count, order_key):
@@ -183,7 +169,7 @@ class StepContext:
     def shape_key(self):
         """What fixes the layout of the device arrays (and so what a captured graph of the
         step depends on): numbers of tokens, sequences and wanted rows, table widths."""
-        return (self.n_tokens, self.n_seqs, int(self.host.want_rows.shape[0]), tuple(t.shape[1] for t in self.host_tables))
+        return (self.n_tokens, self.n_seqs, int(self.host.want_rows.shape[0]), tuple(w for _, w in self._table_shapes))
 
     def page_table(self, group):
         """[sequences of the step, width] int32 page ids of a cache group, on the device."""
