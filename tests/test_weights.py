@@ -71,6 +71,16 @@ def test_tied_model_refuses_a_head_and_untied_needs_one(tmp_path):
     model = Model.from_config_dict(TINY_A, "float32", "cpu")
     with pytest.raises(WeightError, match="Unexpected tensor: lm_head.weight"):
         load_folder(folder, model.tensor_specs(), torch.float32, "cpu")
+    # on request the tensors a model does not use are named in a warning instead (the reference never looks them up);
+    # what is missing or misshapen stays an error
+    with pytest.warns(UserWarning, match="lm_head.weight"):
+        got = Model.from_dir(folder, dtype="float32", device="cpu", strict=False)
+    assert got.head is got.embedding
+    del t["model.norm.weight"]
+    save_file(t, path)
+    with pytest.raises(WeightError, match="Missing tensor: model.norm.weight") as e:
+        Model.from_dir(folder, dtype="float32", device="cpu", strict=False)
+    assert "Unexpected" not in str(e.value)
 
 
 def test_dtype_policy(tmp_path):

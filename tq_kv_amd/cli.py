@@ -40,6 +40,8 @@ def _add_model(p):
     p.add_argument("model", help="Model folder, or name of a shape to run with random weights (see `tq list`)")
     p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     p.add_argument("--weights-seed", type=int, default=0, help="Seed of the random weights of a shape")
+    p.add_argument("--allow-extra-tensors", action="store_true",
+                   help="Tensors in the folder that the model does not use are a warning, not an error")
     p.add_argument("--max-cache-tokens", type=int, default=0,
                    help="Positions the cache holds for all live requests together (0: what the prompts need)")
 
@@ -79,11 +81,11 @@ def build_parser():
     return ap
 
 
-def load_model(name, dtype, weights_seed):
+def load_model(name, dtype, weights_seed, strict=True):
     from .config import catalog
     from .engine import Model
     if os.path.isdir(name):
-        return Model.from_dir(name, dtype=dtype)
+        return Model.from_dir(name, dtype=dtype, strict=strict)
     if catalog.find(name) is None:
         raise SystemExit("Model '%s' not found: no such folder and no such shape. Available shapes: %s"
                          % (name, ", ".join("%s:%s" % e for e in catalog.entries())))
@@ -115,7 +117,7 @@ def cmd_generate(args):
             prompts.append(tokenizer.encode(text, add_special_tokens=False).ids)       # as src/engine.rs:342-345
     if not prompts:
         raise SystemExit("no prompt: give --prompt-ids, --prompt-file or --prompt")
-    model = load_model(args.model, args.dtype, args.weights_seed)
+    model = load_model(args.model, args.dtype, args.weights_seed, strict=not args.allow_extra_tensors)
     params = GenerationParams(max_tokens=args.max_tokens, temperature=args.temperature, top_p=args.top_p,
                               top_k=args.top_k, repeat_penalty=args.repeat_penalty, seed=args.seed)
     eos = _ids(args.eos) if args.eos is not None else list(model.stop_token_ids)

@@ -106,11 +106,12 @@ class Model:
         return cls(spec_for(name, config), dtype, device, config=config)
 
     @classmethod
-    def from_dir(cls, model_dir, dtype="bfloat16", device="cuda"):
-        """A model folder: config.json picks the architecture, *.safetensors hold the weights."""
+    def from_dir(cls, model_dir, dtype="bfloat16", device="cuda", strict=True):
+        """A model folder: config.json picks the architecture, *.safetensors hold the weights.
+        strict=False: tensors the model does not use are a warning, not an error."""
         model = cls.from_config_dict(read_config_json(model_dir), dtype, device)
         model.stop_token_ids = stop_token_ids(model_dir, model.spec.eos_token_ids)
-        return model.load(load_folder(model_dir, model.tensor_specs(), model.dtype, model.device))
+        return model.load(load_folder(model_dir, model.tensor_specs(), model.dtype, model.device, strict))
 
     @classmethod
     def random(cls, shape, seed=0, dtype="bfloat16", device="cuda"):

@@ -44,11 +44,18 @@ def target_dtype(stored, kind, run_dtype):
     return run_dtype
 
 
-def check(stored, wanted):
+def check(stored, wanted, strict=True):
     """stored: name -> object with .shape and .dtype; wanted: name -> TensorSpec.
-    Raises WeightError unless names and shapes agree exactly."""
+    Raises WeightError unless names and shapes agree exactly.  strict=False: tensors the model
+    does not ask for (a tied checkpoint that still ships its head, rotary tables of an older
+    export) are named in a warning instead, as the reference simply never looks them up
+    (src/models/turbo_generic.rs:2056-2066)."""
     missing = [n for n in wanted if n not in stored]
     unexpected = sorted(n for n in stored if n not in wanted)
+    if unexpected and not strict:
+        import warnings
+        warnings.warn("the folder holds %d tensors the model does not use: %s" % (len(unexpected), ", ".join(unexpected)))
+        unexpected = []
     wrong_shape, wrong_kind = [], []
     for n, spec in wanted.items():
         if n not in stored:
@@ -62,10 +69,10 @@ def check(stored, wanted):
         raise WeightError(missing, unexpected, wrong_shape, wrong_kind)
 
 
-def load_folder(model_dir, wanted, run_dtype, device):
+def load_folder(model_dir, wanted, run_dtype, device, strict=True):
     """name -> tensor on `device` for every wanted name, after the check."""
     stored = open_folder(model_dir)
-    check(stored, wanted)
+    check(stored, wanted, strict)
     out = {}
     for name, spec in wanted.items():
         st = stored[name]
