@@ -70,6 +70,9 @@ def main():
     H, I, V = raw["hidden_size"], raw["intermediate_size"], raw["vocab_size"]
     nh, nkv, d = raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"]
     ctx_len = raw["max_position_embeddings"]
+    needed = args.prompt_len + args.steps + args.warmup + 2
+    if needed > ctx_len:             # other contexts than the shape's own: the position tables grow with them
+        ctx_len = raw["max_position_embeddings"] = (needed + 1023) // 1024 * 1024
     note("making random weights for %s (%d layers)" % (args.shape, layers))
     model = Model.random(raw, seed=0, dtype="bfloat16", device="cuda:0")
     max_batch = 64 if not args.no_points else args.batch
