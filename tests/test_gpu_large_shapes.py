@@ -35,7 +35,7 @@ def tensors_for(raw, seed):
 @pytest.mark.parametrize("shape", ["qwen2.5:7b", "qwen2.5:1.5b", "qwen2.5:32b"])
 def test_bfloat16_tracks_float32_at_large_sizes(shape):
     raw = two_layer(shape)
-    tensors = tensors_for(raw, 3)
+    tensors = sharpened(tensors_for(raw, 3))
     lens = [300, 70, 1]
     prompts = [helpers.random_tokens(n, raw["vocab_size"], 50 + i) for i, n in enumerate(lens)]
     nxt = [7, 11, 13]
@@ -52,7 +52,8 @@ def test_bfloat16_tracks_float32_at_large_sizes(shape):
         torch.cuda.empty_cache()
     scale = outs["float32"].abs().max().item()
     assert 0.05 < scale < 50
-    torch.testing.assert_close(outs["bfloat16"], outs["float32"], atol=0.03 * max(1.0, scale), rtol=0.03)
+    rms, worst = row_errors(outs["bfloat16"], outs["float32"])
+    assert rms.max().item() < 0.07 and worst.max().item() < 0.35, (rms.max().item(), worst.max().item())
 
 
 @pytest.mark.parametrize("shape,n_seqs", [("qwen2.5:7b", 20), ("qwen2.5:32b", 40)])

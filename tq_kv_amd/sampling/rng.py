@@ -1,6 +1,7 @@
 """The uniform number of one draw: a function of (seed, request, step) and nothing
 else, so that what a request draws does not depend on which other requests share
-its batch.  Integer mixing (two rounds of the splitmix64 finaliser), top 24 bits
+its batch.  Integer mixing (three rounds of the splitmix64 finaliser, one each for seed, request
+and step), top 24 bits
 taken as a float32 in [0, 1)."""
 
 _M = (1 << 64) - 1
