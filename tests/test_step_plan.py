@@ -87,3 +87,26 @@ def test_the_native_cache_reports_what_goes_wrong():
     c.check()
     with pytest.raises(native.EngineLibraryError, match="no slot 7"):
         c.length(7)
+
+
+def test_the_library_refuses_steps_that_cannot_run():
+    c = native.NativeCache(3, [(8, 0)])
+    a, b = c.acquire(), c.acquire()
+    i32 = lambda *v: np.asarray(v, dtype=np.int32)
+    c.check_step(i32(a, b), i32(2, 1), i32(0, 99, 5), 100, 128)
+    c.check_step(i32(a), i32(1), None, 100, 128)               # tokens the host does not know
+    for slots, n_new, tokens, vocab, positions, what in [
+            (i32(), i32(), i32(), 100, 128, "at least one sequence"),
+            (i32(a, a), i32(1, 1), i32(1, 2), 100, 128, "slot 0 appears twice"),
+            (i32(a, b), i32(1, 0), i32(1), 100, 128, "Empty prompt"),
+            (i32(a, b), i32(2, 1), i32(1, 2, 100), 100, 128, "token id 100 is outside the vocabulary of 100"),
+            (i32(a), i32(1), i32(-1), 100, 128, "token id -1"),
+            (i32(a), i32(129), i32(*([1] * 129)), 100, 128, "would reach 129 positions, the model has 128")]:
+        with pytest.raises(native.StepError, match=what):
+            c.check_step(slots, n_new, tokens, vocab, positions)
+    with pytest.raises(AssertionError, match="slot 2 is not held"):
+        c.check_step(i32(2), i32(1), i32(1), 100, 128)
+    c.reserve([(a, 100)]), c.commit([(a, 100)])
+    c.check_step(i32(a), i32(28), None, 100, 128)
+    with pytest.raises(native.StepError, match="would reach 129 positions"):
+        c.check_step(i32(a), i32(29), None, 100, 128)

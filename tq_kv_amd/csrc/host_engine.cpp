@@ -243,6 +243,29 @@ int tqe_cache_check(const tqe_cache_t* c) {
 }
 
 // ---- the step's arrays ------------------------------------------------------------------------
+int tqe_check_step(const tqe_cache_t* c, int n_seqs, const int32_t* slots, const int32_t* n_new, const int32_t* tokens,
+                   int vocab_size, int max_positions) {
+    if (!c) return fail(TQE_ERR_ARGUMENT, "tqe_check_step: null pointer");
+    if (n_seqs < 1 || !slots || !n_new) return fail(TQE_ERR_STEP, "a step needs at least one sequence");
+    std::vector<uint8_t> seen(c->max_slots, 0);
+    size_t at = 0;
+    for (int i = 0; i < n_seqs; ++i) {
+        const int s = slots[i];
+        if (s < 0 || s >= c->max_slots || !c->slots.held[s]) return fail(TQE_ERR_STATE, "slot %d is not held", s);
+        if (seen[s]) return fail(TQE_ERR_STEP, "slot %d appears twice in one step", s);
+        seen[s] = 1;
+        if (n_new[i] < 1) return fail(TQE_ERR_STEP, "Empty prompt");
+        if (tokens)
+            for (int t = 0; t < n_new[i]; ++t, ++at)
+                if (tokens[at] < 0 || tokens[at] >= vocab_size)
+                    return fail(TQE_ERR_STEP, "token id %d is outside the vocabulary of %d", tokens[at], vocab_size);
+        if ((long long)c->lengths[s] + n_new[i] > max_positions)
+            return fail(TQE_ERR_STEP, "sequence would reach %lld positions, the model has %d", (long long)c->lengths[s] + n_new[i], max_positions);
+    }
+    return TQE_OK;
+}
+
+
 int tqe_plan_step(const tqe_cache_t* c, int n_seqs, const int32_t* slots, const int32_t* starts, const int32_t* n_new,
                   const int32_t* tokens, const int32_t* want_counts, const int32_t* want_idx, int width_step,
                   int32_t* out, int out_cap, int32_t* meta) {

@@ -21,6 +21,7 @@ enum {
     TQE_ERR_FULL = -2,          /* no free slot, or not enough free pages: nothing was changed */
     TQE_ERR_STATE = -3,         /* a slot that is not held, something freed twice, a broken invariant */
     TQE_ERR_RANGE = -4,         /* a wanted place outside its sequence's tokens */
+    TQE_ERR_STEP = -5,          /* a step the engine cannot run: see tqe_check_step */
     TQE_NO_LIST = -100          /* tqe_cache_pages: the slot has no page list in the group (not an error) */
 };
 
@@ -57,6 +58,15 @@ int tqe_cache_pages(const tqe_cache_t* cache, int group, int slot, int32_t* out,
 int tqe_cache_check(const tqe_cache_t* cache);
 
 /* ---- the arrays of one step ----------------------------------------------------------------- */
+/* What a step must satisfy before anything is reserved or launched (TQE_ERR_STEP with the
+ * finding otherwise): at least one sequence, no slot twice, every sequence brings a token
+ * (the reference's "Empty prompt", src/engine.rs:347-349), token ids inside the vocabulary,
+ * and no sequence grows beyond max_positions.  tokens: all sequences' tokens one after the
+ * other, or NULL where the host does not know them (they were chosen on the device). */
+int tqe_check_step(const tqe_cache_t* cache, int n_seqs, const int32_t* slots, const int32_t* n_new,
+                   const int32_t* tokens, int vocab_size, int max_positions);
+
+
 /* Sequence i of the step lives in slots[i], held starts[i] positions before the step (NULL: what
  * the cache says) and brings n_new[i] tokens (tokens: all of them, sequence after sequence);
  * want_counts[i] of its places are wanted, want_idx lists them (indices among the sequence's

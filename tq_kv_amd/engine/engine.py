@@ -7,14 +7,12 @@ sequences with unequal numbers of new tokens (whole prompts, or one token each, 
 anything between), runs exactly those tokens against what the cache holds, and
 returns the logits at the wanted places.
 """
+import numpy as np
 import torch
 
 from ..cache.store import Cache
+from ..native import StepError
 from .context import HostStaging, StepContext
-
-
-class StepError(ValueError):
-    pass
 
 
 _NoUpload = object()       # StepContext(into=_NoUpload): build the host arrays only
@@ -73,19 +71,14 @@ class Engine:
             if device_tokens.dtype != torch.int32 or tuple(device_tokens.shape) != (len(items),) \
                     or device_tokens.device.type != self.model.device.type:
                 raise StepError("device_tokens must be int32 [%d] on %s" % (len(items), self.model.device))
-        seen = set()
-        for slot, tokens, _ in items:
-            if slot in seen:
-                raise StepError("slot %d appears twice in one step" % slot)
-            seen.add(slot)
-            if len(tokens) == 0:
-                raise StepError("Empty prompt")          # src/engine.rs:347-349
-            lo, hi = min(tokens), max(tokens)
-            if lo < 0 or hi >= self.vocab_size:
-                raise StepError("token id %d is outside the vocabulary of %d" % (lo if lo < 0 else hi, self.vocab_size))
-            if self.cache.length(slot) + len(tokens) > self.max_positions:
-                raise StepError("sequence would reach %d positions, the model has %d"
-                                % (self.cache.length(slot) + len(tokens), self.max_positions))
+        # the host library checks the rest: slots held and named once, no empty prompt, tokens inside the
+        # vocabulary (where the host knows them), no sequence beyond the model's positions
+        flat = None
+        if device_tokens is None:                   # ids too large for the library's int32 stay too large for any vocabulary
+            flat = np.asarray([t for _, tokens, _ in items for t in tokens], dtype=np.int64).clip(-1, 2 ** 31 - 1).astype(np.int32)
+        self.cache.native.check_step(np.asarray([slot for slot, _, _ in items], dtype=np.int32),
+                                     np.asarray([len(tokens) for _, tokens, _ in items], dtype=np.int32),
+                                     flat, self.vocab_size, self.max_positions)
         sizes = [(slot, len(tokens)) for slot, tokens, _ in items]
         self.cache.reserve(sizes)
         ctx_items = [(slot, self.cache.length(slot), tokens) for slot, tokens, _ in items]

@@ -10,7 +10,7 @@ from .cache.pages import CacheFull
 from .csrc import build as _build
 
 _LIB = None
-OK, ERR_ARGUMENT, ERR_FULL, ERR_STATE, ERR_RANGE, NO_LIST = 0, -1, -2, -3, -4, -100
+OK, ERR_ARGUMENT, ERR_FULL, ERR_STATE, ERR_RANGE, ERR_STEP, NO_LIST = 0, -1, -2, -3, -4, -5, -100
 MAX_GROUPS = 16
 META_SIZE = 12 + 12 + 2 * MAX_GROUPS
 (META_TOTAL, META_TOKENS, META_WANT, META_LAST, META_ALL_DECODE, META_PRUNE_LAST, META_MAX_NEW, META_MAX_END,
@@ -22,6 +22,11 @@ _I32P = ctypes.POINTER(ctypes.c_int32)
 
 class EngineLibraryError(RuntimeError):
     pass
+
+
+class StepError(ValueError):
+    """A step the engine cannot run (no sequence, a slot twice, an empty prompt, a token outside
+    the vocabulary, more positions than the model has)."""
 
 
 def library():
@@ -44,6 +49,7 @@ def library():
                            ("tqe_cache_commit", [ctypes.c_void_p, ctypes.c_int, _I32P, _I32P]),
                            ("tqe_cache_pages", [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, _I32P, ctypes.c_int]),
                            ("tqe_cache_check", [ctypes.c_void_p]),
+                           ("tqe_check_step", [ctypes.c_void_p, ctypes.c_int, _I32P, _I32P, _I32P, ctypes.c_int, ctypes.c_int]),
                            ("tqe_plan_step", [ctypes.c_void_p, ctypes.c_int, _I32P, _I32P, _I32P, _I32P, _I32P, _I32P, ctypes.c_int,
                                               _I32P, ctypes.c_int, _I32P])):
             getattr(lib, name).argtypes = args
@@ -71,6 +77,8 @@ def _raise(status):
         raise AssertionError(msg)
     if status == ERR_RANGE:
         raise IndexError(msg)
+    if status == ERR_STEP:
+        raise StepError(msg)
     raise EngineLibraryError(msg)
 
 
@@ -157,6 +165,13 @@ class NativeCache:
 
     def check(self):
         status = self._lib.tqe_cache_check(self.handle)
+        if status != OK:
+            _raise(status)
+
+    def check_step(self, slots, n_new, tokens, vocab_size, max_positions):
+        """Raises StepError unless the step can run (tqe_check_step).  tokens: int32 array of all the
+        step's tokens, or None where the host does not know them."""
+        status = self._lib.tqe_check_step(self.handle, len(slots), _ptr(slots), _ptr(n_new), _ptr(tokens), int(vocab_size), int(max_positions))
         if status != OK:
             _raise(status)
 
