@@ -37,7 +37,7 @@ def main():
                     help="a preset of shape, batch, prompt length, steps and sampling; the other options override it")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--shape", default=None)
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1, 64 and 128 points")
     ap.add_argument("--no-tune", action="store_true", help="do not let the library pick its fastest kernel per product shape")
     ap.add_argument("--mixed", action="store_true",
                     help="another workload instead: --batch prompts of unequal lengths (uniform in 16..--prompt-len), sampled with "
@@ -75,7 +75,7 @@ def main():
         ctx_len = raw["max_position_embeddings"] = (needed + 1023) // 1024 * 1024
     note("making random weights for %s (%d layers)" % (args.shape, layers))
     model = Model.random(raw, seed=0, dtype="bfloat16", device="cuda:0")
-    max_batch = 64 if not args.no_points else args.batch
+    max_batch = max(128, args.batch) if not args.no_points else args.batch
     total_new = args.steps + args.warmup + 2
     engine = Engine(model, max_tokens=max_batch * ((args.prompt_len + total_new + 63) // 64 * 64))
     gen = torch.Generator().manual_seed(0)
@@ -88,7 +88,7 @@ def main():
 
     # -- prefill of one prompt --------------------------------------------------------------
     if not args.no_tune:
-        # products of more than 64 rows are the library's: let it try its kernels once for the
+        # products of more than 128 rows are the library's: let it try its kernels once for the
         # shapes of the measured prompt pass
         note("library tuning for %d rows" % args.prompt_len)
         model.tune_library(args.prompt_len)
@@ -147,7 +147,7 @@ def main():
     tps, sec_per_step, end_to_end = decode(args.batch, args.steps, args.warmup)
     points = {}
     if not args.no_points:
-        for batch, steps, warmup in ((1, min(args.steps, 64), 8), (64, min(args.steps, 32), 4)):
+        for batch, steps, warmup in ((1, min(args.steps, 64), 8), (64, min(args.steps, 32), 4), (128, min(args.steps, 16), 4)):
             note("decode at batch %d" % batch)
             b_tps, b_sec, _ = decode(batch, steps, warmup)
             gbs = hbm(batch, steps, warmup, b_sec)

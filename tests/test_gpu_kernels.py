@@ -470,9 +470,9 @@ def test_product_of_few_rows(m, n, k, form):
         assert torch.equal(one[0], out[m - 1])
 
 
-@pytest.mark.parametrize("m", [17, 32, 33, 64])
+@pytest.mark.parametrize("m", [17, 32, 33, 64, 65, 100, 128])
 @pytest.mark.parametrize("n,k", [(100, 96), (3584, 3584), (1000, 18944), (4608, 1536), (48, 32), (65610, 64), (152064, 128), (264, 1056)])
-def test_product_of_17_to_64_rows(m, n, k):
+def test_product_of_17_to_128_rows(m, n, k):
     x, w = rand(m, k, seed=32, dtype=torch.bfloat16), rand(n, k, seed=33, scale=0.05, dtype=torch.bfloat16)
     want = x.double() @ w.double().t()
     packed = K.pack_weight(w)
@@ -490,9 +490,9 @@ def test_product_of_17_to_64_rows(m, n, k):
         K.mid_store(x, w, out)
 
 
-@pytest.mark.parametrize("m", [17, 40, 64])
+@pytest.mark.parametrize("m", [17, 40, 64, 65, 90, 128])
 @pytest.mark.parametrize("inter,k", [(112, 64), (18944, 3584), (100, 96), (200, 1312), (18, 1312), (50, 2048), (7, 96)])
-def test_gated_product_of_17_to_64_rows(m, inter, k):
+def test_gated_product_of_17_to_128_rows(m, inter, k):
     x = rand(m, k, seed=34, scale=1.5, dtype=torch.bfloat16)
     w = rand(2 * inter, k, seed=35, scale=0.4 / math.sqrt(k), dtype=torch.bfloat16)       # gate and up of size about 1
     out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
@@ -507,7 +507,8 @@ def test_gated_product_of_17_to_64_rows(m, inter, k):
     torch.testing.assert_close(out.float(), act.float(), atol=2e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("m,n,k", [(40, 96, 2048), (64, 3584, 3584), (17, 100, 1056), (33, 2050, 1024), (64, 3584, 18944)])
+@pytest.mark.parametrize("m,n,k", [(40, 96, 2048), (64, 3584, 3584), (17, 100, 1056), (33, 2050, 1024), (64, 3584, 18944), (128, 3584, 18944),
+                                   (77, 100, 1056)])
 def test_unfinished_sums_of_a_product_are_finished_by_the_next_norm(m, n, k):
     x, w = rand(m, k, seed=36, dtype=torch.bfloat16), rand(n, k, seed=37, scale=0.05, dtype=torch.bfloat16)
     packed = K.pack_weight(w)
@@ -564,10 +565,10 @@ def test_unfinished_sums_of_q_k_v_are_finished_by_the_rotation_kernel(nh, nkv, d
                      keys, values, q, nh, nkv, d)
 
 
-def test_products_of_17_to_64_rows_refuse_what_they_do_not_take():
+def test_products_of_17_to_128_rows_refuse_what_they_do_not_take():
     w = K.pack_weight(rand(16, 64, dtype=torch.bfloat16))
-    with pytest.raises(K.KernelError, match="at most 64"):
-        K.mid_store(rand(65, 64, dtype=torch.bfloat16), w, torch.empty(65, 16, device=DEV))
+    with pytest.raises(K.KernelError, match="at most 128"):
+        K.mid_store(rand(129, 64, dtype=torch.bfloat16), w, torch.empty(129, 16, device=DEV))
     with pytest.raises(K.KernelError, match="packed weight is"):
         K.mid_gated(rand(20, 64, dtype=torch.bfloat16), w, torch.empty(20, 8, dtype=torch.bfloat16, device=DEV))
 

@@ -1,10 +1,10 @@
-// y[M,N] = x[M,K] w[N,K]^T for 17 to 64 rows (decoding steps of larger batches, the wanted rows
+// y[M,N] = x[M,K] w[N,K]^T for 17 to 128 rows (decoding steps of larger batches, the wanted rows
 // of many prompts): bfloat16 in, MFMA, float32 accumulation.  The reference runs these products
 // as candle matmuls (src/models/turbo_generic.rs:68-91).  At these M the product is still bound
 // by the weight bytes, which are streamed from HBM once, straight into registers, from the copy
 // packed in the lanes' order ([tile of 16 rows][K/32][lane][8 values], see skinny_fused.hip).
 //
-// With up to 64 rows x is no longer small beside a tile of weights: every wave needs all of it.
+// With this many rows x is no longer small beside a tile of weights: every wave needs all of it.
 // So a block is 4 to 8 waves that walk K together in chunks of 128; each chunk of x is staged once
 // per block in LDS, in the order the lanes read it ([16 rows][k step][lane] x 16 bytes, so both
 // the block's write and the waves' reads are linear), double buffered with one barrier per
@@ -20,6 +20,13 @@
 // (store, or the gate: silu(gate) * up of src/models/turbo_generic.rs:105-111).  The number of
 // splits depends on the product's shape alone, never on M, so a row's result does not depend on
 // the batch it is in.
+//
+// Beyond 64 rows (8 row groups) every compute unit pulls all of x through its first-level cache
+// beside its own share of the weights (0.9 MB beside 1.15 MB at 128 rows of the 7B gate+up
+// product), and that path, not HBM, sets the time: 4.1 TB/s of weights at 128 rows against 4.9 at
+// 64.  Measured there and left: reads of x two steps ahead, one or two extra waves that only bring
+// x in, a deeper ring of LDS operands (the waves wait for x behind the weights in the same
+// queue, whoever asks for it).
 #include "common.h"
 #include "tq_kernels.h"
 
@@ -31,7 +38,7 @@ enum { MID_STORE = 0, MID_GATED = 1 };
 #define MID_CHUNK 128           // k per stage
 #define MID_MIN_WAVES 4          // waves per block: from the product's shape (mid_plan)
 #define MID_MAX_WAVES 8
-#define MID_MAX_ROWS 64
+#define MID_MAX_ROWS 128
 
 struct MidArgs {
     const bf16_t* x;            // [M, K]
@@ -51,13 +58,15 @@ __device__ __forceinline__ float gate_times_up(float gate_sum, float up_sum) {
     return (g / (1.f + expf(-g))) * up;
 }
 
-// MT: groups of 16 rows of x (2: up to 32 rows, 4: up to 64).  TN: tiles of 16 features per wave
-// (gated: the gate tile and its up tile).
-template <int MT, int TN, int EPI, typename TY>
+// MT: groups of 16 rows of x (2: up to 32 rows, 4: up to 64, 8: up to 128).  TN: tiles of 16
+// features per wave (gated: the gate tile and its up tile).
+// PAR: 256-thread groups of the block that bring x in (2 in a block of 8 waves, else 1).
+template <int MT, int TN, int EPI, typename TY, int PAR>
 __global__ __launch_bounds__(MID_MAX_WAVES * TQK_WAVE)
 void mid_product_kernel(const MidArgs p) {
     constexpr int SLOTS = MT * 256;                 // 16-byte pieces of a chunk of x: [row group][k step][lane]
-    constexpr int XS = SLOTS / (MID_MIN_WAVES * TQK_WAVE);          // pieces per thread at most
+    constexpr bool WIDE = MT > 4;                   // 8 row groups: registers are short, see below
+    constexpr int XS = WIDE ? MT / PAR : SLOTS / (MID_MIN_WAVES * TQK_WAVE);       // pieces of x per thread at most
     static_assert(EPI != MID_GATED || TN == 2, "a gated block holds pairs of tiles");
     extern __shared__ u32x4_t xs[];                 // [2][SLOTS]
     const int lane = threadIdx.x % TQK_WAVE, wave = threadIdx.x / TQK_WAVE;
@@ -78,17 +87,26 @@ void mid_product_kernel(const MidArgs p) {
         const int tile = EPI == MID_GATED ? t * part_tiles + min(tile0, part_tiles - 1) : min(tile0 + t, part_tiles - 1);
         wtile[t] = p.w + (size_t)tile * tile_size + lane * 8;
     }
-    // this thread's pieces of a chunk of x; rows past M repeat the last row.  Pieces past the
-    // chunk's end (whole waves of them, with more than 4 waves) are loaded again and not stored.
-    const bf16_t* xsrc[XS];
-    int xk[XS];
+    // Up to 4 row groups: a thread's pieces of a chunk of x are those at its number plus multiples of
+    // the block's size; rows past M repeat the last row.  Pieces past the chunk's end (whole waves
+    // of them, with more than 4 waves) are loaded again and not stored.
+    const bf16_t* xsrc[WIDE ? 1 : XS];
+    int xk[WIDE ? 1 : XS];
+    if constexpr (!WIDE) {
 #pragma unroll
-    for (int i = 0; i < XS; ++i) {
-        const int s = min((int)threadIdx.x + i * (int)blockDim.x, SLOTS - 1);
-        const int mt = s / 256, ks = (s / 64) % 4, ln = s % 64;
-        xk[i] = ks * 32 + (ln / 16) * 8;
-        xsrc[i] = p.x + (size_t)min(mt * 16 + ln % 16, p.M - 1) * K;
+        for (int i = 0; i < XS; ++i) {
+            const int s = min((int)threadIdx.x + i * (int)blockDim.x, SLOTS - 1);
+            const int mt = s / 256, ks = (s / 64) % 4, ln = s % 64;
+            xk[i] = ks * 32 + (ln / 16) * 8;
+            xsrc[i] = p.x + (size_t)min(mt * 16 + ln % 16, p.M - 1) * K;
+        }
     }
+    // 8 row groups: the block's first 256 threads bring x in, thread t piece t ([k step][lane]) of
+    // every row group, so that its pieces lie 16 rows apart and need one address; in a block of 8
+    // waves the second 256 threads take every other row group (PAR = 2).
+    const int st_half = threadIdx.x / 256;
+    const bool stages = st_half < PAR;
+    const int st_row = threadIdx.x % 16, st_k = ((threadIdx.x / 64) % 4) * 32 + ((threadIdx.x % 64) / 16) * 8;
     floatx4_t acc[TN][MT];
 #pragma unroll
     for (int t = 0; t < TN; ++t)
@@ -98,16 +116,33 @@ void mid_product_kernel(const MidArgs p) {
     // Loads past the end of K stay inside the row (and are valid memory); x is zeroed there as it
     // goes into LDS, so they add nothing.  Nothing is under a condition: the waits can be counted.
     auto load_x = [&](int c, u32x4_t (&xr)[XS]) {
+        if constexpr (WIDE) {
+            if (!stages) return;
+            const uint32_t kk = (uint32_t)min(c + st_k, K - 8);
 #pragma unroll
-        for (int i = 0; i < XS; ++i) xr[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + min(c + xk[i], K - 8));
+            for (int i = 0; i < XS; ++i) {
+                const uint32_t r = (uint32_t)min((i * PAR + st_half) * 16 + st_row, p.M - 1);
+                xr[i] = *reinterpret_cast<const u32x4_t*>(p.x + (r * (uint32_t)K + kk));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < XS; ++i) xr[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + min(c + xk[i], K - 8));
+        }
     };
     auto store_x = [&](int c, int buf, const u32x4_t (&xr)[XS]) {
+        if constexpr (WIDE) {
+            if (!stages) return;
+            const bool past = c + st_k >= k_end;
 #pragma unroll
-        for (int i = 0; i < XS; ++i) {
-            u32x4_t v = xr[i];
-            if (c + xk[i] >= k_end) v = u32x4_t{0, 0, 0, 0};
-            const int s = threadIdx.x + i * blockDim.x;
-            if (s < SLOTS) xs[buf * SLOTS + s] = v;
+            for (int i = 0; i < XS; ++i) xs[buf * SLOTS + (i * PAR + st_half) * 256 + threadIdx.x % 256] = past ? u32x4_t{0, 0, 0, 0} : xr[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < XS; ++i) {
+                u32x4_t v = xr[i];
+                if (c + xk[i] >= k_end) v = u32x4_t{0, 0, 0, 0};
+                const int s = threadIdx.x + i * blockDim.x;
+                if (s < SLOTS) xs[buf * SLOTS + s] = v;
+            }
         }
     };
     auto load_w = [&](int c, bf16x8_t (&a)[TN][4]) {
@@ -118,21 +153,39 @@ void mid_product_kernel(const MidArgs p) {
             for (int t = 0; t < TN; ++t) a[t][u] = *reinterpret_cast<const bf16x8_t*>(wtile[t] + at);
         }
     };
-    auto multiply = [&](int buf, const bf16x8_t (&a)[TN][4]) {
-        u32x4_t bx[2][MT];
+    // x comes from LDS four row groups at a time (two where registers are short), the next ones on
+    // their way while these are multiplied.
+    // RING (8 row groups, where registers are short): a k step's weight registers are asked for
+    // again, for the chunk after those under way, as soon as its products are issued, so that two
+    // register sets keep nearly two chunks on their way.
+    constexpr bool RING = WIDE;
+    auto multiply = [&](int buf, bf16x8_t (&a)[TN][4], int refill_c) {
+        constexpr int G = RING && TN > 1 ? 2 : (MT < 4 ? MT : 4), NG = MT / G, STEPS = 4 * NG;
+        u32x4_t bx[2][G];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) bx[0][mt] = xs[buf * SLOTS + (mt * 4) * 64 + lane];
+        for (int g = 0; g < G; ++g) bx[0][g] = xs[buf * SLOTS + (g * 4) * 64 + lane];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            if (u < 3) {
+        for (int st = 0; st < STEPS; ++st) {
+            const int u = st / NG, grp = st % NG;
+            if (st + 1 < STEPS) {
+                const int u1 = (st + 1) / NG, grp1 = (st + 1) % NG;
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) bx[(u + 1) & 1][mt] = xs[buf * SLOTS + (mt * 4 + u + 1) * 64 + lane];
+                for (int g = 0; g < G; ++g) bx[(st + 1) & 1][g] = xs[buf * SLOTS + ((grp1 * G + g) * 4 + u1) * 64 + lane];
             }
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
+            for (int g = 0; g < G; ++g)
 #pragma unroll
                 for (int t = 0; t < TN; ++t)
-                    acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], __builtin_bit_cast(bf16x8_t, bx[u & 1][mt]), acc[t][mt], 0, 0, 0);
+                    acc[t][grp * G + g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], __builtin_bit_cast(bf16x8_t, bx[st & 1][g]),
+                                                                                  acc[t][grp * G + g], 0, 0, 0);
+            if constexpr (RING) {
+                if (grp == NG - 1) {
+                    const size_t at = (size_t)min(refill_c / 32 + u, K / 32 - 1) * 512;
+#pragma unroll
+                    for (int t = 0; t < TN; ++t) a[t][u] = *reinterpret_cast<const bf16x8_t*>(wtile[t] + at);
+                }
+                __builtin_amdgcn_sched_barrier(0);       // or the reads of many steps are issued at once and held
+            }
         }
     };
 
@@ -140,21 +193,27 @@ void mid_product_kernel(const MidArgs p) {
     // way: what a step waits for was asked for two steps (weights) or one step (x, which comes
     // from the cache) earlier.  Three register sets of weights, two of x and two LDS buffers take
     // turns, so six steps are written out for the names to come round.
-    bf16x8_t a[3][TN][4];
-    u32x4_t xr[2][XS];
+    // With 8 row groups the registers hold one set of x only: the next chunk's x is asked for at the
+    // start of a step and stored at its end (XA = 1), and the weights go round as said above, in
+    // two sets with two tiles per wave, in three with one.
+    constexpr int XA = RING ? 1 : 2;
+    constexpr int WA = RING && TN > 1 ? 2 : 3;
+    bf16x8_t a[WA][TN][4];
+    u32x4_t xr[XA][XS];
     load_w(k_begin, a[0]);
     load_w(k_begin + MID_CHUNK, a[1]);
+    if constexpr (RING && WA == 3) load_w(k_begin + 2 * MID_CHUNK, a[WA - 1]);
     load_x(k_begin, xr[0]);
-    load_x(k_begin + MID_CHUNK, xr[1]);
+    if constexpr (XA == 2) load_x(k_begin + MID_CHUNK, xr[XA - 1]);
     store_x(k_begin, 0, xr[0]);
     __syncthreads();
 #define MID_STEP(J) { \
         const int c = base + (J) * MID_CHUNK; \
-        load_x(c + 2 * MID_CHUNK, xr[(J) % 2]); \
-        load_w(c + 2 * MID_CHUNK, a[((J) + 2) % 3]); \
+        load_x(c + XA * MID_CHUNK, xr[XA == 2 ? (J) % 2 : 0]); \
+        if constexpr (!RING) load_w(c + 2 * MID_CHUNK, a[((J) + 2) % WA]); \
         __builtin_amdgcn_sched_barrier(0); \
-        multiply((J) % 2, a[(J) % 3]); \
-        store_x(c + MID_CHUNK, ((J) + 1) % 2, xr[((J) + 1) % 2]); \
+        multiply((J) % 2, a[(J) % WA], c + WA * MID_CHUNK); \
+        store_x(c + MID_CHUNK, ((J) + 1) % 2, xr[XA == 2 ? ((J) + 1) % 2 : 0]); \
         __syncthreads(); }
     int base = k_begin, left = (k_end - k_begin + MID_CHUNK - 1) / MID_CHUNK;
     for (; left >= 6; left -= 6, base += 6 * MID_CHUNK) {
@@ -307,7 +366,9 @@ static size_t mid_scratch_bytes(int M, int N, int K, bool gated) {
 template <int MT, int TN, int EPI, typename TY>
 static int launch_mid(const MidArgs& a, const MidPlan& plan, bool finish, hipStream_t s) {
     dim3 grid(plan.blocks, plan.splits);
-    mid_product_kernel<MT, TN, EPI, TY><<<grid, plan.waves * TQK_WAVE, 2 * MT * 256 * 16, s>>>(a);
+    constexpr int PAR8 = (MT > 4) ? 2 : 1;
+    if (PAR8 == 2 && plan.waves == MID_MAX_WAVES) mid_product_kernel<MT, TN, EPI, TY, PAR8><<<grid, plan.waves * TQK_WAVE, 2 * MT * 256 * 16, s>>>(a);
+    else mid_product_kernel<MT, TN, EPI, TY, 1><<<grid, plan.waves * TQK_WAVE, 2 * MT * 256 * 16, s>>>(a);
     if (tqk_check_launch("tqk_mid product")) return -1;
     if (plan.splits > 1 && finish) {
         const size_t total = (size_t)a.M * (EPI == MID_GATED ? a.N / 2 : a.N);
@@ -320,8 +381,10 @@ static int launch_mid(const MidArgs& a, const MidPlan& plan, bool finish, hipStr
 template <int EPI, typename TY>
 static int launch_rows(const MidArgs& a, const MidPlan& plan, bool finish, hipStream_t s) {
     if constexpr (EPI == MID_GATED) {
+        if (a.M > 64) return launch_mid<8, 2, EPI, TY>(a, plan, finish, s);
         return a.M > 32 ? launch_mid<4, 2, EPI, TY>(a, plan, finish, s) : launch_mid<2, 2, EPI, TY>(a, plan, finish, s);
     } else {
+        if (a.M > 64) return plan.tn == 2 ? launch_mid<8, 2, EPI, TY>(a, plan, finish, s) : launch_mid<8, 1, EPI, TY>(a, plan, finish, s);
         if (a.M > 32) return plan.tn == 2 ? launch_mid<4, 2, EPI, TY>(a, plan, finish, s) : launch_mid<4, 1, EPI, TY>(a, plan, finish, s);
         return plan.tn == 2 ? launch_mid<2, 2, EPI, TY>(a, plan, finish, s) : launch_mid<2, 1, EPI, TY>(a, plan, finish, s);
     }
@@ -339,7 +402,7 @@ static int check_mid(const MidArgs& a, const void* scratch, bool gated, bool fin
     return 0;
 }
 
-/* y[M,N] = x w^T, M <= 64, w packed; scratch: float32 [tqk_mid_splits(N, K, 0)][M][N] where that
+/* y[M,N] = x w^T, M <= 128, w packed; scratch: float32 [tqk_mid_splits(N, K, 0)][M][N] where that
  * is more than 1.  finish == 0: with more than one piece the pieces' sums are left in scratch
  * (for tqk_add_rmsnorm_sums) and y is not written. */
 extern "C" int tqk_mid_store(const void* x, const void* w_packed, void* y, int y_dtype, int M, int N, int K,

@@ -81,7 +81,7 @@ int tqk_fused_qkv(const void* x, const float* ss_parts, int n_ss_parts, float ep
                   void* keys, void* values, int n_pages, void* q_out,
                   int M, int n_heads, int n_kv_heads, int head_dim, int K, void* stream);
 
-/* Products of up to 64 rows (bfloat16, K a multiple of 32) from the packed copy of the weight.
+/* Products of up to 128 rows (bfloat16, K a multiple of 32) from the packed copy of the weight.
  * K is cut into tqk_mid_splits(N, K, gated) pieces; where that is more than 1, scratch is
  * float32 [pieces][M][N], 16-byte aligned.  finish == 0: with more than one piece the pieces'
  * sums stay in scratch (tqk_add_rmsnorm_sums adds them up) and y is not written. */

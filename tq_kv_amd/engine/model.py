@@ -58,11 +58,11 @@ class Model:
         self.few_head = None
         self.loaded = False
         # a step can be captured as a graph if every part's forward launches the same kernels
-        # whatever the step's data are; up to 64 rows (the hand-written products; where a weight
+        # whatever the step's data are; up to 128 rows (the hand-written products; where a weight
         # has no packed copy the library's, which capture as they are)
         self.graph_safe = (all(getattr(b, "graph_safe", False) for b in self.blocks) and getattr(self.final_norm, "graph_safe", False)
                            and (self.stream_position is None or getattr(self.stream_position, "graph_safe", False)))
-        self.graph_max_rows = 64
+        self.graph_max_rows = K.MID_MAX_ROWS
 
     # -- tensors ----------------------------------------------------------
     def tensor_specs(self):
@@ -137,7 +137,7 @@ class Model:
 
     def tune_library(self, rows):
         """Let the library try its kernels once for every product of the model at `rows`
-        rows (more than 64, or 16 without packed weights: fewer never reach the library) and
+        rows (more than 128, or 16 without packed weights: fewer never reach the library) and
         keep the fastest for later calls.  Takes seconds per distinct weight shape."""
         own_rows = K.MID_MAX_ROWS if L.POLICY["mid"] and L.POLICY["packed"] else L.POLICY["skinny_max_rows"]
         if self.dtype != torch.bfloat16 or rows <= own_rows:
@@ -166,7 +166,7 @@ class Model:
         # small decoding steps: products fold the norms and the residual sums around them in
         ctx.fuse_small = (L.POLICY["fused"] and self.dtype == torch.bfloat16 and ctx.all_decode
                           and ctx.n_tokens <= 16 and s.hidden_size % 32 == 0)
-        # steps of 17 to 64 tokens: a part's last product may leave its sums to the next norm's kernel
+        # steps of 17 to 128 tokens: a part's last product may leave its sums to the next norm's kernel
         ctx.fuse_mid = (L.POLICY["mid"] and self.dtype == torch.bfloat16
                         and L.POLICY["skinny_max_rows"] < ctx.n_tokens <= K.MID_MAX_ROWS)
         # the norm that reads the stream first in every run, and after the last one

@@ -416,7 +416,7 @@ def fused_gated(x, weight_gate_up, out, norm=None):
     return out
 
 
-MID_MAX_ROWS = 64
+MID_MAX_ROWS = 128
 
 
 class PartialSums:
@@ -435,7 +435,7 @@ def _mid_scratch(m, n, k, gated, device):
 
 
 def mid_store(x, weight, out=None, finish=True):
-    """out[M,N] = x weight^T for up to 64 rows of bfloat16; weight: a PackedWeight; out: bfloat16
+    """out[M,N] = x weight^T for up to 128 rows of bfloat16; weight: a PackedWeight; out: bfloat16
     or float32, made here (bfloat16) if not given.  finish=False: where the kernel cuts K into
     pieces, their PartialSums (of out's dtype) are returned in place of out."""
     m, k = x.shape
@@ -454,7 +454,7 @@ def mid_store(x, weight, out=None, finish=True):
 
 
 def mid_gated(x, weight_gate_up, out):
-    """out[M, I] = silu(gate) * up of x [gate; up]^T for up to 64 rows; weight: a PackedWeight in 2 parts."""
+    """out[M, I] = silu(gate) * up of x [gate; up]^T for up to 128 rows; weight: a PackedWeight in 2 parts."""
     m, inter = out.shape
     k = x.shape[1]
     if not isinstance(weight_gate_up, PackedWeight):

@@ -5,7 +5,7 @@ x = x + mixer(norm(x)); x = x + ff(norm(x)), with optional norms on the mixer's 
 the feed-forward's outputs (:1965-1968, :1976-1979).
 
 The residual stream is float32 (parts.linear.Stream).  A part's output is left pending
-on the stream and added inside the next norm's kernel (for steps of 17 to 64 tokens a
+on the stream and added inside the next norm's kernel (for steps of 17 to 128 tokens a
 part's last product may even leave its sums over pieces of K pending: the norm's kernel
 adds those up too).  In small decoding steps the
 framework's parts go further: a product that consumes a norm computes it itself

@@ -11,7 +11,7 @@ The reference's linear layers are candle matmuls, i.e. library GEMMs
            It reads a second copy of the weight, packed at loading time in the order its
            lanes take it (few_rows_form): a decoding step is bound by the weight bytes, and
            in that order they stream faster.
-  bfloat16, 17 to 64 rows (decoding steps of larger batches) where the weight has a packed copy
+  bfloat16, 17 to 128 rows (decoding steps of larger batches) where the weight has a packed copy
         -> the hand-written kernel that stages x in LDS and streams the packed weights
            (kernels.mid_store, kernels.mid_gated)
   bfloat16, more rows (prompts, large decoding batches)
@@ -26,7 +26,7 @@ from .. import kernels as K
 # plain kernel); nothing else reads these.
 # Measured on MI355X at the Qwen2.5-7B sizes: up to 16 rows the skinny kernel is ahead of the
 # library on every product; at 64 rows the library is ahead of it on every one, and the kernel
-# for 17 to 64 rows ("mid") ahead of the library.
+# for 17 to 128 rows ("mid") ahead of the library.
 # "packed": parts keep the second, packed copy of their weights for the few-row kernels (twice
 # the weight memory, about an eighth less time per decoding step).
 POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16, "fused": True, "prune_last": True, "packed": True,
@@ -51,7 +51,7 @@ class Stream:
 
     def add_product(self, x, weight):
         """h += bfloat16(x weight^T), preparing next_norm.  weight: [N, K] or its few-row form.
-        Up to 16 rows: in the product's epilogue.  17 to 64 rows (weight in its few-row form):
+        Up to 16 rows: in the product's epilogue.  17 to 128 rows (weight in its few-row form):
         the product, or where next_norm can add them up its sums over pieces of K, is left
         pending for the next norm's kernel."""
         if x.shape[0] > POLICY["skinny_max_rows"]:
@@ -89,7 +89,7 @@ def few_rows_form(weight, parts=1):
 
 def leaves_sums(x_rows, weight, few):
     """Whether a product of x_rows rows with this weight (few: its few-row form) goes through the
-    kernel for 17 to 64 rows, which can leave its sums to the next norm (Stream.add_product)."""
+    kernel for 17 to 128 rows, which can leave its sums to the next norm (Stream.add_product)."""
     return (POLICY["mid"] and few is not None and weight.dtype == torch.bfloat16
             and POLICY["skinny_max_rows"] < x_rows <= K.MID_MAX_ROWS)
 
@@ -151,7 +151,7 @@ def gated_silu_linear(x, weight_gate_up, few=None):
 def linear(x, weight, bias=None, out_dtype=None, few=None, leave_sums=False):
     """x: [M,K]; weight: [N,K]; bias: [N] or None.  Returns [M,N] of out_dtype
     (default: x's dtype).  few: the weight's few_rows_form, if there is one.  leave_sums: the
-    caller also takes the product unfinished, as kernels.PartialSums (the kernel for 17 to 64
+    caller also takes the product unfinished, as kernels.PartialSums (the kernel for 17 to 128
     rows gives those where it cuts K into pieces)."""
     m, k = x.shape
     n = weight.shape[0]
