@@ -414,8 +414,8 @@ def test_sampled_generation_float32_equals_plain(name):
 
 
 @pytest.fixture(params=["own", "library", "rows"])
-def products_of_17_to_64_rows(request):
-    """The kernel for 17 to 64 rows (the default), the library's products in its place, and
+def products_of_17_to_128_rows(request):
+    """The kernel for 17 to 128 rows (the default), the library's products in its place, and
     weights without a packed copy (then the few-row kernels read the rows and 17 rows on the library)."""
     from tq_kv_amd.parts import linear as L
     old = dict(L.POLICY)
@@ -427,18 +427,20 @@ def products_of_17_to_64_rows(request):
     L.POLICY.update(old)
 
 
+@pytest.mark.parametrize("n_seqs", [40, 100])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_many_sequences_decode_through_replayed_graphs(dtype, products_of_17_to_64_rows):
-    # 40 sequences: more rows than the few-row products take, so the captured step holds the
-    # products for 17 to 64 rows; every replay is checked (with other work between the replays)
-    if dtype == "float32" and products_of_17_to_64_rows != "own":
+def test_many_sequences_decode_through_replayed_graphs(dtype, products_of_17_to_128_rows, n_seqs):
+    # 40 or 100 sequences: more rows than the few-row products take, so the captured step holds the
+    # products for 17 to 128 rows (4 and 8 groups of 16 rows); every replay is checked (with other
+    # work between the replays)
+    if dtype == "float32" and products_of_17_to_128_rows != "own":
         pytest.skip("the switches are for bfloat16 products")
-    if products_of_17_to_64_rows == "own":
+    if products_of_17_to_128_rows == "own":
         eng = G.engine("B", dtype, True)
     else:       # weights loaded and graphs captured under the switched policy
         from tq_kv_amd import Engine, Model
         eng = Engine(Model.from_dir(G.folder("B", True), dtype=dtype), max_tokens=8192)
-    reqs = G.prompts("B", [3 + (7 * i) % 50 for i in range(40)], seed=1000)
+    reqs = G.prompts("B", [3 + (7 * i) % 50 for i in range(n_seqs)], seed=1000)
     slots = [eng.open() for _ in reqs]
     heads = [len(r) - 6 for r in reqs]
     heads = [max(1, h) for h in heads]
