@@ -51,6 +51,18 @@ def test_tq_generate_runs_and_is_greedy_reproducible():
 
 
 @pytest.mark.gpu
+def test_tq_generate_with_packed_weights_only_emits_the_same_tokens():
+    # steps of up to 128 rows run the same kernels with and without the weights' rows
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "tq"), "generate", "tiny:b", "--prompt-ids", "1,2,3",
+           "--prompt-ids", "9 8 7 6 5 4 3 2", "-n", "8", "-t", "0", "--repeat-penalty", "1.0", "--json"]
+    a = subprocess.run(cmd, capture_output=True, text=True)
+    b = subprocess.run(cmd + ["--packed-weights-only"], capture_output=True, text=True)
+    assert a.returncode == 0 and b.returncode == 0, a.stderr + b.stderr
+    outs = [json.loads(r.stdout.strip().splitlines()[-1])["outputs"] for r in (a, b)]
+    assert outs[0] == outs[1] and [len(o) for o in outs[0]] == [8, 8]
+
+
+@pytest.mark.gpu
 def test_tq_generate_on_a_folder_written_by_tq_random_weights_emits_the_plain_tokens(tmp_path):
     """`tq random-weights` writes a folder, `tq generate <folder>` loads it and generates; the
     tokens it prints are the plain implementation's greedy tokens for the same folder, and a stop

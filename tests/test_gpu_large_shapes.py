@@ -237,3 +237,49 @@ def test_a_step_of_more_than_three_thousand_tokens_takes_the_wide_tiles():
     want = plain_rows(tensors, dict(raw), prompts[1] + [5], [0, 99, 100])
     got = torch.cat([outs["float32"][3:5], outs["float32"][6:7]])
     torch.testing.assert_close(got, want, atol=2e-5 * max(1.0, want.abs().max().item()), rtol=2e-5)
+
+
+@pytest.mark.parametrize("shape", ["qwen2.5:7b", "qwen2.5:1.5b"])
+def test_a_model_without_weight_rows_gives_the_same_results(shape):
+    """POLICY["keep_rows"] off: the rows of packed weights are given back and prompts of more than
+    128 tokens go through the kernel for 17 to 128 rows in pieces.  Steps of up to 128 rows run the
+    same kernels either way (equal bit for bit); a prompt of 300 tokens is compared with the plain
+    implementation as the other bfloat16 runs here are."""
+    from tq_kv_amd.parts import linear as L
+    raw = two_layer(shape)
+    tensors = sharpened(tensors_for(raw, 6))
+    prompts = [helpers.random_tokens(n, raw["vocab_size"], 70 + i) for i, n in enumerate([300, 100, 20])]
+    outs, held = {}, {}
+    for keep in (True, False):
+        torch.cuda.empty_cache()
+        before = torch.cuda.memory_allocated()
+        old = L.POLICY["keep_rows"]
+        L.POLICY["keep_rows"] = keep
+        try:
+            model = build(raw, "bfloat16", tensors)
+        finally:
+            L.POLICY["keep_rows"] = old
+        held[keep] = torch.cuda.memory_allocated() - before
+        mixer, ffn = model.blocks[0].mixer, model.blocks[0].feed_forward
+        for w in (mixer.w_qkv, mixer.w_o, ffn.w_gate_up, ffn.w_down):
+            assert torch.is_tensor(w) == keep
+        assert torch.is_tensor(model.head) == (keep or bool(raw.get("tie_word_embeddings")))
+        eng = Engine(model, max_tokens=1024)
+        slots = [eng.open() for _ in prompts]
+        got = [eng.step([(slots[0], prompts[0], [0, 127, 128, 299])]),
+               eng.step([(slots[1], prompts[1], [0, 99]), (slots[2], prompts[2], [19])]),
+               eng.step([(s, [5 + i], [0]) for i, s in enumerate(slots)])]
+        outs[keep] = [g.cpu() for g in got]
+        for s in slots:
+            eng.close(s)
+        del eng, model
+    assert torch.equal(outs[True][1], outs[False][1]) and torch.equal(outs[True][2][1:], outs[False][2][1:])
+    want = plain_rows(tensors, raw, prompts[0], [0, 127, 128, 299])
+    for keep in (True, False):
+        rms, worst = row_errors(outs[keep][0], want)
+        assert rms.max().item() < 0.07 and worst.max().item() < 0.35, (keep, rms, worst)
+    # what is given back: the rows of every packed weight.  Here that shows for the weights the parts
+    # had put together themselves (q/k/v and gate/up); the others' rows are this test's own tensors.
+    rows = sum(v.numel() * 2 for k, v in tensors.items()
+               if k.endswith(".weight") and any(p in k for p in ("q_proj", "k_proj", "v_proj", "gate_proj", "up_proj")))
+    assert abs((held[True] - held[False]) - rows) < 0.02 * rows, (held, rows)

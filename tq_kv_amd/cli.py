@@ -42,6 +42,9 @@ def _add_model(p):
     p.add_argument("--weights-seed", type=int, default=0, help="Seed of the random weights of a shape")
     p.add_argument("--allow-extra-tensors", action="store_true",
                    help="Tensors in the folder that the model does not use are a warning, not an error")
+    p.add_argument("--packed-weights-only", action="store_true",
+                   help="Keep only the copy of the bfloat16 weights that the decoding kernels read (half the weight memory; "
+                        "prompts of more than 128 tokens then run several times slower)")
     p.add_argument("--max-cache-tokens", type=int, default=0,
                    help="Positions the cache holds for all live requests together (0: what the prompts need)")
 
@@ -81,9 +84,12 @@ def build_parser():
     return ap
 
 
-def load_model(name, dtype, weights_seed, strict=True):
+def load_model(name, dtype, weights_seed, strict=True, packed_only=False):
     from .config import catalog
     from .engine import Model
+    if packed_only:
+        from .parts import linear
+        linear.POLICY["keep_rows"] = False
     if os.path.isdir(name):
         return Model.from_dir(name, dtype=dtype, strict=strict)
     if catalog.find(name) is None:
@@ -117,7 +123,8 @@ def cmd_generate(args):
             prompts.append(tokenizer.encode(text, add_special_tokens=False).ids)       # as src/engine.rs:342-345
     if not prompts:
         raise SystemExit("no prompt: give --prompt-ids, --prompt-file or --prompt")
-    model = load_model(args.model, args.dtype, args.weights_seed, strict=not args.allow_extra_tensors)
+    model = load_model(args.model, args.dtype, args.weights_seed, strict=not args.allow_extra_tensors,
+                       packed_only=args.packed_weights_only)
     params = GenerationParams(max_tokens=args.max_tokens, temperature=args.temperature, top_p=args.top_p,
                               top_k=args.top_k, repeat_penalty=args.repeat_penalty, seed=args.seed)
     eos = _ids(args.eos) if args.eos is not None else list(model.stop_token_ids)
@@ -149,7 +156,7 @@ def cmd_bench(args):
     from .cache.store import PAGE
     from .engine import Engine, generate
     from .sampling import GenerationParams
-    model = load_model(args.model, args.dtype, args.weights_seed)
+    model = load_model(args.model, args.dtype, args.weights_seed, packed_only=args.packed_weights_only)
     g = torch.Generator().manual_seed(0)
     prompt = torch.randint(0, model.spec.vocab_size, (args.prompt_len,), generator=g).tolist()
     engine = Engine(model, max_tokens=args.max_cache_tokens or (args.prompt_len + args.tokens + 2 * PAGE) // PAGE * PAGE)

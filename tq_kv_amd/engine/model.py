@@ -96,6 +96,7 @@ class Model:
         if s.head_bias_name is not None:
             self.head_bias = tensors[s.head_bias_name].to(torch.float32)
         self.few_head = L.few_rows_form(self.head)      # the head's copy for the few-row kernel
+        self.head = L.rows_or_stand_in(self.head, self.few_head, needed=s.head_name is None)       # a tied head's rows are the embedding
         self.loaded = True
         return self
 
@@ -145,6 +146,7 @@ class Model:
         L.tune_library(True)
         seen = set()
         products = [w for b in self.blocks for w in b.product_weights()] + [(self.head, torch.float32)]
+        products = [(w, d) for w, d in products if torch.is_tensor(w)]
         for weight, out_dtype in products:
             key = (tuple(weight.shape), out_dtype)
             if weight.dtype != torch.bfloat16 or key in seen:

@@ -11,7 +11,7 @@ import math
 import torch
 
 from .. import kernels as K
-from .linear import LazyNorm, few_rows_form, fusable, leaves_sums, linear
+from .linear import LazyNorm, few_rows_form, fusable, leaves_sums, linear, rows_or_stand_in
 from .registry import Part, register
 from .spec import KVNeed, TensorSpec
 
@@ -75,12 +75,14 @@ class Attention(Part):
         self.b_o = tensors.get("o_proj.bias")
         self.few_qkv = few_rows_form(self.w_qkv)
         self.few_o = few_rows_form(self.w_o)
+        self.w_qkv = rows_or_stand_in(self.w_qkv, self.few_qkv)
+        self.w_o = rows_or_stand_in(self.w_o, self.few_o, needed=self.b_o is not None)
 
     def cache_need(self):
         return KVNeed(self.n_kv_heads, self.head_dim, self.window)
 
     def product_weights(self):
-        return [(self.w_qkv, None), (self.w_o, None)]
+        return [(w, None) for w in (self.w_qkv, self.w_o) if torch.is_tensor(w)]
 
     def _fused_qkv_ok(self, ctx):
         """The folded q/k/v kernel takes decoding steps (row m is sequence m) of rotary

@@ -4,7 +4,7 @@ up are one product with the weights stacked."""
 import torch
 
 from .. import kernels as K
-from .linear import LazyNorm, few_rows_form, fusable, gated_silu_linear, leaves_sums, linear
+from .linear import LazyNorm, few_rows_form, fusable, gated_silu_linear, leaves_sums, linear, rows_or_stand_in
 from .registry import Part, register
 from .spec import TensorSpec
 
@@ -32,9 +32,11 @@ class GatedSiLU(Part):
         self.w_down = tensors["down_proj.weight"]
         self.few_gate_up = few_rows_form(self.w_gate_up, parts=2)
         self.few_down = few_rows_form(self.w_down)
+        self.w_gate_up = rows_or_stand_in(self.w_gate_up, self.few_gate_up)
+        self.w_down = rows_or_stand_in(self.w_down, self.few_down)
 
     def product_weights(self):
-        return [(self.w_gate_up, None), (self.w_down, None)]
+        return [(w, None) for w in (self.w_gate_up, self.w_down) if torch.is_tensor(w)]
 
     def folds_norm(self, ctx):
         return fusable(ctx.n_tokens, self.w_gate_up)

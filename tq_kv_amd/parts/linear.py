@@ -29,8 +29,11 @@ from .. import kernels as K
 # for 17 to 128 rows ("mid") ahead of the library.
 # "packed": parts keep the second, packed copy of their weights for the few-row kernels (twice
 # the weight memory, about an eighth less time per decoding step).
+# "keep_rows": False gives the rows up once a weight is packed (set it before loading): half the
+# weight memory again; products of more than 128 rows (prompts) then go through the kernel for
+# 17 to 128 rows in pieces, each of which streams the weight once, instead of the library.
 POLICY = {"skinny": True, "library": True, "skinny_max_rows": 16, "fused": True, "prune_last": True, "packed": True,
-          "mid": True}
+          "mid": True, "keep_rows": True}
 
 
 class Stream:
@@ -75,6 +78,25 @@ class LazyNorm:
 
     def __init__(self, xw, ss, n_ss, eps):
         self.xw, self.norm = xw, (ss, n_ss, eps)
+
+
+class PackedOnly:
+    """Stands where a weight's rows were: its shape, dtype and device, no data.  The products
+    take the packed copy (`few`) for any number of rows."""
+
+    def __init__(self, weight):
+        self.shape, self.dtype, self.device, self.is_cuda = tuple(weight.shape), weight.dtype, weight.device, weight.is_cuda
+
+    def dim(self):
+        return len(self.shape)
+
+
+def rows_or_stand_in(weight, few, needed=False):
+    """The weight itself, or (POLICY["keep_rows"] off, a packed copy there, and nobody else needing
+    the rows) a PackedOnly in its place, so that the rows' memory is given back."""
+    if POLICY["keep_rows"] or few is None or needed or not (POLICY["mid"] and POLICY["skinny"]):
+        return weight
+    return PackedOnly(weight)
 
 
 def few_rows_form(weight, parts=1):
@@ -145,7 +167,17 @@ def gated_silu_linear(x, weight_gate_up, few=None):
         return K.fused_gated(x, few or weight_gate_up, act)
     if _mid_ok(x, weight_gate_up, few):
         return K.mid_gated(x, few, act)
+    if isinstance(weight_gate_up, PackedOnly):
+        for piece, rows in _pieces(x, act):
+            (K.fused_gated if piece.shape[0] <= POLICY["skinny_max_rows"] else K.mid_gated)(piece, few, rows)
+        return act
     return K.swiglu(linear(x, weight_gate_up), act)
+
+
+def _pieces(x, out):
+    """x and out cut into pieces of as many rows as the kernel for 17 to 128 rows takes."""
+    step = K.MID_MAX_ROWS
+    return [(x[r:r + step], out[r:r + step]) for r in range(0, x.shape[0], step)]
 
 
 def linear(x, weight, bias=None, out_dtype=None, few=None, leave_sums=False):
@@ -166,10 +198,17 @@ def linear(x, weight, bias=None, out_dtype=None, few=None, leave_sums=False):
         if _mid_ok(x, weight, few):
             out = torch.empty((m, n), dtype=out_dtype, device=x.device)
             return K.mid_store(x, few, out, finish=not leave_sums)
+        if isinstance(weight, PackedOnly):
+            out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+            for piece, rows in _pieces(x, out):
+                (K.fused_store if piece.shape[0] <= POLICY["skinny_max_rows"] else K.mid_store)(piece, few, rows)
+            return out
         if POLICY["library"] and m > POLICY["skinny_max_rows"]:
             if out_dtype == torch.bfloat16:
                 return torch.matmul(x, weight.t())
             if out_dtype == torch.float32:
                 return torch.mm(x, weight.t(), out_dtype=torch.float32)
+    if isinstance(weight, PackedOnly):
+        raise RuntimeError("linear: this weight's rows were given up (POLICY['keep_rows']); only bfloat16 products without a bias take its packed copy")
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     return K.gemm(x, weight, bias, out)
