@@ -52,6 +52,8 @@ def _add_model(p):
 def build_parser():
     ap = argparse.ArgumentParser(prog="tq", description="tq for MI355X -- local LLM inference (Qwen2 dense decoder)")
     ap.add_argument("--fp32", action="store_true", help="Run everything in true 32-bit (same as --dtype float32)")
+    ap.add_argument("--trace", action="store_true",
+                    help="Named ranges (model, attn, attn-mlp, rms-norm, output) around the parts of every step, for a profiler's marker trace")
     sub = ap.add_subparsers(dest="command")
     g = sub.add_parser("generate", help="Generate tokens for prompts")
     _add_model(g)
@@ -216,6 +218,9 @@ def main(argv=None):
         return 0
     if getattr(args, "fp32", False) and hasattr(args, "dtype"):
         args.dtype = "float32"
+    if args.trace:
+        from . import tracing
+        tracing.enable()
     if args.command == "generate":
         return cmd_generate(args)
     if args.command == "bench":

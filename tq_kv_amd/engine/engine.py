@@ -12,6 +12,7 @@ import torch
 
 from ..cache.store import Cache
 from ..native import StepError
+from ..tracing import span
 from .context import HostStaging, StepContext
 
 
@@ -79,6 +80,10 @@ class Engine:
         self.cache.native.check_step(np.asarray([slot for slot, _, _ in items], dtype=np.int32),
                                      np.asarray([len(tokens) for _, tokens, _ in items], dtype=np.int32),
                                      flat, self.vocab_size, self.max_positions)
+        with span("step"):
+            return self._step(items, borrow, device_tokens)
+
+    def _step(self, items, borrow, device_tokens):
         sizes = [(slot, len(tokens)) for slot, tokens, _ in items]
         self.cache.reserve(sizes)
         ctx_items = [(slot, self.cache.length(slot), tokens) for slot, tokens, _ in items]

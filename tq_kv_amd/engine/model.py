@@ -14,6 +14,7 @@ from ..parts import linear as L
 from ..parts.linear import linear
 from ..parts.registry import BuildEnv
 from ..parts.spec import TensorSpec
+from ..tracing import span
 from ..weights import load_folder, random_tensors, write_model_folder
 
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
@@ -163,6 +164,10 @@ class Model:
         float32 for ctx's wanted rows."""
         if not self.loaded:
             raise RuntimeError("the model has no weights yet")
+        with span("model"):                 # the reference's span, src/models/turbo_generic.rs:1932
+            return self._forward(ctx, cache)
+
+    def _forward(self, ctx, cache):
         s = self.spec
         h = torch.empty((ctx.n_tokens, s.hidden_size), dtype=torch.float32, device=self.device)
         # small decoding steps: products fold the norms and the residual sums around them in
@@ -194,7 +199,8 @@ class Model:
         n_rows = ctx.dev.want_rows.shape[0]
         if n_rows == 0:
             return torch.empty((0, s.vocab_size), dtype=torch.float32, device=self.device)
-        return self._finish(self._head(stream, ctx, n_rows))
+        with span("output"):                # src/models/turbo_generic.rs:1933
+            return self._finish(self._head(stream, ctx, n_rows))
 
     def _finish(self, logits):
         """Bias, scale and cap of the logits, where the architecture has them."""

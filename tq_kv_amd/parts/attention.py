@@ -22,6 +22,7 @@ class Attention(Part):
     window (None or positions a query sees, itself included), scale (None: 1/sqrt(head_dim)),
     position (PartSpec); optional prompt_tile: queries per tile of the prompt kernel (16, 32, 64 or
     128; default: what the kernel library finds fitting for the step's size and these head counts)."""
+    trace_name = "attn"                 # the reference's span, src/models/turbo_generic.rs:1920
 
     def __init__(self, params, env):
         self.env = env

@@ -13,6 +13,7 @@ framework's parts go further: a product that consumes a norm computes it itself
 that the norm kernels disappear; parts that do not offer this (`folds_norm`,
 `adds_to_stream`) are simply given tensors.
 """
+from ..tracing import span
 from .linear import POLICY
 from .registry import Part, register
 
@@ -74,7 +75,8 @@ class PreNormBlock(Part):
             lazy = norm.lazy(stream)
             if lazy is not None:
                 return lazy
-        x = norm.add_norm(stream.h, stream.pending)
+        with span(getattr(norm, "trace_name", "norm")):
+            x = norm.add_norm(stream.h, stream.pending)
         stream.pending = None
         stream.invalidate()
         return x
@@ -82,12 +84,13 @@ class PreNormBlock(Part):
     def _run(self, part, post_norm, next_norm, x, stream, ctx, *extra):
         """Run a part; its output is added to the stream by the part itself (it returns None)
         or is left pending for the next norm's kernel."""
-        if ((ctx.fuse_small or getattr(ctx, "fuse_mid", False)) and post_norm is None
-                and getattr(part, "adds_to_stream", None) and part.adds_to_stream(ctx)):
-            stream.next_norm = next_norm
-            out = part.forward(x, ctx, *extra, stream=stream)
-        else:
-            out = part.forward(x, ctx, *extra)
+        with span(getattr(part, "trace_name", "part")):
+            if ((ctx.fuse_small or getattr(ctx, "fuse_mid", False)) and post_norm is None
+                    and getattr(part, "adds_to_stream", None) and part.adds_to_stream(ctx)):
+                stream.next_norm = next_norm
+                out = part.forward(x, ctx, *extra, stream=stream)
+            else:
+                out = part.forward(x, ctx, *extra)
         if out is not None:
             if post_norm is not None:
                 out = post_norm.forward(out)
@@ -108,14 +111,18 @@ class PreNormBlock(Part):
         return stream
 
     def _forward_last_rows(self, stream, ctx, entry):
-        x = self.mixer_norm.add_norm(stream.h, stream.pending)
-        y = self.mixer.forward(x, ctx, entry, last_rows=True)          # keys and values of all tokens, output of the rows
+        with span(getattr(self.mixer_norm, "trace_name", "norm")):
+            x = self.mixer_norm.add_norm(stream.h, stream.pending)
+        with span(getattr(self.mixer, "trace_name", "part")):
+            y = self.mixer.forward(x, ctx, entry, last_rows=True)      # keys and values of all tokens, output of the rows
         sub = type(stream)(stream.h.index_select(0, ctx.dev.last_rows))
         sub.of_last_rows = True
         if ctx.n_last == 0:
             return sub
         sub.pending = self.post_mixer_norm.forward(y) if self.post_mixer_norm is not None else y
-        x = self.ff_norm.add_norm(sub.h, sub.pending)
-        out = self.feed_forward.forward(x, ctx)
+        with span(getattr(self.ff_norm, "trace_name", "norm")):
+            x = self.ff_norm.add_norm(sub.h, sub.pending)
+        with span(getattr(self.feed_forward, "trace_name", "part")):
+            out = self.feed_forward.forward(x, ctx)
         sub.pending = self.post_ff_norm.forward(out) if self.post_ff_norm is not None else out
         return sub

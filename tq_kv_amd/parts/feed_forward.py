@@ -13,6 +13,7 @@ from .spec import TensorSpec
 class GatedSiLU(Part):
     """params: hidden, inter."""
     graph_safe = True
+    trace_name = "attn-mlp"             # the reference's span, src/models/turbo_generic.rs:1922
 
     def __init__(self, params, env):
         self.hidden = int(params["hidden"])

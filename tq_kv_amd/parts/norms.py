@@ -12,6 +12,7 @@ from .spec import TensorSpec
 class RMSNorm(Part):
     """params: size, eps."""
     graph_safe = True
+    trace_name = "rms-norm"             # the reference's span, src/models/turbo_generic.rs:36
     takes_partial_sums = True       # add_norm and gather_add_norm take a product's kernels.PartialSums as the update
 
     def __init__(self, params, env):
