@@ -75,9 +75,14 @@ def main():
         ctx_len = raw["max_position_embeddings"] = (needed + 1023) // 1024 * 1024
     note("making random weights for %s (%d layers)" % (args.shape, layers))
     model = Model.random(raw, seed=0, dtype="bfloat16", device="cuda:0")
-    max_batch = max(128, args.batch) if not args.no_points else args.batch
     total_new = args.steps + args.warmup + 2
-    engine = Engine(model, max_tokens=max_batch * ((args.prompt_len + total_new + 63) // 64 * 64))
+    per_seq = (args.prompt_len + total_new + 63) // 64 * 64           # positions a sequence holds at the end
+    # the other batch sizes, as far as their caches fit beside the weights (long contexts: not all do)
+    free_bytes = torch.cuda.mem_get_info(0)[0]
+    point_batches = [] if args.no_points else [b for b in (1, 64, 128)
+                                               if b * per_seq * layers * 2 * nkv * d * 2 < 0.8 * free_bytes]
+    max_batch = max([args.batch] + point_batches)
+    engine = Engine(model, max_tokens=max_batch * per_seq)
     gen = torch.Generator().manual_seed(0)
 
     def prompts(n):
@@ -148,6 +153,8 @@ def main():
     points = {}
     if not args.no_points:
         for batch, steps, warmup in ((1, min(args.steps, 64), 8), (64, min(args.steps, 32), 4), (128, min(args.steps, 16), 4)):
+            if batch not in point_batches:
+                continue
             note("decode at batch %d" % batch)
             b_tps, b_sec, _ = decode(batch, steps, warmup)
             gbs = hbm(batch, steps, warmup, b_sec)
