@@ -210,6 +210,52 @@ def test_rope_store_vector_kernel_equals_the_general_one(nh, nkv, d, with_bias):
         assert ok.any()
 
 
+@pytest.mark.parametrize("with_bias", [True, False])
+@pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (3, 1, 64), (5, 5, 40)])
+def test_rope_store_of_many_tokens_equals_the_general_kernel(nh, nkv, d, with_bias):
+    # steps of 128 tokens and more store their values through a kernel of their own, whose lanes run
+    # along the tokens: three sequences in a packed step (a prompt from 0, a piece that starts inside a
+    # page, one token), scrambled pages; against the general kernel (reached with a float32 bias), and
+    # with the product given as its sums over pieces of K
+    starts, counts = [0, 37, 200], [150, 131, 1]
+    tok_seq = ints([i for i, n in enumerate(counts) for _ in range(n)])
+    tok_pos = ints([s + j for s, n in zip(starts, counts) for j in range(n)])
+    n = sum(counts)
+    n_pages = 12
+    table = ints([[7, 2, 9, -1], [4, 11, 0, -1], [5, 8, 1, 3]])
+    total = (nh + 2 * nkv) * d
+    qkv = rand(n, total, seed=14, dtype=torch.bfloat16)
+    bias = rand(total, seed=15, dtype=torch.bfloat16) if with_bias else None
+    c, s_ = plain.rope_tables(d, 1e4, 300)
+    cos, sin = c.to(DEV), s_.to(DEV)
+    # the same product as sums of three pieces that add up to it exactly (a half and two quarters)
+    sums = K.PartialSums(torch.stack([qkv.float() * 0.5, qkv.float() * 0.25, qkv.float() * 0.25]).contiguous(), torch.bfloat16)
+    results = []
+    for how in ("vector", "general", "sums"):
+        keys, values = make_cache(n_pages, nkv, d, torch.bfloat16)
+        q = torch.empty(n, nh, d, dtype=torch.bfloat16, device=DEV)
+        b = bias
+        if how == "general":
+            b = bias.float() if with_bias else torch.zeros(total, device=DEV)
+        K.rope_store(sums if how == "sums" else qkv, b, cos, sin, d, K.STYLE_HALVES, tok_seq, tok_pos, table, keys, values, q, nh, nkv, d)
+        results.append((q, keys, values))
+    for other in results[1:]:
+        for a, b in zip(results[0], other):
+            assert torch.equal(torch.isnan(a.float()), torch.isnan(b.float()))          # the same places written
+            ok = ~torch.isnan(a.float())
+            torch.testing.assert_close(a.float()[ok], b.float()[ok], atol=1e-2, rtol=1e-2)
+            assert ok.any()
+    # vector kernel and sums: the same numbers rounded the same way
+    for a, b in zip(results[0], results[2]):
+        assert torch.equal(torch.nan_to_num(a.float()), torch.nan_to_num(b.float()))
+    # every value where the layout says: page of the position, kv head, element, place of the position
+    v_want = (qkv.float() + (bias.float() if with_bias else 0)).to(torch.bfloat16).float()[:, (nh + nkv) * d:].reshape(n, nkv, d).cpu()
+    got = results[0][2].float().cpu()
+    for t in range(0, n, 7):
+        page = table.cpu()[tok_seq[t].item(), tok_pos[t].item() // 64].item()
+        assert torch.equal(got[page, :, :, value_place(tok_pos[t].item() % 64)], v_want[t]), t
+
+
 def paged(k, v, page_ids, n_pages, dtype):
     """Lay k, v [nkv, S, d] out in pages given by page_ids; everything else is NaN."""
     nkv, s, d = k.shape

@@ -376,6 +376,55 @@ __global__ void rope_store_kernel(const TA* __restrict__ qkv, const TB* __restri
     }
 }
 
+// The values of a step of many tokens.  The cache keeps them transposed inside a page, so the kernel
+// below, whose lanes run along head_dim, stores every element as 2 bytes into a row of its own:
+// 8 of the 16 us it takes for 2048 tokens at the 7B sizes.  In these blocks the lanes run along the tokens (64
+// per block, one kv head, the waves taking chunks of 8 elements in turn): where the tokens are
+// neighbours in a sequence, as in a prompt, a wave's stores of one element fall into one 128-byte row.
+// Every lane finds its own page and place, so nothing depends on the tokens being neighbours.
+// job: (group of 64 tokens) * n_kv_heads + kv head.
+__device__ __forceinline__ void store_values_bf16(int job, const bf16_t* __restrict__ qkv, const PartSums ps, const bf16_t* __restrict__ bias,
+                                                  const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                                                  const int32_t* __restrict__ page_table, int table_width, bf16_t* __restrict__ values,
+                                                  int n_tokens, int n_heads, int n_kv_heads, int head_dim) {
+    const int lane = threadIdx.x % TQK_WAVE, wave = threadIdx.x / TQK_WAVE, n_waves = blockDim.x / TQK_WAVE;
+    const int t = (job / n_kv_heads) * TQK_WAVE + lane, kvh = job % n_kv_heads;
+    if (t >= n_tokens) return;
+    const int pos = tok_pos[t];
+    const int page = page_table[(size_t)tok_seq[t] * table_width + pos / TQK_PAGE];
+    if (page < 0) return;                              // the host never lets this happen
+    bf16_t* dst = values + ((size_t)page * n_kv_heads + kvh) * TQK_PAGE * head_dim + value_place(pos % TQK_PAGE);
+    const size_t total = (size_t)(n_heads + 2 * n_kv_heads) * head_dim;
+    const size_t at = (size_t)t * total + (size_t)(n_heads + n_kv_heads + kvh) * head_dim;
+    for (int c = wave * 8; c < head_dim; c += n_waves * 8) {
+        float v[8];
+        if (ps.sums) {
+            float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+            for (int s = 0; s < ps.n; ++s) {
+                const float4 pa = *reinterpret_cast<const float4*>(ps.sums + (size_t)s * ps.stride + at + c);
+                const float4 pb = *reinterpret_cast<const float4*>(ps.sums + (size_t)s * ps.stride + at + c + 4);
+                a.x += pa.x; a.y += pa.y; a.z += pa.z; a.w += pa.w;
+                b.x += pb.x; b.y += pb.y; b.z += pb.z; b.w += pb.w;
+            }
+            const float sums[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = to_float(from_float<bf16_t>(sums[k]));
+        } else {
+            const uint4 raw = *reinterpret_cast<const uint4*>(qkv + at + c);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) { v[2 * k] = __uint_as_float(w[k] << 16); v[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u); }
+        }
+        if (bias) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(bias + (size_t)(n_heads + n_kv_heads + kvh) * head_dim + c);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) { v[2 * k] += __uint_as_float(w[k] << 16); v[2 * k + 1] += __uint_as_float(w[k] & 0xffff0000u); }
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) dst[(size_t)(c + k) * TQK_PAGE].bits = (uint16_t)float_to_bf16_bits(v[k]);
+    }
+}
 // The common case in bfloat16 (halves layout over the whole head, head_dim a multiple of 8): a
 // thread takes 4 neighbouring elements of the first half and the 4 they rotate with, 8 bytes
 // per load and store; 16 heads of a token per block.  The q, k, v product may come unfinished, as
@@ -386,7 +435,14 @@ __global__ void rope_store_halves_bf16_kernel(const bf16_t* __restrict__ qkv, co
                                               const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ page_table,
                                               int table_width, bf16_t* __restrict__ keys, bf16_t* __restrict__ values,
                                               bf16_t* __restrict__ q_out, int n_heads, int n_kv_heads, int head_dim,
-                                              int write_kv) {
+                                              int write_kv, int value_layer, int n_tokens) {
+    // write_kv == 2: the values are stored by the blocks of the grid's last layer (blockIdx.y == value_layer)
+    if (write_kv == 2 && (int)blockIdx.y == value_layer) {
+        const int jobs = ((n_tokens + TQK_WAVE - 1) / TQK_WAVE) * n_kv_heads;
+        for (int job = blockIdx.x; job < jobs; job += gridDim.x)
+            store_values_bf16(job, qkv, ps, bias, tok_seq, tok_pos, page_table, table_width, values, n_tokens, n_heads, n_kv_heads, head_dim);
+        return;
+    }
     const int t = blockIdx.x;
     const int per_head = head_dim / 8;                  // threads per head
     const int slot = blockIdx.y * blockDim.x + threadIdx.x;
@@ -394,6 +450,7 @@ __global__ void rope_store_halves_bf16_kernel(const bf16_t* __restrict__ qkv, co
     if (head >= n_heads + 2 * n_kv_heads) return;
     const int kind = head < n_heads ? 0 : (head < n_heads + n_kv_heads ? 1 : 2);
     if (kind != 0 && !write_kv) return;
+    if (kind == 2 && write_kv == 2) return;            // the values are the last layer's
     const int pos = tok_pos[t];
     const size_t total = (size_t)(n_heads + 2 * n_kv_heads) * head_dim;
     float lo[4], hi[4];
@@ -465,6 +522,8 @@ __global__ void rope_store_halves_bf16_kernel(const bf16_t* __restrict__ qkv, co
     *reinterpret_cast<uint2*>(dst + i + half) = make_uint2(hi_bits[0] | (hi_bits[1] << 16), hi_bits[2] | (hi_bits[3] << 16));
 }
 
+#define STORE_VALUES_MIN_TOKENS 128        // fewer tokens: the plain way costs no more
+
 // Whether the 8-byte kernel takes these (then the product may also come as its sums).
 static bool rope_store_vector_case(int act_dtype, const void* bias, int bias_dtype, int rot_dim, int style, int head_dim) {
     return act_dtype == TQK_BF16 && (!bias || bias_dtype == TQK_BF16) && style == 1 && rot_dim == head_dim && head_dim % 8 == 0;
@@ -496,10 +555,13 @@ static int rope_store(const void* qkv, const PartSums ps, int act_dtype, const v
         ((((uintptr_t)qkv) | ((uintptr_t)ps.sums) | ((uintptr_t)bias) | ((uintptr_t)cos_table) | ((uintptr_t)sin_table) |
           ((uintptr_t)keys) | ((uintptr_t)q_out)) & 15) == 0) {
         const int slots = (n_heads + 2 * n_kv_heads) * (head_dim / 8);
-        dim3 vgrid(n_tokens, (slots + 255) / 256);
+        const bool values_apart = write_kv && n_tokens >= STORE_VALUES_MIN_TOKENS;
+        const int layers = (slots + 255) / 256;
+        dim3 vgrid(n_tokens, layers + (values_apart ? 1 : 0));
         rope_store_halves_bf16_kernel<<<vgrid, 256, 0, s>>>(
             (const bf16_t*)qkv, ps, (const bf16_t*)bias, cos_table, sin_table, max_positions, tok_seq, tok_pos, page_table,
-            table_width, (bf16_t*)keys, (bf16_t*)values, (bf16_t*)q_out, n_heads, n_kv_heads, head_dim, write_kv);
+            table_width, (bf16_t*)keys, (bf16_t*)values, (bf16_t*)q_out, n_heads, n_kv_heads, head_dim,
+            values_apart ? 2 : (write_kv ? 1 : 0), layers, n_tokens);
         return tqk_check_launch("tqk_rope_store");
     }
     TQK_REQUIRE(!ps.sums, "tqk_rope_store_sums: only bfloat16, rotation in halves over the whole head, head_dim a multiple of 8, "
