@@ -246,3 +246,38 @@ def test_stop_tokens_default_to_those_the_model_names():
     assert generate(Named(), [[1]], params, make_sampler=make) == [[10]]
     assert generate(Named(), [[1]], params, eos_ids=(), make_sampler=lambda p, ids: ScriptSampler([[10, 99, 12] + [1] * 8], ids))[0][:3] == [10, 99, 12]
     assert generate(FakeEngine(), [[1]], GenerationParams(max_tokens=3, temperature=0.0), make_sampler=make) == [[10, 99, 12]]
+
+
+def test_the_librarys_decisions_about_a_drawn_token():
+    from tq_kv_amd import native
+    p = native.BatchProgress(3, 3, {7, 9, 2 ** 40})        # three tokens each at most; 7 and 9 stop (an id no token can be is left out)
+    assert [p.goes_on(r) for r in range(3)] == [True, True, True]
+    assert p.accept(0, 5) == native.TOKEN_FEED and p.emitted(0) == 1 and p.goes_on(0)
+    assert p.accept(0, 6) == native.TOKEN_FEED and p.emitted(0) == 2 and not p.goes_on(0)     # its next token will be its last
+    assert p.accept(0, 8) == native.TOKEN_LAST and p.emitted(0) == 3 and p.ended(0)
+    assert p.accept(0, 8) == native.TOKEN_DROPPED and p.emitted(0) == 3                        # a step that ran ahead for nothing
+    assert p.accept(1, 9) == native.TOKEN_STOP and p.emitted(1) == 0 and p.ended(1) and not p.goes_on(1)
+    assert p.accept(1, 5) == native.TOKEN_DROPPED
+    assert p.accept(2, 2 ** 40) == native.TOKEN_FEED and not p.ended(2)
+    with pytest.raises(native.EngineLibraryError, match="no request 3"):
+        p.accept(3, 1)
+    none_wanted = native.BatchProgress(1, 0, ())
+    assert not none_wanted.goes_on(0) and none_wanted.accept(0, 5) == native.TOKEN_STOP and none_wanted.emitted(0) == 0
+    one = native.BatchProgress(1, 1, ())
+    assert not one.goes_on(0) and one.accept(0, 5) == native.TOKEN_LAST
+
+
+def test_the_librarys_batches_and_prompt_steps():
+    from tq_kv_amd import native
+    from tq_kv_amd.cache import CacheFull
+    assert native.plan_batches([], 5, 64, 4) == []
+    assert native.plan_batches([1], 1, 64, 4) == [[0]]
+    assert native.plan_batches([64, 64, 64], 1, 128, 8) == [[0, 1], [2]]            # 64 + 0 more positions: one page each
+    assert native.plan_batches([64, 64, 64], 2, 128, 8) == [[0], [1], [2]]          # 65 positions: two pages each
+    assert native.plan_batches([5] * 5, 3, 10 ** 12, 2) == [[0, 1], [2, 3], [4]]
+    with pytest.raises(CacheFull, match="request 1 needs 192 cache positions, the engine has 128"):
+        native.plan_batches([10, 129], 5, 128, 8)
+    assert native.prompt_steps([], 8) == []
+    assert native.prompt_steps([3, 4, 2], 5) == [[(0, 0, 3), (1, 0, 2)], [(1, 2, 4), (2, 0, 2)]]
+    assert native.prompt_steps([10], 10) == [[(0, 0, 10)]]
+    assert native.prompt_steps([2, 2, 2, 2], 4) == [[(0, 0, 2), (1, 0, 2)], [(2, 0, 2), (3, 0, 2)]]

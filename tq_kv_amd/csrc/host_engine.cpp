@@ -98,7 +98,7 @@ struct tqe_cache {
 extern "C" {
 
 const char* tqe_last_error(void) { return g_error; }
-int tqe_abi_version(void) { return 1; }
+int tqe_abi_version(void) { return 2; }
 
 tqe_cache_t* tqe_cache_new(int max_slots, int n_groups, const int32_t* pages_per_group, const int32_t* window_per_group) {
     if (max_slots < 1 || n_groups < 0 || n_groups > TQE_MAX_GROUPS || (n_groups > 0 && (!pages_per_group || !window_per_group))) {
@@ -390,3 +390,103 @@ int tqe_plan_step(const tqe_cache_t* c, int n_seqs, const int32_t* slots, const 
 }
 
 }  // extern "C"
+
+// ---- the generation loop's decisions ------------------------------------------------------------
+struct tqe_batch {
+    int max_new;
+    std::vector<int32_t> stop;          // sorted
+    std::vector<int32_t> emitted;
+    std::vector<uint8_t> ended;
+};
+
+int tqe_plan_batches(int n, const int32_t* prompt_lens, int max_new, long long max_tokens, int max_batch, int holds_pages,
+                     int32_t* batch_of) {
+    if (n < 0 || (n > 0 && (!prompt_lens || !batch_of)) || max_batch < 1) return fail(TQE_ERR_ARGUMENT, "tqe_plan_batches: bad arguments");
+    int batch = 0, in_batch = 0;
+    long long used = 0;
+    for (int i = 0; i < n; ++i) {
+        long long need = 0;
+        if (holds_pages) need = (long long)pages_for((long long)prompt_lens[i] + std::max(0, max_new - 1)) * TQE_PAGE;
+        if (need > max_tokens) return fail(TQE_ERR_FULL, "request %d needs %lld cache positions, the engine has %lld", i, need, max_tokens);
+        if (in_batch > 0 && (in_batch >= max_batch || used + need > max_tokens)) {
+            ++batch;
+            in_batch = 0;
+            used = 0;
+        }
+        batch_of[i] = batch;
+        ++in_batch;
+        used += need;
+    }
+    return n > 0 ? batch + 1 : 0;
+}
+
+int tqe_prompt_steps(int n, const int32_t* lens, int max_step_tokens, int32_t* pieces, int capacity) {
+    if (n < 0 || (n > 0 && !lens) || max_step_tokens < 1 || capacity < 0 || (capacity > 0 && !pieces))
+        return fail(TQE_ERR_ARGUMENT, "tqe_prompt_steps: bad arguments");
+    int count = 0, step = 0, room = max_step_tokens;
+    for (int i = 0; i < n; ++i) {
+        int begin = 0;
+        while (begin < lens[i]) {
+            const int take = std::min(lens[i] - begin, room);
+            if (count < capacity) {
+                int32_t* p = pieces + (size_t)count * 4;
+                p[0] = i; p[1] = begin; p[2] = begin + take; p[3] = step;
+            }
+            ++count;
+            begin += take;
+            room -= take;
+            if (room == 0) {
+                ++step;
+                room = max_step_tokens;
+            }
+        }
+    }
+    return count;
+}
+
+tqe_batch_t* tqe_batch_new(int n_requests, int max_new, const int32_t* stop_ids, int n_stop_ids) {
+    if (n_requests < 0 || n_stop_ids < 0 || (n_stop_ids > 0 && !stop_ids)) {
+        fail(TQE_ERR_ARGUMENT, "tqe_batch_new: bad arguments");
+        return nullptr;
+    }
+    tqe_batch_t* b = new (std::nothrow) tqe_batch_t();
+    if (!b) {
+        fail(TQE_ERR_ARGUMENT, "tqe_batch_new: out of memory");
+        return nullptr;
+    }
+    b->max_new = max_new;
+    b->stop.assign(stop_ids, stop_ids + n_stop_ids);
+    std::sort(b->stop.begin(), b->stop.end());
+    b->emitted.assign(n_requests, 0);
+    b->ended.assign(n_requests, 0);
+    return b;
+}
+
+void tqe_batch_free(tqe_batch_t* b) { delete b; }
+
+int tqe_batch_accept(tqe_batch_t* b, int row, int token) {
+    if (!b || row < 0 || row >= (int)b->emitted.size()) return fail(TQE_ERR_ARGUMENT, "tqe_batch_accept: no request %d", row);
+    if (b->ended[row]) return TQE_TOKEN_DROPPED;
+    if (b->emitted[row] >= b->max_new || std::binary_search(b->stop.begin(), b->stop.end(), (int32_t)token)) {
+        b->ended[row] = 1;
+        return TQE_TOKEN_STOP;
+    }
+    if (++b->emitted[row] >= b->max_new) {
+        b->ended[row] = 1;
+        return TQE_TOKEN_LAST;
+    }
+    return TQE_TOKEN_FEED;
+}
+
+int tqe_batch_goes_on(const tqe_batch_t* b, int row) {
+    return b && row >= 0 && row < (int)b->emitted.size() && !b->ended[row] && b->emitted[row] + 1 < b->max_new;
+}
+
+int tqe_batch_emitted(const tqe_batch_t* b, int row) {
+    if (!b || row < 0 || row >= (int)b->emitted.size()) return fail(TQE_ERR_ARGUMENT, "tqe_batch_emitted: no request %d", row);
+    return b->emitted[row];
+}
+
+int tqe_batch_ended(const tqe_batch_t* b, int row) {
+    return b && row >= 0 && row < (int)b->emitted.size() && b->ended[row];
+}

@@ -90,6 +90,41 @@ int tqe_plan_step(const tqe_cache_t* cache, int n_seqs, const int32_t* slots, co
                   const int32_t* tokens, const int32_t* want_counts, const int32_t* want_idx, int width_step,
                   int32_t* out, int out_cap, int32_t* meta);
 
+/* ---- the generation loop's decisions -------------------------------------------------------
+ * The loop computes nothing: it decides which requests run together, how their prompts are cut
+ * into steps, and what becomes of every drawn token (the reference's loop for one request:
+ * src/engine.rs:364-438). */
+
+/* Cut the requests, in order, into batches that start together: at most max_batch requests each
+ * and, where the cache holds pages (holds_pages), at most max_tokens positions, a request counted
+ * as prompt + max_new - 1 positions rounded up to whole pages (its last token is never fed).
+ * batch_of[i]: the number of request i's batch.  Returns the number of batches, or TQE_ERR_FULL
+ * where one request alone needs more than max_tokens. */
+int tqe_plan_batches(int n_requests, const int32_t* prompt_lens, int max_new, long long max_tokens, int max_batch,
+                     int holds_pages, int32_t* batch_of);
+
+/* Cut a batch's prompts into steps of at most max_step_tokens tokens: whole prompts together while
+ * they fit, a longer one in pieces that come in order.  pieces: [capacity][4] = prompt, begin, end,
+ * step.  Returns the number of pieces (none written beyond capacity: call again with as many). */
+int tqe_prompt_steps(int n_prompts, const int32_t* lens, int max_step_tokens, int32_t* pieces, int capacity);
+
+/* A batch's progress: how many tokens each of its requests has emitted and which have ended. */
+typedef struct tqe_batch tqe_batch_t;
+tqe_batch_t* tqe_batch_new(int n_requests, int max_new, const int32_t* stop_ids, int n_stop_ids);
+void tqe_batch_free(tqe_batch_t* batch);
+enum {
+    TQE_TOKEN_FEED = 0,     /* emitted; the request goes on with it */
+    TQE_TOKEN_LAST = 1,     /* emitted; the request has its max_new tokens and ends */
+    TQE_TOKEN_STOP = 2,     /* a stop token, or nothing more was wanted: not emitted (src/engine.rs:381), the request ends */
+    TQE_TOKEN_DROPPED = 3   /* the request had ended before (a step that ran ahead for nothing) */
+};
+/* What becomes of the token drawn for request `row`; counts it.  TQE_ERR_ARGUMENT for a bad row. */
+int tqe_batch_accept(tqe_batch_t* batch, int row, int token);
+/* Whether `row` will want another step after its next token unless that is a stop token. */
+int tqe_batch_goes_on(const tqe_batch_t* batch, int row);
+int tqe_batch_emitted(const tqe_batch_t* batch, int row);
+int tqe_batch_ended(const tqe_batch_t* batch, int row);
+
 #ifdef __cplusplus
 }
 #endif

@@ -10,9 +10,13 @@ every request has been served.
 
 The loop only decides; it computes nothing.  It needs of the engine `open()`,
 `close(slot)`, `step(items)`, `max_tokens` and `max_positions`, and of the sampler
-`sample(logits, rows)`, so it can be tested without a GPU.
+`sample(logits, rows)`, so it can be tested without a GPU.  The decisions themselves (which
+requests run together, how prompts are cut into steps, what becomes of a drawn token) are the
+engine's host library's (tqe_plan_batches, tqe_prompt_steps, tqe_batch_*); this file calls the
+engine and the sampler in the order they ask for.
 """
-from ..cache.store import PAGE
+from .. import native
+from ..cache.pages import CacheFull
 from ..sampling.params import GenerationParams
 
 
@@ -20,29 +24,14 @@ class GenerationError(ValueError):
     pass
 
 
-def _room(prompt_len, max_new):
-    """Cache positions a request may come to hold, counted in whole pages."""
-    longest = prompt_len + max(0, max_new - 1)      # the last emitted token is never fed
-    return (longest + PAGE - 1) // PAGE * PAGE
-
-
 def plan_batches(prompt_lens, max_new, max_tokens, max_batch, holds_pages=True):
     """Cut the requests, in order, into batches that fit the cache: at most max_batch
     requests and at most max_tokens positions (whole pages each; not counted where the
     engine's cache holds no pages: holds_pages False).  Returns lists of request indices."""
-    batches, cur, used = [], [], 0
-    for i, n in enumerate(prompt_lens):
-        need = _room(n, max_new) if holds_pages else 0
-        if need > max_tokens:
-            raise GenerationError("request %d needs %d cache positions, the engine has %d" % (i, need, max_tokens))
-        if cur and (len(cur) >= max_batch or used + need > max_tokens):
-            batches.append(cur)
-            cur, used = [], 0
-        cur.append(i)
-        used += need
-    if cur:
-        batches.append(cur)
-    return batches
+    try:
+        return native.plan_batches(prompt_lens, max_new, max_tokens, max_batch, holds_pages)
+    except CacheFull as e:
+        raise GenerationError(str(e))
 
 
 def generate(engine, prompts, params=None, eos_ids=None, on_tokens=None, max_batch=64, make_sampler=None,
@@ -84,20 +73,7 @@ def generate(engine, prompts, params=None, eos_ids=None, on_tokens=None, max_bat
 def _prompt_steps(lens, max_step_tokens):
     """Cut prompts of the given lengths into steps of at most max_step_tokens tokens.
     Returns steps, each a list of (index, begin, end); a prompt's pieces come in order."""
-    steps, cur, room = [], [], max_step_tokens
-    for i, n in enumerate(lens):
-        begin = 0
-        while begin < n:
-            take = min(n - begin, room)
-            cur.append((i, begin, begin + take))
-            begin += take
-            room -= take
-            if room == 0:
-                steps.append(cur)
-                cur, room = [], max_step_tokens
-    if cur:
-        steps.append(cur)
-    return steps
+    return native.prompt_steps(lens, max_step_tokens)
 
 
 class _Known:
@@ -139,30 +115,29 @@ def _run_batch(engine, prompts, batch, params, eos, emitted, on_tokens, sampler,
                 drawn.update(zip(ends, sampler.sample(logits, ends)))
         rows = list(range(len(batch)))                 # indices into `batch` whose token is in `draw`
         draw = _Known([drawn[b] for b in rows])
-        stopped = set()                                # requests that ended while a step with them was under way
+        progress = native.BatchProgress(len(batch), params.max_tokens, eos)
         while rows:
             # the step after this draw, for those that go on if their unread token is no stop token
             next_rows, next_draw = [], None
             if ahead and not isinstance(draw, _Known):
-                next_rows = [b for b in rows if b not in stopped and len(emitted[batch[b]]) + 1 < params.max_tokens]
+                next_rows = [b for b in rows if progress.goes_on(b)]
                 if next_rows:
                     tokens = sampler.pick(draw, [rows.index(b) for b in next_rows])
                     logits = engine.step([(slots[batch[b]], [0], [0]) for b in next_rows], device_tokens=tokens, **borrow)
                     next_draw = sampler.draw(logits, next_rows)
             feed, pairs = [], []
             for b, tok in zip(rows, draw.read()):
-                if b in stopped:
+                what = progress.accept(b, tok)
+                if what == native.TOKEN_DROPPED:        # it ended while a step with it was under way
                     continue
                 r = batch[b]
-                if len(emitted[r]) >= params.max_tokens or tok in eos:
+                if what == native.TOKEN_STOP:
                     engine.close(slots.pop(r))          # stop tokens are not emitted (src/engine.rs:381)
-                    stopped.add(b)
                     continue
                 emitted[r].append(tok)
                 pairs.append((r, tok))
-                if len(emitted[r]) >= params.max_tokens:
+                if what == native.TOKEN_LAST:
                     engine.close(slots.pop(r))          # nothing more to draw for it
-                    stopped.add(b)
                     continue
                 feed.append((b, tok))
             if on_tokens is not None and pairs:

@@ -51,9 +51,19 @@ def library():
                            ("tqe_cache_check", [ctypes.c_void_p]),
                            ("tqe_check_step", [ctypes.c_void_p, ctypes.c_int, _I32P, _I32P, _I32P, ctypes.c_int, ctypes.c_int]),
                            ("tqe_plan_step", [ctypes.c_void_p, ctypes.c_int, _I32P, _I32P, _I32P, _I32P, _I32P, _I32P, ctypes.c_int,
-                                              _I32P, ctypes.c_int, _I32P])):
+                                              _I32P, ctypes.c_int, _I32P]),
+                           ("tqe_plan_batches", [ctypes.c_int, _I32P, ctypes.c_int, ctypes.c_longlong, ctypes.c_int, ctypes.c_int, _I32P]),
+                           ("tqe_prompt_steps", [ctypes.c_int, _I32P, ctypes.c_int, _I32P, ctypes.c_int]),
+                           ("tqe_batch_accept", [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]),
+                           ("tqe_batch_goes_on", [ctypes.c_void_p, ctypes.c_int]),
+                           ("tqe_batch_emitted", [ctypes.c_void_p, ctypes.c_int]),
+                           ("tqe_batch_ended", [ctypes.c_void_p, ctypes.c_int])):
             getattr(lib, name).argtypes = args
             getattr(lib, name).restype = ctypes.c_int
+        lib.tqe_batch_new.restype = ctypes.c_void_p
+        lib.tqe_batch_new.argtypes = [ctypes.c_int, ctypes.c_int, _I32P, ctypes.c_int]
+        lib.tqe_batch_free.argtypes = [ctypes.c_void_p]
+        lib.tqe_batch_free.restype = None
         _LIB = lib
     return _LIB
 
@@ -194,3 +204,78 @@ def plan_step(cache, slots, starts, n_new, tokens, want_counts, want_idx, width_
     if status != OK:
         _raise(status)
     return out[:int(meta[META_TOTAL])], meta
+
+
+# ---- the generation loop's decisions ----------------------------------------------------------
+TOKEN_FEED, TOKEN_LAST, TOKEN_STOP, TOKEN_DROPPED = 0, 1, 2, 3
+
+
+def plan_batches(prompt_lens, max_new, max_tokens, max_batch, holds_pages=True):
+    """tqe_plan_batches: lists of request indices, one list per batch.  CacheFull where one request
+    alone does not fit."""
+    lens = np.ascontiguousarray(prompt_lens, dtype=np.int32)
+    batch_of = np.zeros(len(lens), dtype=np.int32)
+    n = library().tqe_plan_batches(len(lens), _ptr(lens), int(max_new), int(max_tokens), int(max_batch), 1 if holds_pages else 0,
+                                   _ptr(batch_of))
+    if n < 0:
+        _raise(n)
+    batches = [[] for _ in range(n)]
+    for i, b in enumerate(batch_of.tolist()):
+        batches[b].append(i)
+    return batches
+
+
+def prompt_steps(lens, max_step_tokens):
+    """tqe_prompt_steps: steps, each a list of (prompt, begin, end)."""
+    lens = np.ascontiguousarray(lens, dtype=np.int32)
+    n = library().tqe_prompt_steps(len(lens), _ptr(lens), int(max_step_tokens), None, 0)
+    if n < 0:
+        _raise(n)
+    pieces = np.zeros((max(n, 1), 4), dtype=np.int32)
+    n = library().tqe_prompt_steps(len(lens), _ptr(lens), int(max_step_tokens), _ptr(pieces), len(pieces))
+    if n < 0:
+        _raise(n)
+    steps = []
+    for i, begin, end, step in pieces[:n].tolist():
+        while len(steps) <= step:
+            steps.append([])
+        steps[step].append((i, begin, end))
+    return steps
+
+
+class BatchProgress:
+    """tqe_batch_t: how many tokens each request of a batch has emitted, which have ended, and
+    what becomes of a drawn token."""
+
+    def __init__(self, n_requests, max_new, stop_ids):
+        stop = np.ascontiguousarray(sorted(set(int(t) for t in stop_ids if -2 ** 31 <= int(t) < 2 ** 31)), dtype=np.int32)
+        self._lib = library()
+        self.handle = self._lib.tqe_batch_new(int(n_requests), int(max_new), _ptr(stop) if len(stop) else None, len(stop))
+        if not self.handle:
+            raise EngineLibraryError(_message())
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            self._lib.tqe_batch_free(self.handle)
+            self.handle = None
+
+    def accept(self, row, token):
+        token = int(token)
+        if not -2 ** 31 <= token < 2 ** 31:
+            token = -1                       # no stop id is outside the library's int32
+        status = self._lib.tqe_batch_accept(self.handle, int(row), token)
+        if status < 0:
+            _raise(status)
+        return status
+
+    def goes_on(self, row):
+        return bool(self._lib.tqe_batch_goes_on(self.handle, int(row)))
+
+    def emitted(self, row):
+        n = self._lib.tqe_batch_emitted(self.handle, int(row))
+        if n < 0:
+            _raise(n)
+        return n
+
+    def ended(self, row):
+        return bool(self._lib.tqe_batch_ended(self.handle, int(row)))
