@@ -78,7 +78,8 @@ def test_the_native_cache_reports_what_goes_wrong():
         c.reserve([(a, 1)])
     assert c.acquire() == a                       # what came back last goes out first
     c.reserve([(a, PAGE + 1)])
-    assert c.pages(0, a) == [0, 1] and c.pages(0, b) is None and c.counts(0) == (1, 3)
+    first = c.pages(0, a)
+    assert len(set(first)) == 2 and all(0 <= p < 3 for p in first) and c.pages(0, b) is None and c.counts(0) == (1, 3)
     with pytest.raises(CacheFull, match="2 more pages"):
         c.reserve([(b, 2 * PAGE)])
     assert c.pages(0, b) is None and c.counts(0) == (1, 3)        # nothing was taken
@@ -110,3 +111,30 @@ def test_the_library_refuses_steps_that_cannot_run():
     c.check_step(i32(a), i32(28), None, 100, 128)
     with pytest.raises(native.StepError, match="would reach 129 positions"):
         c.check_step(i32(a), i32(29), None, 100, 128)
+
+
+def test_runs_of_pages_lie_an_odd_number_of_pages_apart():
+    # equally long prompts would otherwise get runs of pages a power of two apart in memory
+    for run in (32, 31, 16, 2):
+        c = native.NativeCache(8, [(8 * 40, 0)])
+        slots = [c.acquire() for _ in range(6)]
+        c.reserve([(s, run * PAGE) for s in slots])
+        c.commit([(s, run * PAGE) for s in slots])
+        firsts = [c.pages(0, s)[0] for s in slots]
+        for s in slots:
+            pages = c.pages(0, s)
+            assert pages == list(range(pages[0], pages[0] + run))          # a run of neighbours
+        assert all((b - a) % 2 == 1 and b - a <= run + 2 for a, b in zip(firsts, firsts[1:])), (run, firsts)
+        # single pages, as decoding takes them, pass nothing over; what was passed over is still free
+        c.reserve([(s, 1) for s in slots])
+        tails = [c.pages(0, s)[-1] for s in slots]
+        assert tails == list(range(tails[0], tails[0] + 6))
+        free, n = c.counts(0)
+        assert free == 8 * 40 - 6 * (run + 1) and n == 8 * 40
+        c.check()
+    # a pool that has exactly what is needed gives it all
+    c = native.NativeCache(2, [(64, 0)])
+    a, b = c.acquire(), c.acquire()
+    c.reserve([(a, 32 * PAGE), (b, 32 * PAGE)])
+    assert sorted(c.pages(0, a) + c.pages(0, b)) == list(range(64))
+    c.check()
