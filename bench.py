@@ -100,7 +100,7 @@ def main():
     p = prompts(1)[0]
     times = []
     note("prefill of %d tokens" % args.prompt_len)
-    for i in range(5):
+    for i in range(8):
         slot = engine.open()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
