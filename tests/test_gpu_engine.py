@@ -417,14 +417,14 @@ def test_sampled_generation_float32_equals_plain(name):
 def products_of_17_to_128_rows(request):
     """The kernel for 17 to 128 rows (the default), the library's products in its place, and
     weights without a packed copy (then the few-row kernels read the rows and 17 rows on the library)."""
-    from tq_kv_amd.parts import linear as L
-    old = dict(L.POLICY)
+    from tq_kv_amd import POLICY
+    old = dict(POLICY.items())
     if request.param == "library":
-        L.POLICY["mid"] = False
+        POLICY["mid"] = False
     if request.param == "rows":
-        L.POLICY["packed"] = False
+        POLICY["packed"] = False
     yield request.param
-    L.POLICY.update(old)
+    POLICY.update(old)
 
 
 @pytest.mark.parametrize("n_seqs", [40, 100])

@@ -871,7 +871,7 @@ def test_fused_kernels_refuse_what_they_do_not_take():
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_random_normal_on_the_gpu_equals_the_hosts_bit_for_bit(dtype):
     import numpy as np
-    from tq_kv_amd.weights.random_init import standard_normal_host, tensor_key
+    from tq_kv_amd.weights import standard_normal_host, tensor_key
     key = tensor_key(11, "some.weight")
     n = 3_000_001
     for std, plus_one in ((0.02, False), (0.02, True), (1.0, False)):

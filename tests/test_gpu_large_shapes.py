@@ -159,7 +159,7 @@ def test_prompts_of_two_thousand_tokens_and_graphed_decoding_at_7b_sizes():
     the probabilities alone, so they agree far more closely than bfloat16 and float32 do (whose
     difference at these sizes is rounding noise of 2 to 4 % of the logits' spread in every row):
     close enough that one foreign page among a sequence's 33 shows, which the last part asserts."""
-    from tq_kv_amd.parts import attention as A
+    from tq_kv_amd import POLICY
     raw = two_layer("qwen2.5:7b")
     tensors = sharpened(tensors_for(raw, 6))
     lens = [2100, 1990, 2048, 1500, 2111, 64, 1, 700]
@@ -188,12 +188,12 @@ def test_prompts_of_two_thousand_tokens_and_graphed_decoding_at_7b_sizes():
     f32, _ = run("float32")
     bf16, n_graphs = run("bfloat16")
     assert n_graphs >= 1                                   # the one-token steps went through captured graphs
-    old = dict(A.POLICY)
-    A.POLICY.update(decode_mfma=False, prefill_mfma=False)
+    old = dict(POLICY.items())
+    POLICY.update(decode_mfma=False, prefill_mfma=False)
     try:
         bf16_plain_kernel, _ = run("bfloat16")
     finally:
-        A.POLICY.update(old)
+        POLICY.update(old)
     rms, worst = row_errors(bf16, f32)
     assert rms.max().item() < 0.07 and worst.max().item() < 0.35, (rms.max().item(), worst.max().item())
     rms, worst = row_errors(bf16, bf16_plain_kernel)
@@ -245,25 +245,28 @@ def test_a_model_without_weight_rows_gives_the_same_results(shape):
     128 tokens go through the kernel for 17 to 128 rows in pieces.  Steps of up to 128 rows run the
     same kernels either way (equal bit for bit); a prompt of 300 tokens is compared with the plain
     implementation as the other bfloat16 runs here are."""
-    from tq_kv_amd.parts import linear as L
+    from tq_kv_amd import POLICY
     raw = two_layer(shape)
     tensors = sharpened(tensors_for(raw, 6))
     prompts = [helpers.random_tokens(n, raw["vocab_size"], 70 + i) for i, n in enumerate([300, 100, 20])]
     outs, held = {}, {}
     for keep in (True, False):
         torch.cuda.empty_cache()
-        before = torch.cuda.memory_allocated()
-        old = L.POLICY["keep_rows"]
-        L.POLICY["keep_rows"] = keep
+        torch.cuda.synchronize()
+        before = torch.cuda.mem_get_info()[0]         # the model's memory is the engine library's, not torch's
+        old = POLICY["keep_rows"]
+        POLICY["keep_rows"] = keep
         try:
             model = build(raw, "bfloat16", tensors)
         finally:
-            L.POLICY["keep_rows"] = old
-        held[keep] = torch.cuda.memory_allocated() - before
-        mixer, ffn = model.blocks[0].mixer, model.blocks[0].feed_forward
-        for w in (mixer.w_qkv, mixer.w_o, ffn.w_gate_up, ffn.w_down):
-            assert torch.is_tensor(w) == keep
-        assert torch.is_tensor(model.head) == (keep or bool(raw.get("tie_word_embeddings")))
+            POLICY["keep_rows"] = old
+        torch.cuda.synchronize()
+        held[keep] = before - torch.cuda.mem_get_info()[0]
+        for name in ("self_attn.qkv.weight", "self_attn.o_proj.weight", "mlp.gate_up.weight", "mlp.down_proj.weight"):
+            assert model.holds("model.layers.0." + name) == keep and model.holds("model.layers.0." + name + ".packed")
+        if not raw.get("tie_word_embeddings"):
+            assert model.holds("lm_head.weight") == keep
+        assert model.holds("model.embed_tokens.weight") and model.holds("head.packed")
         eng = Engine(model, max_tokens=1024)
         slots = [eng.open() for _ in prompts]
         got = [eng.step([(slots[0], prompts[0], [0, 127, 128, 299])]),
@@ -278,8 +281,7 @@ def test_a_model_without_weight_rows_gives_the_same_results(shape):
     for keep in (True, False):
         rms, worst = row_errors(outs[keep][0], want)
         assert rms.max().item() < 0.07 and worst.max().item() < 0.35, (keep, rms, worst)
-    # what is given back: the rows of every packed weight.  Here that shows for the weights the parts
-    # had put together themselves (q/k/v and gate/up); the others' rows are this test's own tensors.
+    # what is given back: the rows of every packed weight (all the products' weights, and an untied head)
     rows = sum(v.numel() * 2 for k, v in tensors.items()
-               if k.endswith(".weight") and any(p in k for p in ("q_proj", "k_proj", "v_proj", "gate_proj", "up_proj")))
-    assert abs((held[True] - held[False]) - rows) < 0.02 * rows, (held, rows)
+               if k.endswith("_proj.weight") or k == "lm_head.weight")
+    assert abs((held[True] - held[False]) - rows) < 0.05 * rows + (8 << 20), (held, rows)

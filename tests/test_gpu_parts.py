@@ -51,7 +51,15 @@ def test_rotary_part_tables():
     rot = env.build("position", PartSpec("rotary", {"theta": 1e6, "rot_dim": 48, "max_positions": 300, "style": "halves"}))
     cos, sin, rot_dim, _ = rot.tables()
     c, s = plain.rope_tables(48, 1e6, 300)
-    assert rot_dim == 48 and torch.equal(cos.cpu(), c) and torch.equal(sin.cpu(), s)
+    # the engine takes the float32 power, cosine and sine from the C library (as the reference's Rust does), the plain
+    # implementation from torch: where the two round theta_j differently by one unit in the last place, the angle at
+    # position p differs by p * 6e-8 * theta_j, which is all that this allowance covers (a wrong base, pairing or
+    # position would be off by far more)
+    assert rot_dim == 48 and cos.shape == c.shape
+    torch.testing.assert_close(cos.cpu(), c, atol=300 * 6e-8 + 2e-7, rtol=0)
+    torch.testing.assert_close(sin.cpu(), s, atol=300 * 6e-8 + 2e-7, rtol=0)
+    assert torch.equal(cos[0].cpu(), torch.ones(24)) and torch.equal(sin[0].cpu(), torch.zeros(24))
+    torch.testing.assert_close(cos[:, 0].cpu(), c[:, 0], atol=2e-7, rtol=0)         # theta_0 = 1: the angle is the position itself
     with pytest.raises(ValueError):
         env.build("position", PartSpec("rotary", {"theta": 1e4, "rot_dim": 7, "max_positions": 8}))
 
@@ -525,17 +533,23 @@ def test_embedding_scale_positions_on_the_stream_head_bias_and_logit_scale_and_c
         stream_position=PartSpec("toy_learned", {"hidden": h, "max_positions": cfg["max_position_embeddings"]}),
         stream_position_prefix="model.positions.", head_bias_name="lm_head.bias", logit_scale=0.5, logit_cap=0.75)
     model = Model(spec, dtype, DEV)
-    assert {"model.positions.weight", "lm_head.bias"} <= set(model.tensor_specs()) and model.graph_safe
+    assert {"model.positions.weight", "lm_head.bias"} <= set(model.tensor_specs()) and not model.graph_safe
     std = {"model.positions.weight": 0.5, "lm_head.bias": 1.0, "model.embed_tokens.weight": 0.1}
     specs = {n: TensorSpec(s.shape, s.init, std.get(n, 0.08) if s.init == "normal" else 0.1) for n, s in model.tensor_specs().items()}
     w = random_tensors(specs, 12, DT[dtype], "cpu")
     model.load({k: v.to(DEV) for k, v in w.items()})
+    bare = Model(dataclasses.replace(spec, stream_position=None), dtype, DEV)
+    assert bare.graph_safe
+    bare.load({k: v.to(DEV) for k, v in w.items() if k != "model.positions.weight"})
     w = {k: v.float() for k, v in w.items()}
     eps = cfg["rms_norm_eps"]
+    with_positions = [True]
 
     def plain_forward(tokens):
         t = len(tokens)
-        x = w["model.embed_tokens.weight"][tokens] * (float(h) ** 0.5) + w["model.positions.weight"][:t]
+        x = w["model.embed_tokens.weight"][tokens] * (float(h) ** 0.5)
+        if with_positions[0]:
+            x = x + w["model.positions.weight"][:t]
         nh, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
         for l in range(cfg["num_hidden_layers"]):
             p = "model.layers.%d." % l
@@ -548,9 +562,11 @@ def test_embedding_scale_positions_on_the_stream_head_bias_and_logit_scale_and_c
         logits = (plain.linear(plain.rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"]) + w["lm_head.bias"]) * 0.5
         return 0.75 * torch.tanh(logits / 0.75)
 
-    eng = Engine(model, max_tokens=1024)
     a, b = helpers.random_tokens(30, 256, 14), helpers.random_tokens(12, 256, 15)
-    for round_ in range(2):                               # the second round replays the graphs of the first
+    for round_ in range(4):                               # with positions twice, then without twice: the last round replays the graphs of the third
+        with_positions[0] = round_ < 2
+        if round_ in (0, 2):
+            eng = Engine(model if with_positions[0] else bare, max_tokens=1024)
         sa, sb = eng.open(), eng.open()
         out = eng.step([(sa, a[:20], list(range(20))), (sb, b[:5], list(range(5)))])
         got_a, got_b = [out[:20]], [out[20:]]
@@ -562,11 +578,11 @@ def test_embedding_scale_positions_on_the_stream_head_bias_and_logit_scale_and_c
             got_a.append(eng.step([(sa, [a[t]], [0])]))
         eng.close(sa)
         want_a, want_b = plain_forward(a), plain_forward(b)
-        assert want_a.abs().max() > 0.6 and want_a.abs().max() < 0.75          # the cap bites, and holds
+        assert want_a.abs().max() > 0.55 and want_a.abs().max() < 0.75         # the cap bites, and holds
         tol = dict(atol=2e-5, rtol=2e-5) if dtype == "float32" else dict(atol=0.1 * want_a.std().item(), rtol=0.02)
         torch.testing.assert_close(torch.cat(got_a).cpu(), want_a, **tol)
         torch.testing.assert_close(torch.cat(got_b).cpu(), want_b, **tol)
-    assert len(eng.graphs) >= 1
+        assert (len(eng.graphs) >= 1) == (round_ >= 2)
     with pytest.raises(ValueError, match="cannot act on the stream"):
         Model(dataclasses.replace(spec, stream_position=PartSpec("none", {})), dtype, DEV)
 

@@ -1,6 +1,7 @@
-"""The engine's host library under AddressSanitizer and UndefinedBehaviorSanitizer: built with
-them into a temporary folder, loaded in a child process in place of the ordinary build, and
-driven by the cache, step-plan and generation-loop tests (none of which needs a GPU)."""
+"""The engine library under AddressSanitizer and UndefinedBehaviorSanitizer: built with them into a
+temporary folder, loaded in a child process in place of the ordinary build, and driven by the tests
+that need no GPU: configuration, weights and their errors (models in host memory), the cache, the
+step's arrays, and the generation loop over stand-in engines and samplers."""
 import os
 import shutil
 import subprocess
@@ -13,9 +14,6 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CHILD = r"""
 import sys
 sys.path.insert(0, {root!r})
-import tq_kv_amd.csrc.build as build
-build.find_host_library = lambda: {lib!r}
-build.ensure_host_built = lambda *a, **k: {lib!r}
 import pytest
 rc = pytest.main(["-x", "-q", "-m", "not gpu", "-p", "no:cacheprovider"] + {tests!r})
 loaded = [line.split()[-1] for line in open("/proc/self/maps") if "tqengine" in line]
@@ -25,6 +23,7 @@ sys.exit(rc)
 
 
 def test_host_library_is_clean_under_address_and_ub_sanitizers(tmp_path):
+    from tq_kv_amd.csrc import build
     cxx = shutil.which("g++")
     if cxx is None:
         pytest.skip("no g++")
@@ -32,14 +31,15 @@ def test_host_library_is_clean_under_address_and_ub_sanitizers(tmp_path):
                 for n in ("libasan.so", "libubsan.so")]
     if not all(os.path.isabs(p) and os.path.exists(p) for p in runtimes):
         pytest.skip("this g++ has no sanitizer runtimes")
+    build.ensure_built(verbose=False)             # the kernel library (not sanitized) answers the engine's questions about sizes
     lib = str(tmp_path / "libtqengine_sanitized.so")
-    src = os.path.join(ROOT, "tq_kv_amd", "csrc", "host_engine.cpp")
-    built = subprocess.run([cxx, "-O1", "-g", "-fPIC", "-std=c++17", "-shared", "-Wall", "-fsanitize=address,undefined",
-                            "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer", src, "-o", lib], capture_output=True, text=True)
-    assert built.returncode == 0, built.stderr
-    tests = [os.path.join(ROOT, "tests", n) for n in ("test_cache.py", "test_step_plan.py", "test_generate_loop.py")]
-    env = dict(os.environ, LD_PRELOAD=" ".join(runtimes), ASAN_OPTIONS="detect_leaks=0:abort_on_error=1")
+    os.environ.setdefault("CXX", cxx)
+    build.compile_host(lib, extra_flags=["-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer"])
+    tests = [os.path.join(ROOT, "tests", n) for n in ("test_cache.py", "test_step_plan.py", "test_generate_loop.py", "test_config.py",
+                                                      "test_weights.py")]
+    env = dict(os.environ, LD_PRELOAD=" ".join(runtimes), ASAN_OPTIONS="detect_leaks=0:abort_on_error=1",
+               TQ_KERNEL_LIBRARY=build.find_library(), TQ_ENGINE_LIBRARY=lib)
     child = subprocess.run([sys.executable, "-c", CHILD.format(root=ROOT, lib=lib, tests=tests)], capture_output=True, text=True, env=env,
-                           timeout=600)
+                           timeout=900)
     assert child.returncode == 0, child.stdout[-3000:] + child.stderr[-3000:]
     assert "passed" in child.stdout and "ERROR: AddressSanitizer" not in child.stderr and "runtime error" not in child.stderr

@@ -52,6 +52,9 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     model = Model.from_config_dict(TINY_B, "float32", "cpu")
     with pytest.raises(WeightError) as e:
         load_folder(folder, model.tensor_specs(), torch.float32, "cpu")
+    with pytest.raises(WeightError) as whole:
+        Model.from_dir(folder, dtype="float32", device="cpu")               # the same error from the loader inside the library
+    assert str(whole.value) == str(e.value) and whole.value.missing == e.value.missing
     msg = str(e.value)
     assert "Missing tensor: model.layers.1.self_attn.k_proj.bias" in msg and "Missing tensor: lm_head.weight" in msg
     assert "Unexpected tensor: model.layers.2.rogue.weight" in msg
@@ -75,7 +78,7 @@ def test_tied_model_refuses_a_head_and_untied_needs_one(tmp_path):
     # what is missing or misshapen stays an error
     with pytest.warns(UserWarning, match="lm_head.weight"):
         got = Model.from_dir(folder, dtype="float32", device="cpu", strict=False)
-    assert got.head is got.embedding
+    assert got.head_is_embedding and not got.holds("lm_head.weight")
     del t["model.norm.weight"]
     save_file(t, path)
     with pytest.raises(WeightError, match="Missing tensor: model.norm.weight") as e:
@@ -101,6 +104,16 @@ def test_dtype_policy(tmp_path):
     got = load_folder(folder, model.tensor_specs(), f32, "cpu")
     assert all(v.dtype == f32 for v in got.values())
     assert torch.equal(got["model.embed_tokens.weight"], t["model.embed_tokens.weight"].to(f32))
+    # and what the library's own loader keeps, in host memory here
+    kept = Model.from_dir(folder, dtype="bfloat16", device="cpu")
+    assert kept.tensor("model.norm.weight").dtype == f32 and torch.equal(kept.tensor("model.norm.weight"), t["model.norm.weight"])
+    assert kept.tensor("model.embed_tokens.weight").dtype == bf
+    assert torch.equal(kept.tensor("model.embed_tokens.weight"), t["model.embed_tokens.weight"])
+    kept = Model.from_dir(folder, dtype="float32", device="cpu")
+    assert torch.equal(kept.tensor("model.embed_tokens.weight"), t["model.embed_tokens.weight"].to(f32))
+    assert torch.equal(kept.tensor("model.layers.1.mlp.down_proj.weight"), t["model.layers.1.mlp.down_proj.weight"].to(f32))
+    qkv = torch.cat([t["model.layers.0.self_attn.%s_proj.weight" % x] for x in "qkv"]).to(f32)
+    assert torch.equal(kept.tensor("model.layers.0.self_attn.qkv.weight"), qkv)
 
 
 def test_random_folder_is_seeded_and_has_the_stated_distributions(tmp_path):
@@ -127,7 +140,7 @@ def test_random_stream_is_a_function_of_key_and_index_alone():
     """Element i is the same whatever piece of the stream is asked for; the values are standard
     normal (moments and a Kolmogorov-Smirnov distance), bounded by sqrt(48 ln 2), never NaN."""
     import numpy as np
-    from tq_kv_amd.weights.random_init import standard_normal_host, tensor_key
+    from tq_kv_amd.weights import standard_normal_host, tensor_key
     key = tensor_key(3, "model.embed_tokens.weight")
     assert key == tensor_key(3, "model.embed_tokens.weight") != tensor_key(4, "model.embed_tokens.weight")
     whole = standard_normal_host(key, 0, 5000)

@@ -7,10 +7,11 @@ seeded random-weights shape to generated tokens on one GPU.
     engine = Engine(model, max_tokens=4096)
     out = generate(engine, [[1, 2, 3]], GenerationParams(max_tokens=8, temperature=0.0))
 """
-from . import architectures  # noqa: F401  (registers the architectures)
+from . import architectures  # noqa: F401  (the typed configurations as Python sees them)
 from .config import ConfigError
 from .engine import Engine, GenerationError, Model, StepError, generate
+from .policy import POLICY
 from .sampling import GenerationParams
 
-__all__ = ["Model", "Engine", "StepError", "ConfigError", "GenerationError", "GenerationParams", "generate"]
+__all__ = ["Model", "Engine", "StepError", "ConfigError", "GenerationError", "GenerationParams", "generate", "POLICY"]
 __version__ = "0.1.0"

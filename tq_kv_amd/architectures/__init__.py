@@ -1,5 +1,3 @@
-"""Architectures: each file registers a configuration class and a ModelSpec builder."""
-from ..config.registry import register_architecture
-from . import qwen2
-
-register_architecture("Qwen2ForCausalLM", qwen2.Qwen2Config, qwen2.build_spec, model_types=("qwen2",))
+"""Architectures: the Python mirrors of their typed configurations (the architectures themselves
+are registered in the engine library, one file each under csrc/engine/)."""
+from . import qwen2  # noqa: F401

@@ -1,4 +1,3 @@
-from .pages import CacheFull
-from .store import PAGE, Cache, KVEntry, StateEntry
+from .store import PAGE, Cache, CacheFull, Entry
 
-__all__ = ["CacheFull", "PAGE", "Cache", "KVEntry", "StateEntry"]
+__all__ = ["CacheFull", "PAGE", "Cache", "Entry"]

@@ -1,66 +1,55 @@
-"""The cache: a slot for each live sequence, keys and values for each cached run of
-the order, fixed-size state beside them.
+"""The cache as Python sees it: a slot for each live sequence, keys and values for each cached
+run of the order, fixed-size state beside them.
 
-Runs of the order with the same need (same kv heads, head size and window) form a
-group.  A group has storage of its own: one pool of pages of PAGE positions,
+Runs of the order with the same need form a group.  A group of pages has storage of its own,
 
-    keys:   [runs in group, pages, kv heads, PAGE, head_dim]
-    values: [runs in group, pages, kv heads, head_dim, PAGE]   (transposed inside a page:
-            the attention kernels read 8 consecutive positions of one element at once)
+    keys:   [runs in group, pages, key page...]      values: [runs in group, pages, value page...]
 
-and, per slot, the list of pages that hold the slot's positions.  A group with a
-window gives pages back as soon as every position in them has left the window; a
-group without keeps them until the slot is released.  Mixers with a fixed-size
-state get one float32 row per slot, zeroed when the slot is taken.
+(what a page looks like inside is the mixer's business: its need names the two shapes; the
+attention kernels' pages are keys [kv heads, PAGE, head_dim] and values [kv heads, head_dim,
+PAGE], transposed inside a page) and, per slot, the list of pages that hold the slot's positions.
+A group with a window gives pages back as soon as every position in them has left the window.
+Mixers with a fixed-size state get one row per slot, zeroed when the slot is taken.
 
-The bookkeeping (free slots, lengths, page lists) is the engine's host library's
-(csrc/host_engine.cpp behind the C boundary csrc/tq_engine.h); the classes here own the
-storage tensors and show the bookkeeping to Python.
+Storage and bookkeeping are the engine library's (csrc/engine/store.cpp, csrc/host_engine.cpp);
+the classes here hold its handle and show its memory as torch tensors (views, no copies).
 
 The reference keeps one growing tensor pair per layer and one sequence
-(src/models/turbo_generic.rs:1606-1618) and resets by position
-(src/engine.rs:322-324); lengths after prompt(8), +1, +1 are 8, 9, 10 as in
-tq-kv/src/candle_kv.rs:266-299.
+(src/models/turbo_generic.rs:1606-1618) and resets by position (src/engine.rs:322-324); lengths
+after prompt(8), +1, +1 are 8, 9, 10 as in tq-kv/src/candle_kv.rs:266-299.
 """
+import json
+
 import numpy as np
-import torch
 
 from .. import native
-from ..parts.spec import KVNeed, StateNeed
-from .pages import CacheFull
+from ..native import CacheFull
+from ..parts.spec import need_from_json, need_to_json
 
-PAGE = 64
+PAGE = native.page_size()
 
 
 def pages_for(n_positions):
     return (n_positions + PAGE - 1) // PAGE
 
 
-class KVEntry:
-    """What an attention-like mixer sees of the cache for one run of the order."""
+class Entry:
+    """What a mixer sees of the cache for one run of the order."""
 
-    def __init__(self, group, index, writes):
-        self.group = group
-        self.keys = group.keys[index]
-        self.values = group.values[index]
-        self.writes = writes          # False: reads another run's cache
+    def __init__(self, cache, run, group, index, writes):
+        self.cache, self.run, self.group, self.writes = cache, run, group, writes
+        if isinstance(group, KVGroup):
+            self.keys, self.values = group.keys[index], group.values[index]
+        else:
+            self.state = group.state[index]
 
     @property
     def need(self):
         return self.group.need
 
 
-class StateEntry:
-    """What a mixer with fixed-size state sees: state[slot] is its sequence's row."""
-
-    def __init__(self, group, index, writes):
-        self.group = group
-        self.state = group.state[index]
-        self.writes = writes
-
-
 class _PoolView:
-    """Free and held counts of a pool of the native cache (the slots, or a group's pages)."""
+    """Free and held counts of a pool of the bookkeeping (the slots, or a group's pages)."""
 
     def __init__(self, cache, group):
         self._cache, self._group = cache, group
@@ -85,7 +74,7 @@ class _PoolView:
 
 
 class _PagesView:
-    """slot -> list of page ids (-1 where given back) of a group, read from the native cache."""
+    """slot -> list of page ids (-1 where given back) of a group, read from the bookkeeping."""
 
     def __init__(self, cache, group):
         self._cache, self._group = cache, group
@@ -110,15 +99,21 @@ class _PagesView:
         return [self[s] for s in self]
 
 
+def _tensor(info, on_gpu, keep):
+    return native.view(info["data"], {"float32": native.F32, "bfloat16": native.BF16, "int32": native.I32}[info["dtype"]], info["shape"],
+                       on_gpu, keep=keep)
+
+
 class KVGroup:
-    def __init__(self, need, runs, n_pages, dtype, device):
-        self.need = need
-        self.runs = list(runs)
-        self.n_pages = n_pages
-        shape = (len(self.runs), n_pages, need.n_kv_heads, PAGE, need.head_dim)
-        self.keys = torch.zeros(shape, dtype=dtype, device=device)
-        self.values = torch.zeros(shape[:3] + (need.head_dim, PAGE), dtype=dtype, device=device)
-        self.pool = self.pages = None      # views of the native bookkeeping, set by the cache
+    def __init__(self, index, info, book, on_gpu, keep):
+        self.index = index
+        self.need = need_from_json(info["need"])
+        self.runs = list(info["runs"])
+        self.n_pages = info["n_pages"]
+        self.keys = _tensor(info["keys"], on_gpu, keep)
+        self.values = _tensor(info["values"], on_gpu, keep)
+        self.pool = _PoolView(book, index)
+        self.pages = _PagesView(book, index)
 
     def first_needed(self, length):
         """First position a query at or after `length` can still see."""
@@ -127,90 +122,77 @@ class KVGroup:
         return max(0, length + 1 - self.need.window)
 
 
-STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
-
-
 class StateGroup:
-    def __init__(self, need, runs, n_slots, device):
-        self.need = need
-        self.runs = list(runs)
-        if need.dtype not in STATE_DTYPES:
-            raise TypeError("state of kind %r (known: %s)" % (need.dtype, ", ".join(sorted(STATE_DTYPES))))
-        self.state = torch.zeros((len(self.runs), n_slots) + tuple(need.shape),
-                                 dtype=STATE_DTYPES[need.dtype], device=device)
-
-    def reset(self, slot):
-        self.state[:, slot].zero_()
+    def __init__(self, info, on_gpu, keep):
+        self.need = need_from_json(info["need"])
+        self.runs = list(info["runs"])
+        self.state = _tensor(info["state"], on_gpu, keep)
 
 
 class Cache:
     """Slots, lengths, page tables and storage for all groups of one model.
 
-    needs: for each run of the order its need (KVNeed, StateNeed or None).
-    cache_of: for each run None, or the index of the run whose cache it reads.
-    max_tokens: positions that live sequences may hold together, each sequence
-    counted up to a multiple of PAGE.
+    needs: for each run of the order its need (KVNeed, StateNeed or None).  cache_of: for each run
+    None, or the index of the run whose cache it reads.  max_tokens: positions that live sequences
+    may hold together, each sequence counted up to a multiple of PAGE.  An engine's cache is shown
+    through the same class (of_engine).
     """
 
-    def __init__(self, needs, cache_of, max_tokens, max_slots, dtype, device):
-        # pages bound the cache only where some run keeps keys and values: a model whose runs all
-        # keep fixed-size state (or nothing) is bounded by its slots alone
-        self.holds_pages = any(isinstance(need, KVNeed) and cache_of[run] is None for run, need in enumerate(needs))
-        if self.holds_pages and max_tokens < PAGE:
-            raise ValueError("max_tokens must be at least %d, got %d" % (PAGE, max_tokens))
-        self.n_pages = max_tokens // PAGE if self.holds_pages else 0
-        self.max_slots = max(1, min(int(max_slots), self.n_pages)) if self.holds_pages else max(1, int(max_slots))
-        self.device = device
-        self.kv_groups = []
-        self.state_groups = []
-        self._entry = {}              # run index -> (group, index within group)
-        by_need = {}
-        for run, need in enumerate(needs):
-            if need is None or cache_of[run] is not None:
-                continue
-            by_need.setdefault(need, []).append(run)
-        for need, runs in by_need.items():
-            if isinstance(need, KVNeed):
-                group = KVGroup(need, runs, self.n_pages, dtype, device)
-                self.kv_groups.append(group)
-            elif isinstance(need, StateNeed):
-                group = StateGroup(need, runs, self.max_slots, device)
-                self.state_groups.append(group)
-            else:
-                raise TypeError("unknown cache need %r" % (need,))
-            for i, run in enumerate(runs):
-                self._entry[run] = (group, i)
-        if len(self.kv_groups) > native.MAX_GROUPS:
-            raise ValueError("%d groups of cached runs, the engine's library takes %d" % (len(self.kv_groups), native.MAX_GROUPS))
-        # the bookkeeping: free slots, lengths, page lists
-        self.native = native.NativeCache(self.max_slots, [(g.n_pages, g.need.window) for g in self.kv_groups])
+    def __init__(self, needs, cache_of, max_tokens, max_slots, dtype, device, _engine=None):
+        import torch
+        import weakref
+        self._lib = native.library()
+        self._engine = weakref.proxy(_engine) if _engine is not None else None      # the engine owns its cache, not the other way round
+        self.device = torch.device(device)
+        self.on_gpu = self.device.type == "cuda"
+        if _engine is None:
+            co = np.ascontiguousarray([-1 if c is None else int(c) for c in cache_of], dtype=np.int32)
+            self.handle = native.handle(self._lib.tqe_store_new(
+                native.enc(json.dumps([need_to_json(n) for n in needs])), co.ctypes.data_as(native._I32P), len(needs), int(max_tokens),
+                int(max_slots), native.dtype_code(dtype), 1 if self.on_gpu else 0))
+            info = native.parsed(self._lib.tqe_store_describe(self.handle))
+            book = self._lib.tqe_store_cache(self.handle)
+        else:
+            self.handle = None
+            info = native.parsed(self._lib.tqe_engine_describe(_engine.handle))
+            book = self._lib.tqe_engine_cache(_engine.handle)
+        self.holds_pages = bool(info["holds_pages"])
+        self.n_pages = info["n_pages"]
+        self.max_slots = info["max_slots"]
+        self.native = native.NativeCache(self.max_slots, [(g["n_pages"], g["need"].get("window")) for g in info["page_groups"]], handle=book)
+        self.kv_groups = [KVGroup(i, g, self.native, self.on_gpu, None) for i, g in enumerate(info["page_groups"])]
+        self.state_groups = [StateGroup(g, self.on_gpu, None) for g in info["state_groups"]]
         self.slots = _PoolView(self.native, -1)
-        for i, g in enumerate(self.kv_groups):
-            g.index = i
-            g.pool = _PoolView(self.native, i)
-            g.pages = _PagesView(self.native, i)
         self._views = {}
-        for run, need in enumerate(needs):
-            src = cache_of[run]
-            if need is None:
+        n_runs = len(needs)
+        for run in range(n_runs):
+            if needs[run] is None:
                 self._views[run] = None
                 continue
-            owner = run if src is None else src
-            if owner not in self._entry:
-                raise ValueError("run %d reads the cache of run %d, which keeps none" % (run, owner))
-            group, i = self._entry[owner]
-            if src is not None and group.need != need:
-                raise ValueError("run %d needs %r but run %d's cache is %r" % (run, need, owner, group.need))
-            cls = KVEntry if isinstance(group, KVGroup) else StateEntry
-            self._views[run] = cls(group, i, writes=(src is None))
+            owner = run if cache_of[run] is None else cache_of[run]
+            for group in self.kv_groups + self.state_groups:
+                if owner in group.runs:
+                    self._views[run] = Entry(self, run, group, group.runs.index(owner), cache_of[run] is None)
+
+    @classmethod
+    def of_engine(cls, engine, needs, cache_of, dtype, device):
+        return cls(needs, cache_of, 0, 0, dtype, device, _engine=engine)
+
+    def __del__(self):
+        h, self.handle = getattr(self, "handle", None), None
+        if h:
+            self.kv_groups = self.state_groups = []
+            self._lib.tqe_store_free(h)
 
     # -- slots ------------------------------------------------------------
     def acquire(self):
         """A free slot with length 0 and zeroed state."""
-        slot = self.native.acquire()
-        for g in self.state_groups:
-            g.reset(slot)
-        return slot
+        import ctypes
+        if self._engine is not None:
+            return self._engine.open()
+        slot = ctypes.c_int32(-1)
+        native.check(self._lib.tqe_store_acquire(self.handle, ctypes.byref(slot), native.current_stream() if self.on_gpu else None))
+        return slot.value
 
     def release(self, slot):
         """Give the slot and everything it holds back."""

@@ -69,8 +69,6 @@ def build_parser():
     b.add_argument("-n", "--tokens", type=int, default=100, help="Number of tokens to generate per run")
     b.add_argument("--prompt-len", type=int, default=32, help="Length of the random prompt")
     b.add_argument("--json", action="store_true", help="Output results as JSON")
-    b.add_argument("--tune", action="store_true",
-                   help="Let the matrix library try its kernels for the prompt's size first (takes some seconds)")
     r = sub.add_parser("replay", help="Replay a trace of steps from standard input and write logits")
     r.add_argument("--model", required=True)
     r.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
@@ -90,8 +88,8 @@ def load_model(name, dtype, weights_seed, strict=True, packed_only=False):
     from .config import catalog
     from .engine import Model
     if packed_only:
-        from .parts import linear
-        linear.POLICY["keep_rows"] = False
+        from .policy import POLICY
+        POLICY["keep_rows"] = False
     if os.path.isdir(name):
         return Model.from_dir(name, dtype=dtype, strict=strict)
     if catalog.find(name) is None:
@@ -163,8 +161,6 @@ def cmd_bench(args):
     prompt = torch.randint(0, model.spec.vocab_size, (args.prompt_len,), generator=g).tolist()
     engine = Engine(model, max_tokens=args.max_cache_tokens or (args.prompt_len + args.tokens + 2 * PAGE) // PAGE * PAGE)
     params = GenerationParams(max_tokens=args.tokens, temperature=0.0, repeat_penalty=1.0)
-    if args.tune:
-        model.tune_library(len(prompt))
     generate(engine, [prompt], GenerationParams(max_tokens=4, temperature=0.0, repeat_penalty=1.0))      # warm-up
     marks = []
     torch.cuda.synchronize()

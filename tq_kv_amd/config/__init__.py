@@ -1,6 +1,6 @@
-from .base import ConfigError, KeyReader, read_config_json
-from .registry import (architecture_name, config_from_dict, known_architectures, load_config,
-                       register_architecture, spec_for)
+from . import catalog
+from .base import ConfigError, read_config_json
+from .registry import config_from_dict, known_architectures, load_config, spec_for, spec_from_dict
 
-__all__ = ["ConfigError", "KeyReader", "read_config_json", "architecture_name", "config_from_dict",
-           "known_architectures", "load_config", "register_architecture", "spec_for"]
+__all__ = ["catalog", "ConfigError", "read_config_json", "config_from_dict", "known_architectures", "load_config", "spec_for",
+           "spec_from_dict"]

@@ -94,6 +94,8 @@ void attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ key
     }
 }
 
+extern "C" int tqk_attention_max_head_dim(void) { return ATT_MAX_D; }
+
 extern "C" int tqk_attention(const void* q, const void* keys, const void* values, int act_dtype,
                              const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* page_table,
                              int table_width, int n_seqs, int n_pages, int window, float scale, void* out,

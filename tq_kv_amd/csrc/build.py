@@ -18,12 +18,20 @@ import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["host.cpp", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip",
-           "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip", "random_init.hip"]
+           "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip", "random_init.hip", "utility.hip"]
 HEADERS = ["common.h", "tq_kernels.h"]
-# the engine's host side: no GPU code, built with the host compiler into a library of its own
-HOST_SOURCES = ["host_engine.cpp"]
-HOST_HEADERS = ["tq_engine.h"]
-HOST_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-shared", "-Wall"]
+# the engine: host code only (config, weights, parts, model, cache, step, loop), built with the host compiler into a
+# library of its own that reaches the GPU through the HIP runtime, hipBLASLt and the kernel library above
+HOST_SOURCES = ["host_engine.cpp"] + ["engine/" + n for n in (
+    "api.cpp", "config.cpp", "core.cpp", "engine.cpp", "generate.cpp", "json.cpp", "linear.cpp", "model.cpp", "parts_builtin.cpp",
+    "plugin.cpp", "qwen2.cpp", "spec.cpp", "step.cpp", "store.cpp", "trace.cpp", "weights.cpp")]
+HOST_HEADERS = ["tq_engine.h"] + ["engine/" + n for n in (
+    "config.h", "core.h", "engine.h", "generate.h", "json.h", "kernels.h", "linear.h", "model.h", "parts.h", "plugin.h", "spec.h",
+    "step.h", "store.h", "trace.h", "weights.h")]
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+# no contraction of a multiplication with the addition after it: the random weights' recipe needs each rounded on its own
+HOST_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-Wall", "-ffp-contract=off", "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(ROCM, "include")]
+HOST_LINK = ["-shared", "-L" + os.path.join(ROCM, "lib"), "-Wl,-rpath," + os.path.join(ROCM, "lib"), "-lamdhip64", "-lhipblaslt", "-ldl", "-lpthread"]
 ARCH = "gfx950"
 # Packed float32 instructions are switched off for all device code.
 HIPCC_FLAGS = ["-O3", "-fPIC", "-std=c++17", "--offload-arch=" + ARCH,
@@ -62,7 +70,7 @@ def host_source_hash():
         with open(os.path.join(HERE, name), "rb") as f:
             h.update(name.encode())
             h.update(f.read())
-    h.update(" ".join(HOST_FLAGS).encode())
+    h.update(" ".join(HOST_FLAGS + HOST_LINK).encode())
     return h.hexdigest()[:12]
 
 
@@ -95,6 +103,10 @@ def find_library():
 
 
 def find_host_library():
+    """Path of a built engine library that matches the sources, or None.  TQ_ENGINE_LIBRARY names another build of it outright (a
+    sanitizer build, for instance)."""
+    if os.environ.get("TQ_ENGINE_LIBRARY"):
+        return os.environ["TQ_ENGINE_LIBRARY"]
     name = host_library_name()
     for folder in (HERE, _fallback_dir()):
         path = os.path.join(folder, name)
@@ -120,10 +132,7 @@ def build_host(force=True, verbose=True):
         raise BuildError("cannot write the engine library to %s or %s" % (HERE, out_dir))
     target = os.path.join(out_dir, host_library_name())
     tmp = target + ".tmp%d" % os.getpid()
-    cmd = [_host_compiler()] + HOST_FLAGS + ["-I", HERE] + [os.path.join(HERE, n) for n in HOST_SOURCES] + ["-o", tmp]
-    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if proc.returncode != 0:
-        raise BuildError("the host compiler failed on %s:\n%s" % (", ".join(HOST_SOURCES), proc.stdout))
+    compile_host(tmp, verbose=verbose)
     os.replace(tmp, target)
     for name in os.listdir(out_dir):
         if name.startswith("libtqengine_") and name.endswith(".so") and name != os.path.basename(target):
@@ -133,6 +142,45 @@ def build_host(force=True, verbose=True):
                 pass
     if verbose:
         print("[tq_kv_amd build] built %s" % target, file=sys.stderr, flush=True)
+    return target
+
+
+def compile_host(target, extra_flags=(), obj_dir=None, verbose=False):
+    """Compile the engine's sources (in parallel) and link them into `target`.  extra_flags: more compiler and linker
+    flags (a sanitizer build).  Objects go to obj_dir (default: a folder beside the target that is removed afterwards)."""
+    cxx = _host_compiler()
+    own = obj_dir is None
+    if own:
+        obj_dir = tempfile.mkdtemp(prefix="tq_host_obj_", dir=os.path.dirname(os.path.abspath(target)))
+    os.makedirs(obj_dir, exist_ok=True)
+    errors, objects, threads = [], [], []
+    gate = threading.Semaphore(max(1, min(8, os.cpu_count() or 1)))
+
+    def compile_one(src, obj):
+        with gate:
+            proc = subprocess.run([cxx] + HOST_FLAGS + list(extra_flags) + ["-I", HERE, "-c", os.path.join(HERE, src), "-o", obj],
+                                  stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0:
+            errors.append("the host compiler failed on %s:\n%s" % (src, proc.stdout))
+
+    try:
+        for src in HOST_SOURCES:
+            obj = os.path.join(obj_dir, src.replace("/", "_").rsplit(".", 1)[0] + ".o")
+            objects.append(obj)
+            th = threading.Thread(target=compile_one, args=(src, obj))
+            th.start()
+            threads.append(th)
+        for th in threads:
+            th.join()
+        if errors:
+            raise BuildError(errors[0])
+        proc = subprocess.run([cxx] + list(extra_flags) + objects + HOST_LINK + ["-o", target], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                              text=True)
+        if proc.returncode != 0:
+            raise BuildError("linking the engine library failed:\n%s" % proc.stdout)
+    finally:
+        if own:
+            shutil.rmtree(obj_dir, ignore_errors=True)
     return target
 
 

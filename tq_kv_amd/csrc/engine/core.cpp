@@ -1,0 +1,232 @@
+#include "core.h"
+
+#include <dlfcn.h>
+#include <glob.h>
+#include <hip/hip_runtime_api.h>
+#include <stdlib.h>
+
+#include <algorithm>
+#include <mutex>
+
+namespace tq {
+
+std::string format(const char* fmt, ...) {
+    char buf[2048];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    return buf;
+}
+
+void raise(int code, const char* fmt, ...) {
+    char buf[2048];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    throw Error(code, buf);
+}
+
+const char* dtype_name(int dt) { return dt == F32 ? "float32" : dt == BF16 ? "bfloat16" : dt == I32 ? "int32" : "?"; }
+
+std::string Tensor::describe() const {
+    std::string s = dtype_name(dtype);
+    s += " [";
+    for (int i = 0; i < ndim; ++i) s += format(i ? ", %lld" : "%lld", (long long)shape[i]);
+    return s + "]";
+}
+
+// ---- device ----------------------------------------------------------------------------------
+static thread_local bool g_null_device = false;
+bool null_device() { return g_null_device; }
+void set_null_device(bool on) { g_null_device = on; }
+
+void hip_check(int status, const char* what) {
+    if (status != hipSuccess) raise(TQE_ERR_DEVICE, "%s: %s", what, hipGetErrorString((hipError_t)status));
+}
+
+void* device_malloc(size_t bytes) {
+    void* p = nullptr;
+    if (g_null_device) {
+        p = calloc(1, bytes ? bytes : 1);
+        if (!p) raise(TQE_ERR_DEVICE, "out of host memory (%zu bytes)", bytes);
+        return p;
+    }
+    const hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) raise(TQE_ERR_DEVICE, "cannot allocate %zu bytes of device memory: %s", bytes, hipGetErrorString(e));
+    return p;
+}
+
+void device_free(void* p, bool null) {
+    if (!p) return;
+    if (null) { free(p); return; }
+    (void)hipFree(p);
+}
+
+void copy_to_device(void* dst, const void* src, size_t bytes, hipStream_t stream) {
+    if (!bytes) return;
+    if (g_null_device) { memcpy(dst, src, bytes); return; }
+    hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, stream), "copy to the device");
+}
+
+void copy_to_host(void* dst, const void* src, size_t bytes, hipStream_t stream) {
+    if (g_null_device) { if (bytes) memcpy(dst, src, bytes); return; }
+    if (bytes) hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, stream), "copy to the host");
+    hip_check(hipStreamSynchronize(stream), "waiting for the device");
+}
+
+void copy_on_device(void* dst, const void* src, size_t bytes, hipStream_t stream) {
+    if (!bytes) return;
+    if (g_null_device) { memmove(dst, src, bytes); return; }
+    hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, stream), "copy on the device");
+}
+
+void zero_device(void* dst, size_t bytes, hipStream_t stream) {
+    if (!bytes) return;
+    if (g_null_device) { memset(dst, 0, bytes); return; }
+    hip_check(hipMemsetAsync(dst, 0, bytes, stream), "clearing device memory");
+}
+
+void stream_synchronize(hipStream_t stream) {
+    if (g_null_device) return;
+    hip_check(hipStreamSynchronize(stream), "waiting for the device");
+}
+
+void device_synchronize() {
+    if (g_null_device) return;
+    hip_check(hipDeviceSynchronize(), "waiting for the device");
+}
+
+// ---- workspace -------------------------------------------------------------------------------
+static size_t round_up(size_t n, size_t to) { return (n + to - 1) / to * to; }
+
+void Workspace::reserve(size_t bytes) {
+    chunks_.clear();
+    chunks_.emplace_back();
+    chunks_.back().mem.allocate(round_up(std::max<size_t>(bytes, 256), 256));
+    step_ = 0;
+}
+
+size_t Workspace::capacity() const {
+    size_t n = 0;
+    for (const Chunk& c : chunks_) n += c.mem.bytes();
+    return n;
+}
+
+void Workspace::reset(hipStream_t stream) {
+    if (chunks_.size() > 1 && !fixed_) {
+        // what the last step needed, in one piece: first let that step finish
+        const size_t want = capacity() + capacity() / 4;
+        stream_synchronize(stream);
+        reserve(want);
+    }
+    for (Chunk& c : chunks_) c.used = 0;
+    step_ = 0;
+}
+
+void* Workspace::alloc(size_t bytes) {
+    bytes = round_up(std::max<size_t>(bytes, 1), 256);
+    if (chunks_.empty() || chunks_.back().used + bytes > chunks_.back().mem.bytes()) {
+        if (fixed_ && !chunks_.empty())
+            raise(TQE_ERR_DEVICE, "a captured step's workspace of %zu bytes is too small (%zu more asked for)", capacity(), bytes);
+        const size_t grow = std::max(bytes, std::max<size_t>(capacity(), (size_t)8 << 20));
+        chunks_.emplace_back();
+        chunks_.back().mem.allocate(grow);
+    }
+    Chunk& c = chunks_.back();
+    void* p = (char*)c.mem.data() + c.used;
+    c.used += bytes;
+    step_ += bytes;
+    high_ = std::max(high_, step_);
+    return p;
+}
+
+// ---- staging ---------------------------------------------------------------------------------
+Staging::Staging(int depth) : slots_((size_t)depth) {}
+
+Staging::~Staging() {
+    for (Slot& s : slots_) {
+        if (s.event) { (void)hipEventSynchronize(s.event); (void)hipEventDestroy(s.event); }
+        if (s.host) (void)hipHostFree(s.host);
+    }
+}
+
+void Staging::upload(void* dst, const void* src, size_t n_bytes, hipStream_t stream) {
+    if (!n_bytes) return;
+    if (g_null_device) { memcpy(dst, src, n_bytes); return; }
+    Slot& s = slots_[(size_t)turn_];
+    turn_ = (turn_ + 1) % (int)slots_.size();
+    if (s.busy) { hip_check(hipEventSynchronize(s.event), "waiting for an upload"); s.busy = false; }
+    if (s.cap < n_bytes) {
+        if (s.host) hip_check(hipHostFree(s.host), "freeing pinned memory");
+        s.cap = std::max<size_t>(16384, 2 * n_bytes);
+        s.host = nullptr;
+        hip_check(hipHostMalloc(&s.host, s.cap, hipHostMallocDefault), "allocating pinned memory");
+    }
+    if (!s.event) hip_check(hipEventCreateWithFlags(&s.event, hipEventDisableTiming), "creating an event");
+    memcpy(s.host, src, n_bytes);
+    hip_check(hipMemcpyAsync(dst, s.host, n_bytes, hipMemcpyHostToDevice, stream), "uploading a step's arrays");
+    hip_check(hipEventRecord(s.event, stream), "recording an event");
+    s.busy = true;
+}
+
+// ---- the kernel library ------------------------------------------------------------------------
+static std::mutex g_kernel_mutex;
+static std::string g_kernel_path;
+static void* g_kernel_handle = nullptr;
+
+void set_kernel_library(const std::string& path) {
+    std::lock_guard<std::mutex> lock(g_kernel_mutex);
+    if (g_kernel_handle && path != g_kernel_path) { dlclose(g_kernel_handle); g_kernel_handle = nullptr; }
+    g_kernel_path = path;
+}
+
+static std::string find_kernel_library() {
+    if (const char* env = getenv("TQ_KERNEL_LIBRARY")) return env;
+    // beside this library: csrc/libtqkernels_<hash of its sources>.so
+    Dl_info info;
+    if (dladdr((void*)&find_kernel_library, &info) && info.dli_fname) {
+        std::string dir = info.dli_fname;
+        const size_t slash = dir.rfind('/');
+        dir = slash == std::string::npos ? "." : dir.substr(0, slash);
+        glob_t g;
+        std::string found;
+        if (glob((dir + "/libtqkernels_*.so").c_str(), 0, nullptr, &g) == 0) {
+            if (g.gl_pathc > 0) found = g.gl_pathv[g.gl_pathc - 1];
+            globfree(&g);
+        }
+        if (!found.empty()) return found;
+    }
+    return "";
+}
+
+std::string kernel_library_path() {
+    std::lock_guard<std::mutex> lock(g_kernel_mutex);
+    if (g_kernel_path.empty()) g_kernel_path = find_kernel_library();
+    return g_kernel_path;
+}
+
+void* kernel_symbol(const char* name) {
+    std::lock_guard<std::mutex> lock(g_kernel_mutex);
+    if (!g_kernel_handle) {
+        if (g_kernel_path.empty()) g_kernel_path = find_kernel_library();
+        if (g_kernel_path.empty())
+            throw Error(TQE_ERR_DEVICE, "the HIP kernel library is not built: no libtqkernels_*.so beside the engine library "
+                                        "(build it with tq_kv_amd/csrc/build.py, or name it in TQ_KERNEL_LIBRARY)");
+        g_kernel_handle = dlopen(g_kernel_path.c_str(), RTLD_NOW | RTLD_LOCAL);
+        if (!g_kernel_handle) throw Error(TQE_ERR_DEVICE, format("cannot load the HIP kernel library %s: %s", g_kernel_path.c_str(), dlerror()));
+    }
+    void* sym = dlsym(g_kernel_handle, name);
+    if (!sym) throw Error(TQE_ERR_DEVICE, format("the kernel library %s has no entry point %s (built from other sources?)", g_kernel_path.c_str(), name));
+    return sym;
+}
+
+void raise_kernel_error(const char* what) {
+    static KernelFn<const char*()> last("tqk_last_error");
+    const char* msg = last.raw();
+    const char* short_name = strncmp(what, "tqk_", 4) ? what : what + 4;
+    throw Error(TQE_ERR_KERNEL, format("%s: %s", short_name, msg ? msg : "failed"));
+}
+
+}  // namespace tq

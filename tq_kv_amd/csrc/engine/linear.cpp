@@ -1,0 +1,346 @@
+#include "linear.h"
+
+#include <hip/hip_runtime_api.h>
+#include <hipblaslt/hipblaslt.h>
+
+#include <algorithm>
+#include <mutex>
+
+#include "kernels.h"
+
+namespace tq {
+
+Policy& policy() {
+    static Policy p;
+    return p;
+}
+
+int* policy_field(const std::string& name) {
+    Policy& p = policy();
+    if (name == "skinny") return &p.skinny;
+    if (name == "library") return &p.library;
+    if (name == "fused") return &p.fused;
+    if (name == "prune_last") return &p.prune_last;
+    if (name == "packed") return &p.packed;
+    if (name == "mid") return &p.mid;
+    if (name == "keep_rows") return &p.keep_rows;
+    if (name == "decode_mfma") return &p.decode_mfma;
+    if (name == "prefill_mfma") return &p.prefill_mfma;
+    return nullptr;
+}
+
+int skinny_max_rows() {
+    static int n = K::skinny_max_rows.raw();
+    return n;
+}
+
+int mid_max_rows() {
+    static int n = K::mid_max_rows.raw();
+    return n;
+}
+
+OwnedPtr make_owned(int dtype, const std::vector<int64_t>& dims) {
+    OwnedPtr o = std::make_shared<Owned>();
+    o->t.dtype = dtype;
+    o->t.ndim = (int)dims.size();
+    if (dims.size() > 6) raise(TQE_ERR_ARGUMENT, "tensors of %zu dimensions are not supported (6 at most)", dims.size());
+    for (size_t i = 0; i < dims.size(); ++i) o->t.shape[i] = dims[i];
+    o->mem.allocate(o->t.bytes());
+    o->t.data = o->mem.data();
+    return o;
+}
+
+OwnedPtr make_owned(int dtype, std::initializer_list<int64_t> dims) { return make_owned(dtype, std::vector<int64_t>(dims)); }
+
+Weight make_weight(OwnedPtr rows, int parts, bool rows_needed, hipStream_t stream) {
+    Weight w;
+    const Tensor& t = rows->t;
+    if (t.ndim != 2) raise(TQE_ERR_WEIGHTS, "a product's weight must have two dimensions, got %s", t.describe().c_str());
+    w.n = t.shape[0];
+    w.k = t.shape[1];
+    w.parts = parts;
+    w.dtype = t.dtype;
+    w.rows = rows;
+    const Policy& p = policy();
+    if (p.packed && p.skinny && t.dtype == BF16 && !null_device() && w.k % 32 == 0 && w.n % parts == 0) {
+        const int64_t per = w.n / parts, tiles = (per + 15) / 16;
+        w.packed = make_owned(BF16, {parts * tiles, w.k / 32, 64, 8});
+        K::pack_weight(t.data, w.packed->t.data, (int)w.n, (int)w.k, parts, stream);
+        if (!p.keep_rows && !rows_needed && p.mid && p.skinny) {
+            stream_synchronize(stream);         // the packing kernel has read the rows
+            w.rows = nullptr;
+        }
+    }
+    return w;
+}
+
+bool fusable(int64_t x_rows, const Weight& w, bool adds) {
+    const Policy& p = policy();
+    return p.fused && p.skinny && x_rows <= skinny_max_rows() && w.dtype == BF16 && w.k % 32 == 0 && (!adds || w.n % 4 == 0);
+}
+
+bool leaves_sums(int64_t x_rows, const Weight& w) {
+    const Policy& p = policy();
+    return p.mid && w.packed && w.dtype == BF16 && x_rows > skinny_max_rows() && x_rows <= mid_max_rows();
+}
+
+void classify_step(StepContext& c, int64_t hidden) {
+    const Policy& p = policy();
+    c.fuse_small = p.fused && c.act_dtype == BF16 && c.all_decode && c.n_tokens <= skinny_max_rows() && hidden % 32 == 0;
+    c.fuse_mid = p.mid && c.act_dtype == BF16 && c.n_tokens > skinny_max_rows() && c.n_tokens <= mid_max_rows();
+}
+
+static bool skinny_ok(const Tensor& x, const Weight& w) {
+    return policy().skinny && x.dtype == BF16 && w.dtype == BF16 && x.shape[1] % 32 == 0 && x.shape[0] <= skinny_max_rows();
+}
+
+static bool mid_ok(const Tensor& x, const Weight& w) { return x.dtype == BF16 && leaves_sums(x.shape[0], w); }
+
+// pointer and packed flag of a product's weight for the few-row kernels
+static const void* few_ptr(const Weight& w, int* packed) {
+    if (w.packed) { *packed = 1; return w.packed->t.data; }
+    if (!w.rows) raise(TQE_ERR_STATE, "a weight has neither rows nor a packed copy");
+    *packed = 0;
+    return w.rows->t.data;
+}
+
+static void k_fused_store(StepContext& c, const Tensor& x, const int32_t* rows, const LazyNorm* norm, const Weight& w, Tensor& out) {
+    int packed = 0;
+    const void* wp = few_ptr(w, &packed);
+    K::fused_store(x.data, rows, norm ? (const float*)norm->ss.data : nullptr, norm ? norm->n_ss : 0, norm ? norm->eps : 0.f, wp, packed,
+                   out.data, out.dtype, (int)out.shape[0], (int)w.n, (int)w.k, c.stream);
+}
+
+static void k_fused_gated(StepContext& c, const Tensor& x, const LazyNorm* norm, const Weight& w, Tensor& out) {
+    int packed = 0;
+    const void* wp = few_ptr(w, &packed);
+    K::fused_gated(x.data, norm ? (const float*)norm->ss.data : nullptr, norm ? norm->n_ss : 0, norm ? norm->eps : 0.f, wp, packed, out.data,
+                   (int)out.shape[0], (int)w.n, (int)w.k, c.stream);
+}
+
+// the product through the kernel for mid-sized steps; leave: its sums where it cuts K into pieces
+static Product k_mid_store(StepContext& c, const Tensor& x, const Weight& w, int out_dtype, bool leave, Tensor* out) {
+    const int64_t m = x.shape[0];
+    const int splits = K::mid_splits.raw((int)w.n, (int)w.k, 0);
+    Product p;
+    Tensor scratch;
+    if (splits > 1) scratch = c.alloc(F32, {splits, m, w.n});
+    if (leave && splits > 1) {
+        K::mid_store(x.data, w.packed->t.data, nullptr, out_dtype, (int)m, (int)w.n, (int)w.k, scratch.data, 0, c.stream);
+        p.is_sums = true;
+        p.sums.sums = scratch;
+        p.sums.dtype = out_dtype;
+        return p;
+    }
+    p.t = out ? *out : c.alloc(out_dtype, {m, w.n});
+    K::mid_store(x.data, w.packed->t.data, p.t.data, out_dtype, (int)m, (int)w.n, (int)w.k, scratch.data, 1, c.stream);
+    return p;
+}
+
+static void k_mid_gated(StepContext& c, const Tensor& x, const Weight& w, Tensor& out) {
+    const int64_t m = x.shape[0];
+    const int splits = K::mid_splits.raw((int)w.n, (int)w.k, 1);
+    Tensor scratch;
+    if (splits > 1) scratch = c.alloc(F32, {splits, m, w.n});
+    K::mid_gated(x.data, w.packed->t.data, out.data, (int)m, (int)w.n, (int)w.k, scratch.data, c.stream);
+}
+
+static void k_gemm(StepContext& c, const Tensor& x, const Tensor& w, const Tensor* bias, Tensor& out) {
+    const int m = (int)x.shape[0], k = (int)x.shape[1], n = (int)w.shape[0];
+    const int bias_dt = bias ? bias->dtype : 0;
+    const size_t need = K::gemm_scratch_bytes.raw(x.dtype, w.dtype, bias_dt, out.dtype, m, n, k);
+    void* scratch = need ? c.ws->alloc(need) : nullptr;
+    K::gemm(x.data, x.dtype, w.data, w.dtype, bias ? bias->data : nullptr, bias_dt, out.data, out.dtype, m, n, k, scratch, c.stream);
+}
+
+Product linear(StepContext& c, const Tensor& x, const Weight& w, const Tensor* bias, int out_dtype, bool leave_sums, Tensor* out) {
+    if (x.ndim != 2 || x.shape[1] != w.k)
+        raise(TQE_ERR_ARGUMENT, "linear: x has %lld columns but the weight has %lld", (long long)(x.ndim == 2 ? x.shape[1] : -1), (long long)w.k);
+    const int64_t m = x.shape[0];
+    const bool both_bf16 = x.dtype == BF16 && w.dtype == BF16;
+    Product p;
+    if (both_bf16 && !bias) {
+        if (skinny_ok(x, w)) {
+            p.t = out ? *out : c.alloc(out_dtype, {m, w.n});
+            k_fused_store(c, x, nullptr, nullptr, w, p.t);
+            return p;
+        }
+        if (mid_ok(x, w)) return k_mid_store(c, x, w, out_dtype, leave_sums, out);
+        if (!w.rows) {
+            // the rows were given up: every number of rows through the own kernels, in pieces that each stream the weight once
+            p.t = out ? *out : c.alloc(out_dtype, {m, w.n});
+            const int64_t step = mid_max_rows();
+            for (int64_t r = 0; r < m; r += step) {
+                Tensor xs = x.slice(r, std::min(m, r + step)), os = p.t.slice(r, std::min(m, r + step));
+                if (xs.shape[0] <= skinny_max_rows()) k_fused_store(c, xs, nullptr, nullptr, w, os);
+                else k_mid_store(c, xs, w, out_dtype, false, &os);
+            }
+            return p;
+        }
+        if (policy().library && m > skinny_max_rows() && !null_device()) {
+            p.t = out ? *out : c.alloc(out_dtype, {m, w.n});
+            library_gemm(x, w.rows->t, p.t, c.stream);
+            return p;
+        }
+    }
+    if (!w.rows)
+        raise(TQE_ERR_STATE, "linear: this weight's rows were given up (policy keep_rows); only bfloat16 products without a bias take its packed copy");
+    p.t = out ? *out : c.alloc(out_dtype, {m, w.n});
+    k_gemm(c, x, w.rows->t, bias, p.t);
+    return p;
+}
+
+Tensor gated_silu_linear(StepContext& c, const Tensor& x, const Weight& w) {
+    const int64_t m = x.shape[0], inter = w.n / 2;
+    Tensor act = c.alloc(x.dtype, {m, inter});
+    if (skinny_ok(x, w)) { k_fused_gated(c, x, nullptr, w, act); return act; }
+    if (mid_ok(x, w)) { k_mid_gated(c, x, w, act); return act; }
+    if (!w.rows) {
+        const int64_t step = mid_max_rows();
+        for (int64_t r = 0; r < m; r += step) {
+            Tensor xs = x.slice(r, std::min(m, r + step)), os = act.slice(r, std::min(m, r + step));
+            if (xs.shape[0] <= skinny_max_rows()) k_fused_gated(c, xs, nullptr, w, os);
+            else k_mid_gated(c, xs, w, os);
+        }
+        return act;
+    }
+    Product both = linear(c, x, w, nullptr, x.dtype);
+    K::swiglu(both.t.data, act.data, act.dtype, (int)m, (int)inter, c.stream);
+    return act;
+}
+
+void add_product(StepContext& c, Stream& stream, const Tensor& x, const Weight& w) {
+    if (x.shape[0] > skinny_max_rows()) {
+        const bool leave = stream.next_norm && stream.next_norm->takes_partial_sums();
+        Product p = k_mid_store(c, x, w, BF16, leave, nullptr);
+        stream.pending = p.is_sums ? Pending::of(p.sums) : Pending::of(p.t);
+        stream.invalidate();
+        return;
+    }
+    const Norm* norm = stream.next_norm && stream.next_norm->foldable() ? stream.next_norm : nullptr;
+    int packed = 0;
+    const void* wp = few_ptr(w, &packed);
+    const int parts = K::fused_residual_parts.raw((int)w.n, (int)w.k);
+    if (stream.ss_buffer.defined() && stream.ss_buffer.numel() < (int64_t)parts * 16)
+        raise(TQE_ERR_STATE, "the stream's buffer for sums of squares holds %lld values, %d pieces of 16 are written",
+              (long long)stream.ss_buffer.numel(), parts);
+    K::fused_residual(x.data, wp, packed, (float*)stream.h.data, norm ? norm->fold_weight()->data : nullptr, stream.xw_buffer.data,
+                      (float*)stream.ss_buffer.data, (int)x.shape[0], (int)w.n, (int)w.k, c.stream);
+    stream.n_ss = parts;
+    stream.xw_for = norm;
+    stream.pending = Pending();
+}
+
+void k_add_rmsnorm(StepContext& c, float* h, const Pending& delta, const Tensor& weight, float eps, const int32_t* rows, int64_t n_rows,
+                   int64_t src_rows, Tensor& out, bool write_back) {
+    const int hidden = (int)weight.shape[0];
+    if (!rows && src_rows != n_rows) raise(TQE_ERR_ARGUMENT, "add_rmsnorm: %lld input rows but %lld output rows", (long long)src_rows, (long long)n_rows);
+    if (delta.kind == Pending::Sums) {
+        const PartialSums& s = delta.s;
+        if (s.dtype != out.dtype || s.rows() != src_rows || s.cols() != hidden)
+            raise(TQE_ERR_ARGUMENT, "add_rmsnorm: the update's sums are [%lld, %lld] of %s, wanted [%lld, %d] of %s", (long long)s.rows(),
+                  (long long)s.cols(), dtype_name(s.dtype), (long long)src_rows, hidden, dtype_name(out.dtype));
+        K::add_rmsnorm_sums(h, (const float*)s.sums.data, (int)s.sums.shape[0], (int)src_rows, out.dtype, weight.data, weight.dtype, eps, rows,
+                            (int)n_rows, hidden, out.data, write_back ? 1 : 0, c.stream);
+        return;
+    }
+    const void* d = delta.kind == Pending::Plain ? delta.t.data : nullptr;
+    if (d && (delta.t.dtype != out.dtype || delta.t.shape[0] != src_rows || delta.t.cols() != hidden))
+        raise(TQE_ERR_ARGUMENT, "add_rmsnorm: the update is %s, wanted [%lld, %d] of %s", delta.t.describe().c_str(), (long long)src_rows, hidden,
+              dtype_name(out.dtype));
+    K::add_rmsnorm(h, d, out.dtype, weight.data, weight.dtype, eps, rows, (int)n_rows, hidden, out.data, write_back ? 1 : 0, c.stream);
+}
+
+void k_gather_rows(StepContext& c, const Tensor& src, const int32_t* rows, int64_t n_rows, Tensor& out) {
+    if (out.shape[0] != n_rows || out.row_bytes() != src.row_bytes())
+        raise(TQE_ERR_ARGUMENT, "gather_rows: %s from %s", out.describe().c_str(), src.describe().c_str());
+    K::gather_rows(src.data, rows, (int)n_rows, (long long)src.row_bytes(), out.data, c.stream);
+}
+
+// ---- the library's product ---------------------------------------------------------------------
+namespace {
+
+struct Library {
+    std::mutex mutex;
+    hipblasLtHandle_t handle = nullptr;
+    void* workspace = nullptr;
+    size_t workspace_bytes = (size_t)128 << 20;
+    struct Plan {
+        hipblasLtMatmulDesc_t desc = nullptr;
+        hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr;
+        hipblasLtMatmulAlgo_t algo;
+    };
+    std::map<std::tuple<int64_t, int64_t, int64_t, int>, Plan> plans;
+};
+
+Library& library() {
+    static Library lib;
+    return lib;
+}
+
+void lt_check(hipblasStatus_t s, const char* what) {
+    if (s != HIPBLAS_STATUS_SUCCESS) raise(TQE_ERR_DEVICE, "hipBLASLt: %s failed with status %d", what, (int)s);
+}
+
+}  // namespace
+
+void library_gemm(const Tensor& x, const Tensor& w, Tensor& out, hipStream_t stream) {
+    const int64_t m = x.shape[0], k = x.shape[1], n = w.shape[0];
+    if (x.dtype != BF16 || w.dtype != BF16 || w.shape[1] != k || out.shape[0] != m || out.cols() != n || (out.dtype != BF16 && out.dtype != F32))
+        raise(TQE_ERR_ARGUMENT, "library product: %s times %s^T into %s", x.describe().c_str(), w.describe().c_str(), out.describe().c_str());
+    if (m == 0) return;
+    Library& lib = library();
+    std::lock_guard<std::mutex> lock(lib.mutex);
+    if (!lib.handle) {
+        lt_check(hipblasLtCreate(&lib.handle), "creating the handle");
+        lib.workspace = device_malloc(lib.workspace_bytes);
+    }
+    const auto key = std::make_tuple(m, n, k, out.dtype);
+    auto it = lib.plans.find(key);
+    if (it == lib.plans.end()) {
+        // in the library's column-major terms: out^T [n, m] = w [n, k] (the k x n matrix, transposed) * x^T [k, m]
+        Library::Plan plan;
+        lt_check(hipblasLtMatmulDescCreate(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F), "creating a product");
+        const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
+        lt_check(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)), "setting a product");
+        lt_check(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)), "setting a product");
+        lt_check(hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, (uint64_t)k, (uint64_t)n, k), "describing the weight");
+        lt_check(hipblasLtMatrixLayoutCreate(&plan.b, HIP_R_16BF, (uint64_t)k, (uint64_t)m, k), "describing x");
+        lt_check(hipblasLtMatrixLayoutCreate(&plan.c, out.dtype == F32 ? HIP_R_32F : HIP_R_16BF, (uint64_t)n, (uint64_t)m, n), "describing the output");
+        hipblasLtMatmulPreference_t pref;
+        lt_check(hipblasLtMatmulPreferenceCreate(&pref), "creating a preference");
+        lt_check(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &lib.workspace_bytes, sizeof(lib.workspace_bytes)),
+                 "setting the workspace");
+        hipblasLtMatmulHeuristicResult_t found[4];
+        int n_found = 0;
+        lt_check(hipblasLtMatmulAlgoGetHeuristic(lib.handle, plan.desc, plan.a, plan.b, plan.c, plan.c, pref, 4, found, &n_found), "choosing a kernel");
+        hipblasLtMatmulPreferenceDestroy(pref);
+        int pick = -1;
+        for (int i = 0; i < n_found && pick < 0; ++i)
+            if (found[i].workspaceSize <= lib.workspace_bytes) pick = i;
+        if (pick < 0) raise(TQE_ERR_DEVICE, "hipBLASLt has no kernel for a product of %lld x %lld x %lld", (long long)m, (long long)n, (long long)k);
+        plan.algo = found[pick].algo;
+        it = lib.plans.emplace(key, plan).first;
+    }
+    const Library::Plan& plan = it->second;
+    const float alpha = 1.f, beta = 0.f;
+    lt_check(hipblasLtMatmul(lib.handle, plan.desc, &alpha, w.data, plan.a, x.data, plan.b, &beta, out.data, plan.c, out.data, plan.c, &plan.algo,
+                             lib.workspace, lib.workspace_bytes, stream),
+             "the product");
+}
+
+void library_release() {
+    Library& lib = library();
+    std::lock_guard<std::mutex> lock(lib.mutex);
+    for (auto& e : lib.plans) {
+        hipblasLtMatmulDescDestroy(e.second.desc);
+        hipblasLtMatrixLayoutDestroy(e.second.a);
+        hipblasLtMatrixLayoutDestroy(e.second.b);
+        hipblasLtMatrixLayoutDestroy(e.second.c);
+    }
+    lib.plans.clear();
+    if (lib.workspace) { device_free(lib.workspace, false); lib.workspace = nullptr; }
+    if (lib.handle) { hipblasLtDestroy(lib.handle); lib.handle = nullptr; }
+}
+
+}  // namespace tq

@@ -21,6 +21,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <exception>
 #include <set>
 #include <utility>
 #include <new>
@@ -30,9 +31,11 @@
 
 namespace {
 
-thread_local char g_error[512] = "";
+thread_local char g_error[4096] = "";
+thread_local int g_status = 0;
 
 int fail(int code, const char* fmt, ...) {
+    g_status = code;
     va_list ap;
     va_start(ap, fmt);
     vsnprintf(g_error, sizeof(g_error), fmt, ap);
@@ -100,7 +103,17 @@ struct PagePool {
         late.assign(count, 0);
     }
     int n_free() const { return (int)free.size(); }
+    // what was passed over counts as new again
+    void fold_late() {
+        std::vector<int32_t> all;
+        for (const auto& e : free) all.push_back(e.second);
+        std::sort(all.begin(), all.end());
+        free.clear();
+        for (int32_t j : all) free.insert(free.end(), std::make_pair(0, j));
+        late.assign(n, 0);
+    }
     int take() {
+        if (free.begin()->first != 0) fold_late();                      // no other page is left
         const int i = free.begin()->second;
         free.erase(free.begin());
         held[i] = 1;
@@ -111,10 +124,14 @@ struct PagePool {
         if (i < 0 || i >= n || !held[i]) return false;
         held[i] = 0;
         free.insert(std::make_pair(0, i));
-        if ((int)free.size() == n && free.rbegin()->first != 0) {      // nothing is held: what was passed over counts as new again
-            free.clear();
-            for (int j = 0; j < n; ++j) free.insert(free.end(), std::make_pair(0, j));
-            late.assign(n, 0);
+        // Pages that were passed over stay last only while runs are being laid out above them: once no
+        // held page lies above the lowest of them (an engine that is never wholly idle still comes
+        // here as its oldest sequences end), they are ordinary free pages again.
+        if (!free.empty() && free.rbegin()->first != 0) {
+            const int lowest_late = free.lower_bound(std::make_pair(1, 0))->second;
+            bool held_above = false;
+            for (int j = lowest_late + 1; j < n && !held_above; ++j) held_above = held[j] != 0;
+            if (!held_above) fold_late();
         }
         return true;
     }
@@ -152,6 +169,15 @@ int pages_for(long long positions) { return (int)((positions + TQE_PAGE - 1) / T
 
 }  // namespace
 
+// the calling thread's last message, for the engine's other files
+void tqe_set_error(int code, const char* msg) {
+    g_status = code;
+    snprintf(g_error, sizeof(g_error), "%s", msg ? msg : "");
+}
+
+// No C++ exception crosses the boundary: every entry point that can allocate is a function-try-block
+// that turns a failed allocation or a length error into a status and a message.
+
 struct tqe_cache {
     int max_slots = 0;
     Pool slots;
@@ -162,9 +188,10 @@ struct tqe_cache {
 extern "C" {
 
 const char* tqe_last_error(void) { return g_error; }
+int tqe_last_status(void) { return g_status; }
 int tqe_abi_version(void) { return 2; }
 
-tqe_cache_t* tqe_cache_new(int max_slots, int n_groups, const int32_t* pages_per_group, const int32_t* window_per_group) {
+tqe_cache_t* tqe_cache_new(int max_slots, int n_groups, const int32_t* pages_per_group, const int32_t* window_per_group) try {
     if (max_slots < 1 || n_groups < 0 || n_groups > TQE_MAX_GROUPS || (n_groups > 0 && (!pages_per_group || !window_per_group))) {
         fail(TQE_ERR_ARGUMENT, "tqe_cache_new: bad arguments (slots %d, groups %d)", max_slots, n_groups);
         return nullptr;
@@ -187,20 +214,30 @@ tqe_cache_t* tqe_cache_new(int max_slots, int n_groups, const int32_t* pages_per
         c->groups[g].known.assign(max_slots, 0);
     }
     return c;
+} catch (const std::exception& e) {
+    fail(TQE_ERR_ARGUMENT, "tqe_cache_new: %s", e.what());
+    return nullptr;
+} catch (...) {
+    fail(TQE_ERR_ARGUMENT, "tqe_cache_new: unknown failure");
+    return nullptr;
 }
 
 void tqe_cache_free(tqe_cache_t* c) { delete c; }
 
-int tqe_cache_acquire(tqe_cache_t* c, int32_t* slot_out) {
+int tqe_cache_acquire(tqe_cache_t* c, int32_t* slot_out) try {
     if (!c || !slot_out) return fail(TQE_ERR_ARGUMENT, "tqe_cache_acquire: null pointer");
     if (c->slots.n_free() < 1) return fail(TQE_ERR_FULL, "need 1 slot(s), 0 free of %d", c->max_slots);
     const int s = c->slots.take();
     c->lengths[s] = 0;
     *slot_out = s;
     return TQE_OK;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_acquire: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_acquire: unknown failure");
 }
 
-int tqe_cache_release(tqe_cache_t* c, int slot) {
+int tqe_cache_release(tqe_cache_t* c, int slot) try {
     if (!c) return fail(TQE_ERR_ARGUMENT, "tqe_cache_release: null pointer");
     if (!c->slots.give_back(slot)) return fail(TQE_ERR_STATE, "slot %d given back but not held", slot);
     for (Group& g : c->groups) {
@@ -211,6 +248,10 @@ int tqe_cache_release(tqe_cache_t* c, int slot) {
     }
     c->lengths[slot] = 0;
     return TQE_OK;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_release: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_release: unknown failure");
 }
 
 int tqe_cache_length(const tqe_cache_t* c, int slot) {
@@ -229,10 +270,13 @@ int tqe_cache_counts(const tqe_cache_t* c, int group, int32_t* n_free, int32_t* 
     return TQE_OK;
 }
 
-int tqe_cache_reserve(tqe_cache_t* c, int n, const int32_t* slots, const int32_t* n_new) {
+int tqe_cache_reserve(tqe_cache_t* c, int n, const int32_t* slots, const int32_t* n_new) try {
     if (!c || (n > 0 && (!slots || !n_new))) return fail(TQE_ERR_ARGUMENT, "tqe_cache_reserve: null pointer");
-    for (int i = 0; i < n; ++i)
+    if (n < 0) return fail(TQE_ERR_ARGUMENT, "tqe_cache_reserve: %d sequences", n);
+    for (int i = 0; i < n; ++i) {
         if (slots[i] < 0 || slots[i] >= c->max_slots || !c->slots.held[slots[i]]) return fail(TQE_ERR_STATE, "slot %d is not held", slots[i]);
+        if (n_new[i] < 0) return fail(TQE_ERR_ARGUMENT, "tqe_cache_reserve: %d new positions for slot %d", n_new[i], slots[i]);
+    }
     for (const Group& g : c->groups) {
         long long want = 0;
         for (int i = 0; i < n; ++i) {
@@ -253,13 +297,27 @@ int tqe_cache_reserve(tqe_cache_t* c, int n, const int32_t* slots, const int32_t
             if (took > 1) g.pool.pass_over(took % 2 == 0 ? 1 : 2);
         }
     return TQE_OK;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_reserve: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_reserve: unknown failure");
 }
 
-int tqe_cache_commit(tqe_cache_t* c, int n, const int32_t* slots, const int32_t* n_new) {
+int tqe_cache_commit(tqe_cache_t* c, int n, const int32_t* slots, const int32_t* n_new) try {
     if (!c || (n > 0 && (!slots || !n_new))) return fail(TQE_ERR_ARGUMENT, "tqe_cache_commit: null pointer");
+    if (n < 0) return fail(TQE_ERR_ARGUMENT, "tqe_cache_commit: %d sequences", n);
+    // all of them or none: every slot is looked at before any length changes
     for (int i = 0; i < n; ++i) {
         const int s = slots[i];
         if (s < 0 || s >= c->max_slots || !c->slots.held[s]) return fail(TQE_ERR_STATE, "slot %d is not held", s);
+        if (n_new[i] < 0) return fail(TQE_ERR_ARGUMENT, "tqe_cache_commit: %d new positions for slot %d", n_new[i], s);
+        if ((long long)c->lengths[s] + n_new[i] > 0x7fffffffLL) return fail(TQE_ERR_ARGUMENT, "tqe_cache_commit: slot %d would hold too many positions", s);
+        for (const Group& g : c->groups)
+            if (pages_for((long long)c->lengths[s] + n_new[i]) > (int)g.pages[s].size())
+                return fail(TQE_ERR_STATE, "slot %d commits %d positions that were not reserved", s, n_new[i]);
+    }
+    for (int i = 0; i < n; ++i) {
+        const int s = slots[i];
         c->lengths[s] += n_new[i];
         for (Group& g : c->groups) {
             if (g.window <= 0) continue;
@@ -272,9 +330,33 @@ int tqe_cache_commit(tqe_cache_t* c, int n, const int32_t* slots, const int32_t*
         }
     }
     return TQE_OK;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_commit: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_commit: unknown failure");
 }
 
-int tqe_cache_pages(const tqe_cache_t* c, int group, int slot, int32_t* out, int cap) {
+int tqe_cache_trim(tqe_cache_t* c, int n, const int32_t* slots) try {
+    if (!c || (n > 0 && !slots)) return fail(TQE_ERR_ARGUMENT, "tqe_cache_trim: null pointer");
+    for (int i = 0; i < n; ++i)
+        if (slots[i] < 0 || slots[i] >= c->max_slots || !c->slots.held[slots[i]]) return fail(TQE_ERR_STATE, "slot %d is not held", slots[i]);
+    for (Group& g : c->groups)
+        for (int i = 0; i < n; ++i) {
+            std::vector<int32_t>& have = g.pages[slots[i]];
+            const size_t keep = (size_t)pages_for(c->lengths[slots[i]]);
+            while (have.size() > keep) {
+                if (have.back() >= 0) g.pool.give_back(have.back());
+                have.pop_back();
+            }
+        }
+    return TQE_OK;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_trim: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_trim: unknown failure");
+}
+
+int tqe_cache_pages(const tqe_cache_t* c, int group, int slot, int32_t* out, int cap) try {
     if (!c || group < 0 || group >= (int)c->groups.size() || slot < 0 || slot >= c->max_slots)
         return fail(TQE_ERR_ARGUMENT, "tqe_cache_pages: no group %d or slot %d", group, slot);
     const Group& g = c->groups[group];
@@ -283,9 +365,13 @@ int tqe_cache_pages(const tqe_cache_t* c, int group, int slot, int32_t* out, int
     if (out)
         for (int i = 0; i < (int)have.size() && i < cap; ++i) out[i] = have[i];
     return (int)have.size();
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_pages: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_pages: unknown failure");
 }
 
-int tqe_cache_check(const tqe_cache_t* c) {
+int tqe_cache_check(const tqe_cache_t* c) try {
     if (!c) return fail(TQE_ERR_ARGUMENT, "tqe_cache_check: null pointer");
     char msg[256];
     if (!c->slots.consistent("slot", msg, sizeof(msg))) return fail(TQE_ERR_STATE, "%s", msg);
@@ -306,11 +392,15 @@ int tqe_cache_check(const tqe_cache_t* c) {
             return fail(TQE_ERR_STATE, "%d pages held by sequences, pool says %d", held, g.pool.n - g.pool.n_free());
     }
     return TQE_OK;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_check: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_cache_check: unknown failure");
 }
 
 // ---- the step's arrays ------------------------------------------------------------------------
 int tqe_check_step(const tqe_cache_t* c, int n_seqs, const int32_t* slots, const int32_t* n_new, const int32_t* tokens,
-                   int vocab_size, int max_positions) {
+                   int vocab_size, int max_positions) try {
     if (!c) return fail(TQE_ERR_ARGUMENT, "tqe_check_step: null pointer");
     if (n_seqs < 1 || !slots || !n_new) return fail(TQE_ERR_STEP, "a step needs at least one sequence");
     std::vector<uint8_t> seen(c->max_slots, 0);
@@ -329,12 +419,16 @@ int tqe_check_step(const tqe_cache_t* c, int n_seqs, const int32_t* slots, const
             return fail(TQE_ERR_STEP, "sequence would reach %lld positions, the model has %d", (long long)c->lengths[s] + n_new[i], max_positions);
     }
     return TQE_OK;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_check_step: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_check_step: unknown failure");
 }
 
 
 int tqe_plan_step(const tqe_cache_t* c, int n_seqs, const int32_t* slots, const int32_t* starts, const int32_t* n_new,
                   const int32_t* tokens, const int32_t* want_counts, const int32_t* want_idx, int width_step,
-                  int32_t* out, int out_cap, int32_t* meta) {
+                  int32_t* out, int out_cap, int32_t* meta) try {
     if (n_seqs < 1 || !slots || !n_new || !want_counts || !meta) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: bad arguments");
     if (!c && !starts) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: without a cache the sequences' starts must be given");
     const int n_groups = c ? (int)c->groups.size() : 0;
@@ -344,6 +438,7 @@ int tqe_plan_step(const tqe_cache_t* c, int n_seqs, const int32_t* slots, const 
     for (int i = 0; i < n_seqs; ++i) {
         if (n_new[i] < 1) return fail(TQE_ERR_ARGUMENT, "sequence %d of the step brings no token", i);
         if (c && (slots[i] < 0 || slots[i] >= c->max_slots)) return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: no slot %d", slots[i]);
+        if (want_counts[i] < 0) return fail(TQE_ERR_ARGUMENT, "sequence %d of the step wants %d places", i, want_counts[i]);
         n_tokens += n_new[i];
         n_want += want_counts[i];
         max_new = std::max(max_new, n_new[i]);
@@ -453,6 +548,10 @@ int tqe_plan_step(const tqe_cache_t* c, int n_seqs, const int32_t* slots, const 
         }
     }
     return TQE_OK;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_plan_step: unknown failure");
 }
 
 }  // extern "C"
@@ -466,7 +565,7 @@ struct tqe_batch {
 };
 
 int tqe_plan_batches(int n, const int32_t* prompt_lens, int max_new, long long max_tokens, int max_batch, int holds_pages,
-                     int32_t* batch_of) {
+                     int32_t* batch_of) try {
     if (n < 0 || (n > 0 && (!prompt_lens || !batch_of)) || max_batch < 1) return fail(TQE_ERR_ARGUMENT, "tqe_plan_batches: bad arguments");
     int batch = 0, in_batch = 0;
     long long used = 0;
@@ -484,9 +583,13 @@ int tqe_plan_batches(int n, const int32_t* prompt_lens, int max_new, long long m
         used += need;
     }
     return n > 0 ? batch + 1 : 0;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_plan_batches: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_plan_batches: unknown failure");
 }
 
-int tqe_prompt_steps(int n, const int32_t* lens, int max_step_tokens, int32_t* pieces, int capacity) {
+int tqe_prompt_steps(int n, const int32_t* lens, int max_step_tokens, int32_t* pieces, int capacity) try {
     if (n < 0 || (n > 0 && !lens) || max_step_tokens < 1 || capacity < 0 || (capacity > 0 && !pieces))
         return fail(TQE_ERR_ARGUMENT, "tqe_prompt_steps: bad arguments");
     int count = 0, step = 0, room = max_step_tokens;
@@ -508,9 +611,13 @@ int tqe_prompt_steps(int n, const int32_t* lens, int max_step_tokens, int32_t* p
         }
     }
     return count;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_prompt_steps: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_prompt_steps: unknown failure");
 }
 
-tqe_batch_t* tqe_batch_new(int n_requests, int max_new, const int32_t* stop_ids, int n_stop_ids) {
+tqe_batch_t* tqe_batch_new(int n_requests, int max_new, const int32_t* stop_ids, int n_stop_ids) try {
     if (n_requests < 0 || n_stop_ids < 0 || (n_stop_ids > 0 && !stop_ids)) {
         fail(TQE_ERR_ARGUMENT, "tqe_batch_new: bad arguments");
         return nullptr;
@@ -526,11 +633,17 @@ tqe_batch_t* tqe_batch_new(int n_requests, int max_new, const int32_t* stop_ids,
     b->emitted.assign(n_requests, 0);
     b->ended.assign(n_requests, 0);
     return b;
+} catch (const std::exception& e) {
+    fail(TQE_ERR_ARGUMENT, "tqe_batch_new: %s", e.what());
+    return nullptr;
+} catch (...) {
+    fail(TQE_ERR_ARGUMENT, "tqe_batch_new: unknown failure");
+    return nullptr;
 }
 
 void tqe_batch_free(tqe_batch_t* b) { delete b; }
 
-int tqe_batch_accept(tqe_batch_t* b, int row, int token) {
+int tqe_batch_accept(tqe_batch_t* b, int row, int token) try {
     if (!b || row < 0 || row >= (int)b->emitted.size()) return fail(TQE_ERR_ARGUMENT, "tqe_batch_accept: no request %d", row);
     if (b->ended[row]) return TQE_TOKEN_DROPPED;
     if (b->emitted[row] >= b->max_new || std::binary_search(b->stop.begin(), b->stop.end(), (int32_t)token)) {
@@ -542,6 +655,10 @@ int tqe_batch_accept(tqe_batch_t* b, int row, int token) {
         return TQE_TOKEN_LAST;
     }
     return TQE_TOKEN_FEED;
+} catch (const std::exception& e) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_batch_accept: %s", e.what());
+} catch (...) {
+    return fail(TQE_ERR_ARGUMENT, "tqe_batch_accept: unknown failure");
 }
 
 int tqe_batch_goes_on(const tqe_batch_t* b, int row) {

@@ -353,6 +353,8 @@ static MidPlan mid_plan(int N, int K, bool gated) {
 }
 
 /* Into how many pieces the product's K is cut (1: none, no scratch is needed). */
+extern "C" int tqk_mid_max_rows(void) { return MID_MAX_ROWS; }
+
 extern "C" int tqk_mid_splits(int N, int K, int gated) {
     if (N <= 0 || K <= 0) return 1;
     return mid_plan(N, K, gated != 0).splits;

@@ -433,6 +433,8 @@ static int check_common(const FusedArgs& a, const char* what) {
 /* y[M,N] = x w^T, or with ss_parts (the sums of squares of the stream's rows in n_ss_parts
  * pieces of 16 rows each; x is then the stream times the norm's weight) that divided by
  * sqrt(sum / K + eps).  x_rows (optional) picks the rows of x. */
+extern "C" int tqk_skinny_max_rows(void) { return 16; }
+
 extern "C" int tqk_fused_store(const void* x, const int32_t* x_rows, const float* ss_parts, int n_ss_parts, float eps,
                                const void* w, int w_packed, void* y, int y_dtype, int M, int N, int K, void* stream) {
     FusedArgs a = {};

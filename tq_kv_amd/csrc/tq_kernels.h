@@ -17,6 +17,20 @@ extern "C" {
 
 const char* tqk_last_error(void);
 int tqk_abi_version(void);
+int tqk_page_size(void);                /* positions per cache page, as the kernels were built */
+int tqk_skinny_max_rows(void);          /* most rows the skinny products (tqk_fused_*) take */
+int tqk_mid_max_rows(void);             /* most rows tqk_mid_store and tqk_mid_gated take */
+int tqk_attention_max_head_dim(void);   /* the largest head size any attention kernel here takes (tqk_attention's) */
+
+/* dst row r = src row rows[r], rows of row_bytes bytes each (at most 65535 rows) */
+int tqk_gather_rows(const void* src, const int32_t* rows, int n_rows, long long row_bytes, void* dst, void* stream);
+/* x[r, :] += bias in place; x [n_rows, n], bias [n] */
+int tqk_add_bias(void* x, int x_dtype, const void* bias, int bias_dtype, int n_rows, int n, void* stream);
+/* dst[i] = src[i] in another dtype */
+int tqk_convert(const void* src, int src_dtype, void* dst, int dst_dtype, long long n, void* stream);
+/* A bfloat16 weight [n, k] (k a multiple of 32; `parts` stacked weights of n / parts rows) in the order the lanes of the
+ * few-row kernels take it: out [parts * ceil(n / parts / 16)][k / 32][64][8], see tqk_fused_store. */
+int tqk_pack_weight(const void* w, void* out, int n, int k, int parts, void* stream);
 
 /* out[t, :] = scale * float(table[ids[t], :]); ids outside [0, vocab) give zeros.  copy_bf16
  * (optional): the same values as bfloat16 [tokens, hidden], times copy_weight [hidden]

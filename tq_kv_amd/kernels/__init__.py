@@ -17,8 +17,7 @@ F32, BF16 = 0, 1
 STYLE_NONE, STYLE_HALVES, STYLE_PAIRS = 0, 1, 2
 
 
-class KernelError(RuntimeError):
-    pass
+from ..native import KernelError  # noqa: E402  (the same exception whichever face of the library raises it)
 
 
 def library():
@@ -369,6 +368,10 @@ def pack_weight(weight, parts=1):
                           % (parts, weight.dtype, tuple(weight.shape)))
     per = n // parts
     tiles = (per + 15) // 16
+    if weight.is_cuda:
+        data = torch.empty((parts * tiles, k // 32, 64, 8), dtype=torch.bfloat16, device=weight.device)
+        _check(library().tqk_pack_weight(_dev(weight, "weight"), _dev(data, "data"), n, k, parts, _stream()), "pack_weight")
+        return PackedWeight(data, n, k, parts)
     w = weight.reshape(parts, per, k)
     if per % 16:
         w = torch.cat([w, w.new_zeros((parts, tiles * 16 - per, k))], dim=1)

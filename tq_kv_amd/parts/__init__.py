@@ -1,8 +1,8 @@
-"""Parts that layers are put together from: norms, position encodings, mixers,
-feed-forwards and block arrangements, each chosen by kind from a registry."""
-from . import attention, block, feed_forward, norms, position  # noqa: F401  (registers the kinds)
-from .registry import BuildEnv, Part, known, register
+"""Parts that layers are put together from: norms, position encodings, mixers, feed-forwards and
+block arrangements, each chosen by kind from the engine library's registry; kinds written in
+Python join it through `register`."""
+from .registry import BuildEnv, Part, PartHandle, known, register
 from .spec import KVNeed, LayerSpec, ModelSpec, PartSpec, Run, StateNeed, TensorSpec
 
-__all__ = ["BuildEnv", "Part", "known", "register", "KVNeed", "LayerSpec", "ModelSpec", "PartSpec", "Run",
+__all__ = ["BuildEnv", "Part", "PartHandle", "known", "register", "KVNeed", "LayerSpec", "ModelSpec", "PartSpec", "Run",
            "StateNeed", "TensorSpec"]

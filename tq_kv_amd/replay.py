@@ -29,11 +29,12 @@ def main(argv=None):
                     help="most tokens live requests hold at any time, each request counted up to a multiple of 64")
     args = ap.parse_args(argv)
 
-    from . import kernels
+    from . import kernels, native
+    kernels.library()                       # builds the kernels and the engine on a first call, with progress lines
+    native.library()
     from .cache.store import PAGE
     from .engine import Engine, Model
 
-    kernels.library()                       # builds the kernels on a first call, with progress lines
     os.makedirs(args.out, exist_ok=True)
     model = Model.from_dir(args.model, dtype=args.dtype, device="cuda")
     max_tokens = max(PAGE, (args.max_tokens + PAGE - 1) // PAGE * PAGE)

@@ -1,86 +1,56 @@
-"""Choosing next tokens on the device for the live requests of a batch.
+"""Choosing next tokens on the device for the live requests of a batch (csrc/engine/generate.cpp:
+DeviceSampler, behind tqe_sampler_*; this class holds the handle).
 
-The reference samples one request on the host (src/engine.rs:353-373, 403-423):
-repeat penalty over the generated tokens (not on the first draw, when none exist),
-then argmax if temperature <= 0, else top-k then top-p at the temperature.  Here the
-same steps run as kernels on the rows of the step's logits; the history of generated
-tokens lives on the device and is appended to by a kernel.
+The reference samples one request on the host (src/engine.rs:353-373, 403-423): repeat penalty over
+the generated tokens (not on the first draw, when none exist), then argmax if temperature <= 0,
+else top-k then top-p at the temperature.  Here the same steps run as kernels on the rows of the
+step's logits; the history of generated tokens lives on the device and is appended to by a kernel.
+The generation loop makes its samplers inside the library; this one is for whoever steps an engine
+by hand.
 """
+import ctypes
+
 import numpy as np
-import torch
 
-from .. import kernels as K
-from .rng import uniform
-
-
-class Drawn:
-    """Tokens that have been chosen on the device and are on their way to the host.
-    `device`: int32 [rows].  read() waits for this draw's copy alone, not for work that was
-    started after it."""
-
-    def __init__(self, device, host, event):
-        self.device, self._host, self._event = device, host, event
-
-    def read(self):
-        self._event.synchronize()
-        return self._host.tolist()
+from .. import native
 
 
 class Sampler:
-    """params: GenerationParams.  n_requests: requests of the batch; request_ids: for each
-    its number in the whole run (feeds the random stream)."""
+    """params: GenerationParams.  request_ids: for each request of the batch its number in the
+    whole run (feeds the random stream)."""
 
-    READ_AHEAD = 4         # draws that may be unread at a time
-
-    def __init__(self, params, request_ids, device):
-        from ..engine.context import HostStaging
+    def __init__(self, params, request_ids, device, vocab_size=None):
+        from ..engine.generate import _c_params
+        self._lib = native.library()
         self.params = params
         self.request_ids = list(request_ids)
         self.device = device
-        n = len(self.request_ids)
-        self.use_penalty = params.repeat_penalty != 1.0
-        if self.use_penalty:
-            self.hist = torch.zeros((n, max(1, params.max_tokens + 1)), dtype=torch.int32, device=device)
-            self.hist_times = torch.zeros_like(self.hist)
-            self.hist_len = torch.zeros((n,), dtype=torch.int32, device=device)
-        self.steps = [0] * n
-        self.staging = HostStaging(device, depth=2 * self.READ_AHEAD)
-        self.landing = torch.empty((self.READ_AHEAD, max(1, n)), dtype=torch.int32, pin_memory=True)
-        self.turn = 0
+        self._vocab = vocab_size
+        self._cp = _c_params(params)
+        self.handle = None
 
-    def draw(self, logits, rows):
-        """logits: [R, V] float32 (changed in place by the penalty); rows: for each row the
-        request's index in the batch.  Starts the choice and the copy of the R chosen token
-        ids to the host, waits for neither."""
-        p = self.params
-        n = len(rows)
-        out = torch.empty((n,), dtype=torch.int32, device=self.device)
-        row_req = None
-        if self.use_penalty:
-            row_req = self.staging.upload(np.asarray(rows, dtype=np.int32))
-            K.repeat_penalty(logits, row_req, self.hist, self.hist_times, self.hist_len, p.repeat_penalty)
-        if p.greedy:
-            K.argmax(logits, out)
-        else:
-            u = np.asarray([uniform(p.seed, self.request_ids[r], self.steps[r]) for r in rows], dtype=np.float32)
-            K.sample(logits, p.temperature, p.top_k, p.top_p, self.staging.upload(u), out)
-        for r in rows:
-            self.steps[r] += 1
-        if self.use_penalty:
-            K.append_history(out, row_req, self.hist, self.hist_times, self.hist_len)
-        host = self.landing[self.turn, :n]
-        self.turn = (self.turn + 1) % self.READ_AHEAD
-        host.copy_(out, non_blocking=True)
-        event = torch.cuda.Event()
-        event.record()
-        return Drawn(out, host, event)
+    def _ensure(self, vocab):
+        if self.handle is None:
+            ids = np.asarray(self.request_ids, dtype=np.int32)
+            self._vocab = int(vocab)
+            self.handle = native.handle(self._lib.tqe_sampler_new(ctypes.byref(self._cp), len(ids), native._ptr(ids), self._vocab,
+                                                                  native.current_stream()))
+        elif int(vocab) != self._vocab:
+            raise ValueError("this sampler was made for a vocabulary of %d, the logits have %d" % (self._vocab, vocab))
 
-    def pick(self, drawn, places):
-        """The tokens of a draw at the given places, on the device, in that order."""
-        if list(places) == list(range(drawn.device.shape[0])):
-            return drawn.device
-        return drawn.device[self.staging.upload(np.asarray(places, dtype=np.int32)).long()]
+    def __del__(self):
+        h, self.handle = getattr(self, "handle", None), None
+        if h:
+            self._lib.tqe_sampler_free(h)
 
     def sample(self, logits, rows):
-        """draw() and wait: the R chosen token ids as a list."""
-        return self.draw(logits, rows).read()
+        """logits: [R, V] float32 on the device (changed in place by the penalty); rows: for each row
+        the request's index in the batch.  The R chosen token ids as a list."""
+        import torch
+        if logits.dtype != torch.float32 or not logits.is_contiguous() or logits.dim() != 2 or logits.shape[0] != len(rows):
+            raise ValueError("the sampler takes float32 logits [%d, vocab], got %s %s" % (len(rows), logits.dtype, tuple(logits.shape)))
+        self._ensure(logits.shape[1])
+        r = np.asarray(list(rows), dtype=np.int32)
+        out = np.zeros(max(1, len(r)), dtype=np.int32)
+        native.check(self._lib.tqe_sampler_sample(self.handle, ctypes.c_void_p(logits.data_ptr()), len(r), native._ptr(r), native._ptr(out)))
+        return out[:len(r)].tolist()
