@@ -55,7 +55,7 @@ def main():
 
     from tq_kv_amd import Engine, GenerationParams, Model, generate
     from tq_kv_amd.config import catalog
-    from tq_kv_amd.parts.linear import POLICY
+    from tq_kv_amd import POLICY
 
     t_start = time.perf_counter()
 
@@ -93,7 +93,7 @@ def main():
 
     # -- prefill of one prompt --------------------------------------------------------------
     if not args.no_tune:
-        # products of more than 128 rows are the library's: let it try its kernels once for the
+        # products of more rows than the own kernels take are the library's: let it try its kernels once for the
         # shapes of the measured prompt pass
         note("library tuning for %d rows" % args.prompt_len)
         model.tune_library(args.prompt_len)
@@ -133,7 +133,7 @@ def main():
         ps = prompts(batch)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        out = generate(engine, ps, params, on_tokens=on_tokens, max_batch=batch)
+        out = generate(engine, ps, params, eos_ids=(), on_tokens=on_tokens, max_batch=batch)
         torch.cuda.synchronize()
         whole = time.perf_counter() - t0
         assert all(len(o) == warmup + steps + 2 for o in out)

@@ -28,7 +28,15 @@ TINY_C = {
     "rope_theta": 50000.0, "max_position_embeddings": 640, "tie_word_embeddings": False,
     "use_sliding_window": True, "sliding_window": 100, "max_window_layers": 2,
 }
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# A fourth one with the head size of the large models (128) in three groups of two heads, at a width that is no power of two.
+TINY_D = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_act": "silu",
+    "vocab_size": 411, "hidden_size": 160, "intermediate_size": 288, "num_hidden_layers": 2,
+    "num_attention_heads": 6, "num_key_value_heads": 3, "head_dim": 128, "rms_norm_eps": 2e-6,
+    "rope_theta": 300000.0, "max_position_embeddings": 256, "tie_word_embeddings": True,
+    "use_sliding_window": False,
+}
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
 
 
 def make_folder(tmp, cfg, seed, store_dtype=torch.bfloat16):

@@ -54,6 +54,20 @@ def test_wrong_types_and_combinations():
         config_from_dict(raw)
 
 
+def test_what_no_kernel_takes_is_refused_before_any_weight_is_read(tmp_path):
+    """A head size beyond what the attention kernels take is a fine config.json as far as the architecture goes; the
+    model refuses it when its parts are built (from the kernel library's own word on its limit), not at the first step."""
+    from tq_kv_amd import Model
+    raw = dict(TINY_A, head_dim=320)
+    assert config_from_dict(raw)[1].head_dim == 320
+    with pytest.raises(ConfigError, match="head_dim 320 is more than the attention kernels take"):
+        Model.from_config_dict(raw, "float32", "cpu")
+    (tmp_path / "config.json").write_text(json.dumps(raw))          # a folder without weights: the refusal comes first
+    with pytest.raises(ConfigError, match="head_dim 320"):
+        Model.from_dir(str(tmp_path), dtype="bfloat16", device="cpu")
+    assert Model.from_config_dict(dict(TINY_A, head_dim=256), "float32", "cpu").config.head_dim == 256
+
+
 def test_unknown_architecture_lists_the_known():
     with pytest.raises(ConfigError, match="Qwen2ForCausalLM"):
         config_from_dict(dict(TINY_A, architectures=["LlamaForCausalLM"]))

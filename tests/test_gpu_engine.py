@@ -305,7 +305,8 @@ def test_step_refuses_what_it_cannot_run():
         eng.step([(s, [1], [0]), (s, [2], [0])])
     with pytest.raises(IndexError):
         eng.step([(s, [1, 2], [2])])
-    assert eng.length(s) == 0
+    # nothing of a refused step stays behind: no position, no page
+    assert eng.length(s) == 0 and all(g.pool.n_held == 0 for g in eng.cache.kv_groups)
     eng.close(s)
     from tq_kv_amd import Engine
     small = Engine(eng.model, max_tokens=128)
@@ -461,3 +462,36 @@ def test_many_sequences_decode_through_replayed_graphs(dtype, products_of_17_to_
     for s in slots:
         eng.close(s)
     eng.cache.check()
+
+
+# ---- decoding steps of more sequences than the graphs and the own products take ---------------------
+@pytest.mark.parametrize("n_seqs", [128, 129, 200])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,sharp", [("B", True), ("D", False)])
+def test_decode_steps_of_a_hundred_and_more_sequences(name, sharp, dtype, n_seqs):
+    """Steps of exactly 128 sequences (the last that is captured as a graph and runs the own products), of 129 and of
+    200 (eager, the library's products, the decoding attention kernel with more than 128 rows), and on the way down
+    the steps either side of every change of kernels: 128 and 127, 17 and 16.  Sequences of unequal lengths; every
+    row of every step against the plain implementation."""
+    eng = G.engine(name, dtype, sharp, max_tokens=64 * 256)
+    lens = [1 + (5 * i) % 13 for i in range(n_seqs)]
+    reqs = G.prompts(name, [n + 9 for n in lens], seed=3000)
+    refs = [G.plain_logits(name, r, sharp) for r in reqs]
+    slots = [eng.open() for _ in reqs]
+    out = eng.step([(s, r[:n], [n - 1]) for s, r, n in zip(slots, reqs, lens)])
+    for i in range(n_seqs):
+        G.close(out[i], refs[i][lens[i] - 1], dtype, "seq %d, last place of its prompt" % i)
+    pos = list(lens)
+    live = list(range(n_seqs))
+    for count in [n_seqs, 128, 127, 64, 17, 16, 1]:
+        while len(live) > count:                 # the sequences in the middle of the batch end first
+            eng.close(slots[live.pop(len(live) // 2)])
+        out = eng.step([(slots[i], [reqs[i][pos[i]]], [0]) for i in live])
+        for j, i in enumerate(live):
+            G.close(out[j], refs[i][pos[i]], dtype, "seq %d at %d in a step of %d" % (i, pos[i], len(live)))
+            pos[i] += 1
+    assert len(eng.graphs) >= 6                    # the steps of up to 128 sequences went through captured graphs
+    for i in live:
+        eng.close(slots[i])
+    eng.cache.check()
+    assert eng.cache.slots.n_held == 0

@@ -28,12 +28,43 @@ def ints(values):
 
 
 def test_library_is_built_and_loaded():
-    assert K.library().tqk_abi_version() == 10
+    assert K.library().tqk_abi_version() == 11
     assert K.library_path().endswith(".so")
     with pytest.raises(K.KernelError, match="GPU only"):
         K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
     with pytest.raises(K.KernelError, match="shape"):
         K.swiglu(torch.zeros(2, 5, device=DEV), torch.zeros(2, 2, device=DEV))
+
+
+@pytest.mark.parametrize("shape,dtype", [((37, 70), torch.float32), ((5, 3, 16), torch.bfloat16), ((9, 7), torch.bfloat16), ((4, 33), torch.int32),
+                                         ((300, 1), torch.int32), ((20, 4096), torch.float32)])
+def test_gather_rows(shape, dtype):
+    g = torch.Generator().manual_seed(1)
+    src = (torch.randn(*shape, generator=g) * 100).to(dtype).to(DEV)
+    idx = torch.randint(0, shape[0], (53,), generator=g).to(torch.int32).to(DEV)
+    out = torch.full((53,) + tuple(shape[1:]), 7, dtype=dtype, device=DEV)
+    assert torch.equal(K.gather_rows(src, idx, out), src[idx.long()])
+    assert K.gather_rows(src, idx[:0], out[:0]).shape[0] == 0
+    with pytest.raises(K.KernelError, match="outside"):
+        K.gather_rows(src, ints([shape[0]]), out[:1])
+
+
+@pytest.mark.parametrize("xd,bd", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16),
+                                   (torch.bfloat16, torch.float32)])
+def test_add_bias_and_convert(xd, bd):
+    x, b = rand(13, 77, seed=3, dtype=xd), rand(77, seed=4, dtype=bd)
+    want = (x.float() + b.float()).to(xd)
+    assert torch.equal(K.add_bias(x.clone(), b), want)
+    out = torch.empty(13, 77, dtype=bd, device=DEV)
+    assert torch.equal(K.convert(x, out), x.to(bd))
+
+
+def test_pack_weight_on_the_gpu_equals_the_plain_reordering():
+    for n, k, parts in ((40, 96, 1), (224, 96, 2), (3584, 512, 1), (19, 64, 1)):
+        w = rand(n, k, seed=n, dtype=torch.bfloat16)
+        got = K.pack_weight(w, parts)
+        want = K.pack_weight(w.cpu(), parts)              # torch's reshape and permute on the host
+        assert tuple(got.data.shape) == tuple(want.data.shape) and torch.equal(got.data.cpu(), want.data)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

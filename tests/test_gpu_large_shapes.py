@@ -56,11 +56,51 @@ def test_bfloat16_tracks_float32_at_large_sizes(shape):
     assert rms.max().item() < 0.07 and worst.max().item() < 0.35, (rms.max().item(), worst.max().item())
 
 
-@pytest.mark.parametrize("shape,n_seqs", [("qwen2.5:7b", 20), ("qwen2.5:32b", 40), ("qwen2.5:7b", 100)])
-def test_bfloat16_tracks_float32_in_steps_of_17_to_128_rows_at_large_sizes(shape, n_seqs):
+@pytest.mark.parametrize("shape", ["qwen2.5:32b", "qwen2.5:1.5b"])
+def test_a_wrong_kv_head_is_noticed_at_the_large_sizes(shape):
+    """What the comparison of bfloat16 with the float32 path at these sizes can see: the same model with the keys and
+    values of two kv heads of layer 1 exchanged (in the weights of the bfloat16 run alone, which is what a kernel that
+    maps a query head to the wrong kv head would compute) must fail it, in a prompt step and in a decoding step;
+    the groups are of 5 (32B) and of 6 heads (1.5B)."""
+    raw = two_layer(shape)
+    tensors = sharpened(tensors_for(raw, 3))
+    d, nkv = raw["head_dim"], raw["num_key_value_heads"]
+    swapped = dict(tensors)
+    for part in ("k_proj", "v_proj"):
+        for kind in ("weight", "bias"):
+            name = "model.layers.1.self_attn.%s.%s" % (part, kind)
+            t = tensors[name].clone()
+            a, b = slice(0, d), slice((nkv - 1) * d, nkv * d)
+            t[a], t[b] = tensors[name][b], tensors[name][a]
+            swapped[name] = t
+    prompts = [helpers.random_tokens(n, raw["vocab_size"], 50 + i) for i, n in enumerate([300, 70])]
+
+    def run(dtype, which):
+        eng = Engine(build(raw, dtype, which), max_tokens=1024)
+        slots = [eng.open() for _ in prompts]
+        a = eng.step([(s, p, [len(p) - 1, len(p) // 2]) for s, p in zip(slots, prompts)])
+        b = eng.step([(s, [t], [0]) for s, t in zip(slots, [7, 11])])
+        for s in slots:
+            eng.close(s)
+        del eng
+        torch.cuda.empty_cache()
+        return torch.cat([a, b]).cpu()
+
+    f32, good, bad = run("float32", tensors), run("bfloat16", tensors), run("bfloat16", swapped)
+    rms, worst = row_errors(good, f32)
+    assert rms.max().item() < 0.07 and worst.max().item() < 0.35, (rms.max().item(), worst.max().item())
+    rms_bad, _ = row_errors(bad, f32)
+    assert rms_bad.min().item() > 0.14, rms_bad                   # every row, twice the allowance and more
+    print("clean rms", rms.max().item(), "with two kv heads exchanged", rms_bad.min().item())
+
+
+@pytest.mark.parametrize("shape,n_seqs", [("qwen2.5:7b", 20), ("qwen2.5:32b", 40), ("qwen2.5:7b", 100), ("qwen2.5:7b", 128),
+                                          ("qwen2.5:7b", 129), ("qwen2.5:1.5b", 200)])
+def test_bfloat16_tracks_float32_in_steps_of_17_and_more_rows_at_large_sizes(shape, n_seqs):
     """The kernels for 17 to 128 rows at the real widths (sums over pieces of K finished by the norm
-    and the rotation kernels, the head product with float32 output): a short prompt step of 24
-    tokens, then two decoding steps of n_seqs rows."""
+    and the rotation kernels, the head product with float32 output), and the steps beyond them (129 and
+    200 rows: eager, the library's products): a short prompt step of 24 tokens, then two decoding steps
+    of n_seqs rows."""
     raw = two_layer(shape)
     tensors = tensors_for(raw, 5)
     first = [helpers.random_tokens(1 + i % 3, raw["vocab_size"], 80 + i) for i in range(n_seqs)]

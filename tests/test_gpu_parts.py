@@ -289,6 +289,141 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
     eng.cache.check()
 
 
+@register("mixer", "toy_half_values")
+class ToyHalfValues(Part):
+    """Causal softmax attention of one head whose values are half as wide as its keys, kept in pages of its own layout
+    (keys [page, width], values [page, width / 2], positions in order): the need names the two page shapes and the cache
+    multiplies them out; the mixer writes and reads its pages itself through the step's page table.  No position
+    encoding, no window."""
+
+    def __init__(self, params, env):
+        self.hidden, self.width = params["hidden"], params["width"]
+
+    def tensors(self):
+        h, w = self.hidden, self.width
+        return {"q.weight": TensorSpec((w, h)), "k.weight": TensorSpec((w, h)), "v.weight": TensorSpec((w // 2, h)),
+                "o.weight": TensorSpec((h, w // 2))}
+
+    def load(self, tensors):
+        self.w = {k: v.float() for k, v in tensors.items()}
+
+    def cache_need(self):
+        from tq_kv_amd.cache import PAGE
+        return KVNeed(key_page=(PAGE, self.width), value_page=(PAGE, self.width // 2))
+
+    def forward(self, x, ctx, entry):
+        from tq_kv_amd.cache import PAGE
+        xf = x.float()
+        q, k, v = (xf @ self.w[n + ".weight"].t() for n in "qkv")
+        table = ctx.page_table(entry.group)
+        out = torch.empty_like(xf)
+        for b in range(ctx.n_seqs):
+            a, e, start = int(ctx.host.cu[b]), int(ctx.host.cu[b + 1]), int(ctx.host.seq_start[b])
+            pos = torch.arange(start, start + e - a, device=x.device)
+            pages = table[b].long()[pos // PAGE]
+            assert (pages >= 0).all()
+            entry.keys[pages, pos % PAGE] = k[a:e].to(entry.keys.dtype)
+            entry.values[pages, pos % PAGE] = v[a:e].to(entry.values.dtype)
+            past = torch.arange(start + e - a, device=x.device)
+            keys = entry.keys[table[b].long()[past // PAGE], past % PAGE].float()
+            values = entry.values[table[b].long()[past // PAGE], past % PAGE].float()
+            scores = (q[a:e] @ keys.t()) / self.width ** 0.5
+            scores = scores.masked_fill(past[None, :] > pos[:, None], float("-inf"))
+            out[a:e] = (torch.softmax(scores, -1) @ values) @ self.w["o.weight"].t()
+        return out.to(x.dtype)
+
+
+def test_a_toy_mixer_whose_values_are_half_as_wide_as_its_keys_brings_its_own_pages():
+    cfg = dict(helpers.TINY_A, num_hidden_layers=3)
+    h = cfg["hidden_size"]
+    toy = PartSpec("toy_half_values", {"hidden": h, "width": 24})
+    model = Model(tiny_spec(cfg, mixers={1: toy}), "float32", DEV)       # attention, toy, attention
+    from tq_kv_amd.cache import PAGE
+    assert model.needs[1] == KVNeed(key_page=(PAGE, 24), value_page=(PAGE, 12)) and model.needs[0] == KVNeed(2, 16)
+    specs = {n: TensorSpec(s.shape, s.init, 0.2 if s.init == "normal" else 0.1) for n, s in model.tensor_specs().items()}
+    w = random_tensors(specs, 16, torch.float32, "cpu")
+    model.load({k: v.to(DEV) for k, v in w.items()})
+    eng = Engine(model, max_tokens=1024)
+    groups = eng.cache.kv_groups
+    assert len(groups) == 2 and groups[0].runs == [0, 2] and groups[1].runs == [1]
+    assert tuple(groups[1].keys.shape) == (1, 16, PAGE, 24) and tuple(groups[1].values.shape) == (1, 16, PAGE, 12)
+
+    def plain_forward(tokens):
+        x = w["model.embed_tokens.weight"][tokens]
+        eps, t = cfg["rms_norm_eps"], len(tokens)
+        for l in range(3):
+            p = "model.layers.%d." % l
+            hn = plain.rms_norm(x, w[p + "input_layernorm.weight"], eps)
+            if l == 1:
+                q, k, v = (hn @ w[p + "self_attn.%s.weight" % n].t() for n in "qkv")
+                scores = (q @ k.t()) / 24 ** 0.5
+                scores = scores.masked_fill(~plain.visibility(t), float("-inf"))
+                x = x + (torch.softmax(scores, -1) @ v) @ w[p + "self_attn.o.weight"].t()
+            else:
+                x = x + plain.attention(hn, w, p + "self_attn.", cfg, None)
+            x = x + plain.swiglu_mlp(plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], eps), w, p + "mlp.")
+        return plain.linear(plain.rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"])
+
+    a, b = helpers.random_tokens(100, 256, 4), helpers.random_tokens(9, 256, 5)
+    for round_ in range(2):                      # the second time on pages that were used before
+        sa, sb = eng.open(), eng.open()
+        out = eng.step([(sa, a[:70], list(range(70))), (sb, b[:4], list(range(4)))])       # sequence a crosses a page
+        got_a, got_b = [out[:70]], [out[70:]]
+        for t in range(5):
+            out = eng.step([(sa, [a[70 + t]], [0]), (sb, [b[4 + t]], [0])])
+            got_a.append(out[:1]), got_b.append(out[1:])
+        eng.close(sb)
+        got_a.append(eng.step([(sa, a[75:], list(range(25)))]))
+        eng.close(sa)
+        torch.testing.assert_close(torch.cat(got_a).cpu(), plain_forward(a), atol=2e-5, rtol=2e-5)
+        torch.testing.assert_close(torch.cat(got_b).cpu(), plain_forward(b), atol=2e-5, rtol=2e-5)
+    eng.cache.check()
+    assert all(g.pool.n_held == 0 for g in groups)
+
+
+@register("feed_forward", "toy_fuse")
+class ToyFuse(Part):
+    """A feed-forward that fails when told to: y = x otherwise."""
+    blow = [False]
+
+    def __init__(self, params, env):
+        pass
+
+    def forward(self, x, ctx):
+        if self.blow[0]:
+            raise RuntimeError("the toy blew")
+        return x
+
+
+def test_a_step_that_fails_in_the_model_leaves_nothing_behind():
+    """A part fails in the middle of a step: the caller sees the part's own exception, the sequences keep the lengths they
+    had, the pages reserved for the step are free again, and the next step is as if nothing had happened."""
+    cfg = dict(helpers.TINY_A)
+    model = Model(tiny_spec(cfg, ffs={1: PartSpec("toy_fuse", {})}), "float32", DEV)
+    specs = {n: TensorSpec(s.shape, s.init, 0.2 if s.init == "normal" else 0.1) for n, s in model.tensor_specs().items()}
+    model.load({k: v.to(DEV) for k, v in random_tensors(specs, 17, torch.float32, "cpu").items()})
+    eng = Engine(model, max_tokens=1024)
+    prompt = helpers.random_tokens(120, 256, 9)
+    s = eng.open()
+    first = eng.step([(s, prompt[:10], [9])])
+    held = [g.pool.n_held for g in eng.cache.kv_groups]
+    ToyFuse.blow[0] = True
+    try:
+        with pytest.raises(RuntimeError, match="the toy blew"):
+            eng.step([(s, prompt[10:], [0])])           # would have taken another page
+    finally:
+        ToyFuse.blow[0] = False
+    eng.cache.check()
+    assert eng.length(s) == 10 and [g.pool.n_held for g in eng.cache.kv_groups] == held
+    again = eng.step([(s, prompt[10:], [109])])
+    eng.close(s)
+    s2 = eng.open()
+    whole = eng.step([(s2, prompt, [9, 119])])
+    eng.close(s2)
+    torch.testing.assert_close(torch.cat([first, again]).cpu(), whole.cpu(), atol=2e-5, rtol=2e-5)
+    eng.cache.check()
+
+
 # ---- a toy feed-forward with routing ----------------------------------------------------------
 @register("feed_forward", "toy_routed")
 class ToyRouted(Part):

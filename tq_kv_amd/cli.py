@@ -69,6 +69,8 @@ def build_parser():
     b.add_argument("-n", "--tokens", type=int, default=100, help="Number of tokens to generate per run")
     b.add_argument("--prompt-len", type=int, default=32, help="Length of the random prompt")
     b.add_argument("--json", action="store_true", help="Output results as JSON")
+    b.add_argument("--tune", action="store_true",
+                   help="Let the matrix library try its kernels for the prompt's size first (takes some milliseconds a shape)")
     r = sub.add_parser("replay", help="Replay a trace of steps from standard input and write logits")
     r.add_argument("--model", required=True)
     r.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
@@ -161,11 +163,13 @@ def cmd_bench(args):
     prompt = torch.randint(0, model.spec.vocab_size, (args.prompt_len,), generator=g).tolist()
     engine = Engine(model, max_tokens=args.max_cache_tokens or (args.prompt_len + args.tokens + 2 * PAGE) // PAGE * PAGE)
     params = GenerationParams(max_tokens=args.tokens, temperature=0.0, repeat_penalty=1.0)
-    generate(engine, [prompt], GenerationParams(max_tokens=4, temperature=0.0, repeat_penalty=1.0))      # warm-up
+    if args.tune:
+        model.tune_library(len(prompt))
+    generate(engine, [prompt], GenerationParams(max_tokens=4, temperature=0.0, repeat_penalty=1.0), eos_ids=())      # warm-up
     marks = []
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    out = generate(engine, [prompt], params, on_tokens=lambda pairs: marks.append(time.perf_counter()))
+    out = generate(engine, [prompt], params, eos_ids=(), on_tokens=lambda pairs: marks.append(time.perf_counter()))
     torch.cuda.synchronize()
     total = time.perf_counter() - t0
     res = {"model": args.model, "dtype": args.dtype, "prompt_tokens": len(prompt), "tokens": len(out[0]),

@@ -351,6 +351,14 @@ int tqe_model_randomize(tqe_model_t* model, uint64_t seed, void* stream) {
     });
 }
 
+int tqe_model_tune_library(tqe_model_t* model, int rows, void* stream) {
+    return guarded([&] {
+        need(model, "tqe_model_tune_library");
+        DeviceScope scope(model->m->on_gpu);
+        model->m->tune_library(rows, (hipStream_t)stream);
+    });
+}
+
 const char* tqe_model_describe(const tqe_model_t* model) {
     if (!model) { set_error(TQE_ERR_ARGUMENT, "tqe_model_describe: null pointer"); return nullptr; }
     tqe_model_t* m = const_cast<tqe_model_t*>(model);

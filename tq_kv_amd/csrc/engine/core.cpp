@@ -216,6 +216,17 @@ void* kernel_symbol(const char* name) {
                                         "(build it with tq_kv_amd/csrc/build.py, or name it in TQ_KERNEL_LIBRARY)");
         g_kernel_handle = dlopen(g_kernel_path.c_str(), RTLD_NOW | RTLD_LOCAL);
         if (!g_kernel_handle) throw Error(TQE_ERR_DEVICE, format("cannot load the HIP kernel library %s: %s", g_kernel_path.c_str(), dlerror()));
+        // the two libraries index the same cache pages and share one list of entry points: both must say so
+        typedef int (*Query)(void);
+        Query page = (Query)dlsym(g_kernel_handle, "tqk_page_size"), abi = (Query)dlsym(g_kernel_handle, "tqk_abi_version");
+        const int page_size = page ? page() : -1, abi_version = abi ? abi() : -1;
+        if (page_size != TQE_PAGE || abi_version != TQE_KERNEL_ABI) {
+            dlclose(g_kernel_handle);
+            g_kernel_handle = nullptr;
+            throw Error(TQE_ERR_DEVICE, format("the kernel library %s does not fit this engine library: its cache pages hold %d positions (here %d), "
+                                               "its interface is version %d (here %d); build both from the same sources",
+                                               g_kernel_path.c_str(), page_size, TQE_PAGE, abi_version, TQE_KERNEL_ABI));
+        }
     }
     void* sym = dlsym(g_kernel_handle, name);
     if (!sym) throw Error(TQE_ERR_DEVICE, format("the kernel library %s has no entry point %s (built from other sources?)", g_kernel_path.c_str(), name));

@@ -23,8 +23,9 @@ void prime_graph_launches() {
     K::finish_logits((float*)buf.data(), 1, 64, nullptr, 1.0f, 0.0f, s);
     hip_check(hipStreamEndCapture(s, &graph), "ending a capture");
     hip_check(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "instantiating a graph");
-    hip_check(hipGraphLaunch(exec, s), "launching a graph");
-    stream_synchronize(s);
+    // launched where steps will be launched by a caller that names no stream: the default stream
+    hip_check(hipGraphLaunch(exec, nullptr), "launching a graph");
+    stream_synchronize(nullptr);
     (void)hipGraphExecDestroy(exec);
     (void)hipGraphDestroy(graph);
     (void)hipStreamDestroy(s);

@@ -2,6 +2,7 @@
 
 #include <hip/hip_runtime_api.h>
 #include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
 
 #include <algorithm>
 #include <mutex>
@@ -284,6 +285,59 @@ void lt_check(hipblasStatus_t s, const char* what) {
 
 }  // namespace
 
+namespace {
+
+// the plan of a shape, with the library's proposals for it (the first that fits is the plan's kernel until tuning says otherwise)
+Library::Plan& plan_for(Library& lib, int64_t m, int64_t n, int64_t k, int out_dtype, std::vector<hipblasLtMatmulHeuristicResult_t>* proposals, int want) {
+    if (!lib.handle) {
+        lt_check(hipblasLtCreate(&lib.handle), "creating the handle");
+        lib.workspace = device_malloc(lib.workspace_bytes);
+    }
+    const auto key = std::make_tuple(m, n, k, out_dtype);
+    auto it = lib.plans.find(key);
+    if (it != lib.plans.end() && !proposals) return it->second;
+    // in the library's column-major terms: out^T [n, m] = w [n, k] (the k x n matrix, transposed) * x^T [k, m]
+    Library::Plan fresh;
+    Library::Plan& plan = it != lib.plans.end() ? it->second : fresh;
+    if (it == lib.plans.end()) {
+        lt_check(hipblasLtMatmulDescCreate(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F), "creating a product");
+        const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
+        lt_check(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)), "setting a product");
+        lt_check(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)), "setting a product");
+        lt_check(hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, (uint64_t)k, (uint64_t)n, k), "describing the weight");
+        lt_check(hipblasLtMatrixLayoutCreate(&plan.b, HIP_R_16BF, (uint64_t)k, (uint64_t)m, k), "describing x");
+        lt_check(hipblasLtMatrixLayoutCreate(&plan.c, out_dtype == F32 ? HIP_R_32F : HIP_R_16BF, (uint64_t)n, (uint64_t)m, n), "describing the output");
+    }
+    hipblasLtMatmulPreference_t pref;
+    lt_check(hipblasLtMatmulPreferenceCreate(&pref), "creating a preference");
+    lt_check(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &lib.workspace_bytes, sizeof(lib.workspace_bytes)),
+             "setting the workspace");
+    std::vector<hipblasLtMatmulHeuristicResult_t> found((size_t)want);
+    int n_found = 0;
+    const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(lib.handle, plan.desc, plan.a, plan.b, plan.c, plan.c, pref, want, found.data(), &n_found);
+    hipblasLtMatmulPreferenceDestroy(pref);
+    lt_check(st, "choosing a kernel");
+    found.resize((size_t)std::max(n_found, 0));
+    found.erase(std::remove_if(found.begin(), found.end(), [&](const hipblasLtMatmulHeuristicResult_t& r) { return r.workspaceSize > lib.workspace_bytes; }),
+                found.end());
+    if (found.empty()) raise(TQE_ERR_DEVICE, "hipBLASLt has no kernel for a product of %lld x %lld x %lld", (long long)m, (long long)n, (long long)k);
+    if (it == lib.plans.end()) {
+        plan.algo = found[0].algo;
+        it = lib.plans.emplace(key, plan).first;
+    }
+    if (proposals) *proposals = found;
+    return it->second;
+}
+
+void run_plan(Library& lib, const Library::Plan& plan, const hipblasLtMatmulAlgo_t& algo, const void* w, const void* x, void* out, hipStream_t stream) {
+    const float alpha = 1.f, beta = 0.f;
+    lt_check(hipblasLtMatmul(lib.handle, plan.desc, &alpha, w, plan.a, x, plan.b, &beta, out, plan.c, out, plan.c, &algo, lib.workspace,
+                             lib.workspace_bytes, stream),
+             "the product");
+}
+
+}  // namespace
+
 void library_gemm(const Tensor& x, const Tensor& w, Tensor& out, hipStream_t stream) {
     const int64_t m = x.shape[0], k = x.shape[1], n = w.shape[0];
     if (x.dtype != BF16 || w.dtype != BF16 || w.shape[1] != k || out.shape[0] != m || out.cols() != n || (out.dtype != BF16 && out.dtype != F32))
@@ -291,42 +345,72 @@ void library_gemm(const Tensor& x, const Tensor& w, Tensor& out, hipStream_t str
     if (m == 0) return;
     Library& lib = library();
     std::lock_guard<std::mutex> lock(lib.mutex);
-    if (!lib.handle) {
-        lt_check(hipblasLtCreate(&lib.handle), "creating the handle");
-        lib.workspace = device_malloc(lib.workspace_bytes);
+    const Library::Plan& plan = plan_for(lib, m, n, k, out.dtype, nullptr, 4);
+    run_plan(lib, plan, plan.algo, w.data, x.data, out.data, stream);
+}
+
+double library_tune(int64_t m, int64_t n, int64_t k, int out_dtype, hipStream_t stream) {
+    if (m < 1 || n < 1 || k < 1 || null_device()) return 0.0;
+    Library& lib = library();
+    std::lock_guard<std::mutex> lock(lib.mutex);
+    std::vector<hipblasLtMatmulHeuristicResult_t> proposals;
+    Library::Plan& plan = plan_for(lib, m, n, k, out_dtype, &proposals, 8);
+    {
+        // beside what the library proposes for the shape, every kernel it has for these types that takes the shape
+        std::vector<hipblasLtMatmulHeuristicResult_t> all;
+        const hipDataType out_type = out_dtype == F32 ? HIP_R_32F : HIP_R_16BF;
+        if (hipblaslt_ext::getAllAlgos(lib.handle, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, HIPBLAS_OP_T, HIPBLAS_OP_N, HIP_R_16BF, HIP_R_16BF, out_type,
+                                       out_type, HIPBLAS_COMPUTE_32F, all) == HIPBLAS_STATUS_SUCCESS) {
+            const float one = 1.f, zero = 0.f;
+            for (hipblasLtMatmulHeuristicResult_t& r : all) {
+                size_t ws = 0;
+                if (hipblaslt_ext::matmulIsAlgoSupported(lib.handle, plan.desc, &one, plan.a, plan.b, &zero, plan.c, plan.c, r.algo, ws) ==
+                        HIPBLAS_STATUS_SUCCESS && ws <= lib.workspace_bytes)
+                    proposals.push_back(r);
+            }
+        }
     }
-    const auto key = std::make_tuple(m, n, k, out.dtype);
-    auto it = lib.plans.find(key);
-    if (it == lib.plans.end()) {
-        // in the library's column-major terms: out^T [n, m] = w [n, k] (the k x n matrix, transposed) * x^T [k, m]
-        Library::Plan plan;
-        lt_check(hipblasLtMatmulDescCreate(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F), "creating a product");
-        const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
-        lt_check(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)), "setting a product");
-        lt_check(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)), "setting a product");
-        lt_check(hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, (uint64_t)k, (uint64_t)n, k), "describing the weight");
-        lt_check(hipblasLtMatrixLayoutCreate(&plan.b, HIP_R_16BF, (uint64_t)k, (uint64_t)m, k), "describing x");
-        lt_check(hipblasLtMatrixLayoutCreate(&plan.c, out.dtype == F32 ? HIP_R_32F : HIP_R_16BF, (uint64_t)n, (uint64_t)m, n), "describing the output");
-        hipblasLtMatmulPreference_t pref;
-        lt_check(hipblasLtMatmulPreferenceCreate(&pref), "creating a preference");
-        lt_check(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &lib.workspace_bytes, sizeof(lib.workspace_bytes)),
-                 "setting the workspace");
-        hipblasLtMatmulHeuristicResult_t found[4];
-        int n_found = 0;
-        lt_check(hipblasLtMatmulAlgoGetHeuristic(lib.handle, plan.desc, plan.a, plan.b, plan.c, plan.c, pref, 4, found, &n_found), "choosing a kernel");
-        hipblasLtMatmulPreferenceDestroy(pref);
-        int pick = -1;
-        for (int i = 0; i < n_found && pick < 0; ++i)
-            if (found[i].workspaceSize <= lib.workspace_bytes) pick = i;
-        if (pick < 0) raise(TQE_ERR_DEVICE, "hipBLASLt has no kernel for a product of %lld x %lld x %lld", (long long)m, (long long)n, (long long)k);
-        plan.algo = found[pick].algo;
-        it = lib.plans.emplace(key, plan).first;
+    // operands of the right sizes with values as the model's are (zeros would let the matrix cores run cooler and faster
+    // than real data does): the weight's and x's memory is filled with the random-weights stream
+    Buffer x((size_t)m * k * 2), w((size_t)n * k * 2), out((size_t)m * n * dtype_size(out_dtype));
+    K::random_normal(x.data(), BF16, (long long)(m * k), 0x1234u, 1.0f, 0, stream);
+    K::random_normal(w.data(), BF16, (long long)(n * k), 0x5678u, 0.02f, 0, stream);
+    hipEvent_t a = nullptr, b = nullptr;
+    hip_check(hipEventCreate(&a), "creating an event");
+    hip_check(hipEventCreate(&b), "creating an event");
+    // one run each (after one that does not count), then the eight fastest again, ten runs each: what is kept is the
+    // fastest of those
+    auto time_one = [&](size_t i, int warm, int reps) -> double {
+        const float alpha = 1.f, beta = 0.f;
+        for (int r = 0; r < warm; ++r)
+            if (hipblasLtMatmul(lib.handle, plan.desc, &alpha, w.data(), plan.a, x.data(), plan.b, &beta, out.data(), plan.c, out.data(), plan.c,
+                                &proposals[i].algo, lib.workspace, lib.workspace_bytes, stream) != HIPBLAS_STATUS_SUCCESS)
+                return 1e30;
+        hip_check(hipEventRecord(a, stream), "recording an event");
+        for (int r = 0; r < reps; ++r)
+            if (hipblasLtMatmul(lib.handle, plan.desc, &alpha, w.data(), plan.a, x.data(), plan.b, &beta, out.data(), plan.c, out.data(), plan.c,
+                                &proposals[i].algo, lib.workspace, lib.workspace_bytes, stream) != HIPBLAS_STATUS_SUCCESS)
+                return 1e30;
+        hip_check(hipEventRecord(b, stream), "recording an event");
+        hip_check(hipEventSynchronize(b), "waiting for the device");
+        float ms = 0.f;
+        hip_check(hipEventElapsedTime(&ms, a, b), "reading a time");
+        return ms * 1000.0 / reps;
+    };
+    std::vector<std::pair<double, size_t>> first;
+    for (size_t i = 0; i < proposals.size(); ++i) first.push_back({time_one(i, 1, 1), i});
+    std::sort(first.begin(), first.end());
+    double best = 1e30;
+    size_t best_i = first.empty() ? 0 : first[0].second;
+    for (size_t r = 0; r < first.size() && r < 8; ++r) {
+        if (first[r].first >= 1e29) break;
+        const double us = time_one(first[r].second, 1, 10);
+        if (us < best) { best = us; best_i = first[r].second; }
     }
-    const Library::Plan& plan = it->second;
-    const float alpha = 1.f, beta = 0.f;
-    lt_check(hipblasLtMatmul(lib.handle, plan.desc, &alpha, w.data, plan.a, x.data, plan.b, &beta, out.data, plan.c, out.data, plan.c, &plan.algo,
-                             lib.workspace, lib.workspace_bytes, stream),
-             "the product");
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    if (best < 1e29) plan.algo = proposals[best_i].algo;
+    return best;
 }
 
 void library_release() {

@@ -71,6 +71,10 @@ void add_product(StepContext& c, Stream& stream, const Tensor& x, const Weight& 
 
 // the library product, bfloat16 in, bfloat16 or float32 out
 void library_gemm(const Tensor& x, const Tensor& w_rows, Tensor& out, hipStream_t stream);
+// Lets the library try the kernels it proposes for a product of m rows with a weight [n, k] and keeps the fastest for
+// later calls of that shape (the first proposal is what an untried shape gets).  Takes some milliseconds per shape;
+// it pays for prompts, whose products are the library's.  Returns the microseconds of the kept kernel.
+double library_tune(int64_t m, int64_t n, int64_t k, int out_dtype, hipStream_t stream);
 void library_release();
 
 // thin typed wrappers over the kernel entry points that several files use

@@ -1,5 +1,7 @@
 #include "model.h"
 
+#include <algorithm>
+
 #include "kernels.h"
 #include "trace.h"
 
@@ -170,6 +172,17 @@ Tensor Model::head_logits(StepContext& c, Stream& stream, float* out) {
     final_norm_->gather_add_norm(c, stream.h, stream.pending, want_rows, n_rows, x);
     linear(c, x, head_, nullptr, F32, false, &logits);
     return logits;
+}
+
+void Model::tune_library(int64_t rows, hipStream_t stream) {
+    if (dtype != BF16 || !on_gpu || !policy().library) return;
+    const int64_t own_rows = policy().mid && policy().packed ? mid_max_rows() : skinny_max_rows();
+    if (rows <= own_rows) return;
+    std::vector<std::pair<int64_t, int64_t>> shapes;
+    for (const auto& b : blocks_) b->product_shapes(shapes);
+    std::sort(shapes.begin(), shapes.end());
+    shapes.erase(std::unique(shapes.begin(), shapes.end()), shapes.end());
+    for (const auto& nk : shapes) library_tune(rows, nk.first, nk.second, BF16, stream);
 }
 
 Json Model::describe() const {

@@ -34,6 +34,9 @@ public:
     // the step's wanted rows, written to `out` (device memory) or to workspace memory.
     Tensor forward(StepContext& c, const CacheStore& cache, float* out = nullptr);
     Json describe() const;
+    // Lets the library try its kernels once for every product of the model at `rows` rows (more than the own kernels
+    // take: fewer never reach the library) and keep the fastest for later calls.
+    void tune_library(int64_t rows, hipStream_t stream);
 
 private:
     BuildEnv env_;

@@ -129,6 +129,8 @@ public:
     // ("qkv.weight"): for inspection
     virtual OwnedPtr held(const std::string& name) const { (void)name; return nullptr; }
     virtual Json describe() const;
+    // the matrix products the part runs through linear(): (n, k) of each weight (what the library can be tuned for)
+    virtual void product_shapes(std::vector<std::pair<int64_t, int64_t>>& out) const { (void)out; }
 };
 
 class Norm : public Part {

@@ -290,6 +290,10 @@ public:
         return nullptr;
     }
     const char* trace_name() const override { return "attn"; }             // the reference's span, src/models/turbo_generic.rs:1920
+    void product_shapes(std::vector<std::pair<int64_t, int64_t>>& out) const override {
+        out.push_back({(int64_t)(n_heads_ + 2 * n_kv_heads_) * head_dim_, hidden_});
+        out.push_back({hidden_, (int64_t)n_heads_ * head_dim_});
+    }
 
     CacheNeed cache_need() const override {
         CacheNeed n;
@@ -504,6 +508,10 @@ public:
         return nullptr;
     }
     const char* trace_name() const override { return "attn-mlp"; }         // the reference's span, src/models/turbo_generic.rs:1922
+    void product_shapes(std::vector<std::pair<int64_t, int64_t>>& out) const override {
+        out.push_back({2 * inter_, hidden_});
+        out.push_back({hidden_, inter_});
+    }
 
     bool folds_norm(const StepContext& c) const override { return fusable(c.n_tokens, w_gate_up_); }
     bool adds_to_stream(const StepContext& c) const override {
@@ -598,6 +606,9 @@ public:
         for (const Role& r : roles_) parts.set(r.role, r.part->describe());
         j.set("parts", parts);
         return j;
+    }
+    void product_shapes(std::vector<std::pair<int64_t, int64_t>>& out) const override {
+        for (const Role& r : roles_) r.part->product_shapes(out);
     }
     CacheNeed cache_need() const override { return mixer_->cache_need(); }
     Norm* first_norm() override { return mixer_norm_.get(); }

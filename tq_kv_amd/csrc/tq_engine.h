@@ -19,7 +19,8 @@
 extern "C" {
 #endif
 
-#define TQE_PAGE 64             /* positions per cache page */
+#define TQE_PAGE 64             /* positions per cache page (the kernel library is asked for its own and must agree) */
+#define TQE_KERNEL_ABI 11       /* the version of the kernel library's interface (tqk_abi_version) this engine is written against */
 #define TQE_MAX_GROUPS 16       /* groups of cached runs a cache may have */
 
 enum {
@@ -249,6 +250,9 @@ tqe_model_t* tqe_model_from_spec(const char* spec_json, int dtype, int on_gpu);
 int tqe_model_set_tensor(tqe_model_t* model, const char* name, const tqe_tensor_t* tensor, int on_device, void* stream);
 int tqe_model_finish(tqe_model_t* model, int strict, void* stream);
 int tqe_model_randomize(tqe_model_t* model, uint64_t seed, void* stream);
+/* Lets the matrix library try the kernels it proposes for every product of the model at `rows` rows (prompts: fewer rows than
+ * the own kernels take never reach the library) and keep the fastest for later steps of that size; some milliseconds a shape. */
+int tqe_model_tune_library(tqe_model_t* model, int rows, void* stream);
 /* JSON: spec, config, dtype, graph_safe, loaded, stop_token_ids, needs (per run), cache_of, tensors (name -> spec) */
 const char* tqe_model_describe(const tqe_model_t* model);
 /* where a loaded tensor lives, by its name (tensors folded into others are gone: "layer prefix + qkv.weight",

@@ -166,6 +166,12 @@ class Model:
                                                               native.dtype_code(store_dtype)))
         return str(folder)
 
+    def tune_library(self, rows):
+        """Let the matrix library try its kernels once for every product of the model at `rows` rows (more than the own
+        kernels take: fewer never reach the library) and keep the fastest for later steps of that size.  Takes some
+        milliseconds per distinct weight shape."""
+        native.check(self._lib.tqe_model_tune_library(self.handle, int(rows), native.current_stream() if self.on_gpu else None))
+
     def __repr__(self):
         s = self.spec
         return "Model(architecture=%s, layers=%d, runs=%d, hidden=%d, vocab=%d, dtype=%s)" % (

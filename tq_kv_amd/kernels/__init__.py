@@ -33,6 +33,10 @@ def library():
         lib.tqk_abi_version.restype = ctypes.c_int
         lib.tqk_sample_scratch_bytes.restype = ctypes.c_size_t
         lib.tqk_gemm_scratch_bytes.restype = ctypes.c_size_t
+        from .. import native
+        if int(lib.tqk_page_size()) != native.page_size():
+            raise KernelError("the kernel library's cache pages hold %d positions, the engine library's %d: build both from the same sources"
+                              % (lib.tqk_page_size(), native.page_size()))
         _LIB = lib
     return _LIB
 
@@ -100,6 +104,35 @@ def random_normal(out, key, std, plus_one=False):
     _check(library().tqk_random_normal(_dev(out, "out"), _code(out.dtype), ctypes.c_longlong(out.numel()),
                                        ctypes.c_uint64(int(key) & 0xFFFFFFFFFFFFFFFF), ctypes.c_float(std),
                                        1 if plus_one else 0, _stream()), "random_normal")
+    return out
+
+
+def gather_rows(src, rows, out):
+    """out[r] = src[rows[r]]: rows of any dtype and width gathered by int32 index (at most 65535 of them)."""
+    n = rows.shape[0]
+    row_bytes = src[0].numel() * src.element_size() if src.shape[0] else 0
+    if out.shape[0] != n or out.dtype != src.dtype or tuple(out.shape[1:]) != tuple(src.shape[1:]):
+        raise KernelError("gather_rows: out is %s of %s for %d rows of %s" % (tuple(out.shape), out.dtype, n, tuple(src.shape)))
+    if n and (int(rows.min()) < 0 or int(rows.max()) >= src.shape[0]):
+        raise KernelError("gather_rows: a row index outside the %d rows" % src.shape[0])
+    _check(library().tqk_gather_rows(_dev(src, "src"), _dev(rows, "rows", torch.int32, (n,)), n, ctypes.c_longlong(row_bytes),
+                                     _dev(out, "out"), _stream()), "gather_rows")
+    return out
+
+
+def add_bias(x, bias):
+    """In place: x[r, :] += bias; x [rows, n], bias [n]; float32 or bfloat16 each."""
+    rows, n = x.shape
+    _check(library().tqk_add_bias(_dev(x, "x"), _code(x.dtype), _dev(bias, "bias", None, (n,)), _code(bias.dtype), rows, n, _stream()), "add_bias")
+    return x
+
+
+def convert(src, out):
+    """out = src in out's dtype (float32 and bfloat16)."""
+    if src.numel() != out.numel():
+        raise KernelError("convert: %d values into %d" % (src.numel(), out.numel()))
+    _check(library().tqk_convert(_dev(src, "src"), _code(src.dtype), _dev(out, "out"), _code(out.dtype), ctypes.c_longlong(src.numel()),
+                                 _stream()), "convert")
     return out
 
 

@@ -178,7 +178,7 @@ def library():
                 ("tqe_trace_enabled", []), ("tqe_register_part", [S, S, ctypes.POINTER(tqe_part_callbacks), P]),
                 ("tqe_register_init", [S, INIT_FILL, P]),
                 ("tqe_model_set_tensor", [P, S, T, I, P]), ("tqe_model_finish", [P, I, P]), ("tqe_model_randomize", [P, U64, P]),
-                ("tqe_model_tensor", [P, S, T]), ("tqe_model_set_stop_tokens", [P, I, _I32P]),
+                ("tqe_model_tensor", [P, S, T]), ("tqe_model_tune_library", [P, I, P]), ("tqe_model_set_stop_tokens", [P, I, _I32P]),
                 ("tqe_write_random_folder", [S, S, U64, I]), ("tqe_random_stream", [U64, S, I64, I64, ctypes.POINTER(ctypes.c_float)]),
                 ("tqe_random_stream_of_key", [U64, I64, I64, ctypes.POINTER(ctypes.c_float)]), ("tqe_check_weights", [P, S, I]), ("tqe_write_safetensors", [S, S, ctypes.POINTER(P), S]),
                 ("tqe_part_set_tensor", [P, S, T, I, P]), ("tqe_part_finish", [P, P]), ("tqe_part_tensor", [P, S, T]),
