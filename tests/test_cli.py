@@ -95,3 +95,38 @@ def test_tq_generate_on_a_folder_written_by_tq_random_weights_emits_the_plain_to
     assert c.returncode == 0, c.stderr
     got = json.loads(c.stdout.strip().splitlines()[-1])["outputs"]
     assert got == [plain.generate_greedy(weights, cfg, p, 7, eos_ids=(stop,)) for p in prompts] and len(got[1]) <= 3
+
+
+@pytest.mark.gpu
+def test_tq_generate_takes_text_where_the_folder_holds_a_tokenizer(tmp_path):
+    """`tq generate --prompt TEXT`: the folder's tokenizer.json turns the text into ids (no special tokens added, as
+    src/engine.rs:342-345) and the answer back into text; with -s the text is wrapped in the reference's chat template
+    first.  The ids that reach the model are checked through what it generates: the plain implementation's tokens."""
+    import helpers
+    import plain_qwen2 as plain
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    words = ["<unk>", "<|im_start|>", "<|im_end|>"] + ["w%d" % i for i in range(40)] + ["system", "user", "assistant", "hello", "there"]
+    tok = Tokenizer(models.WordLevel({w: i for i, w in enumerate(words)}, unk_token="<unk>"))
+    tok.pre_tokenizer = pre_tokenizers.WhitespaceSplit()
+    tq = [sys.executable, os.path.join(ROOT, "bin", "tq")]
+    cfg_path = tmp_path / "shape.json"
+    cfg_path.write_text(json.dumps(helpers.TINY_A))
+    folder = str(tmp_path / "model")
+    assert subprocess.run(tq + ["random-weights", str(cfg_path), folder, "--seed", "3", "--store", "float32"], capture_output=True).returncode == 0
+    tok.save(os.path.join(folder, "tokenizer.json"))
+    cfg, weights = helpers.read_folder(folder)
+    text = "hello there w3 w17 w5"
+    ids = tok.encode(text, add_special_tokens=False).ids
+    assert ids == [words.index(w) for w in text.split()]
+    want = plain.generate_greedy(weights, cfg, ids, 6, eos_ids=(2,))            # <|im_end|> is one of the reference's stop strings
+    run = subprocess.run(tq + ["--fp32", "generate", folder, "--prompt", text, "-n", "6", "-t", "0", "--repeat-penalty", "1.0"],
+                         capture_output=True, text=True)
+    assert run.returncode == 0, run.stderr
+    assert run.stdout.strip() == tok.decode(want, skip_special_tokens=True) and "Prompt tokens: 5" in run.stderr
+    as_json = subprocess.run(tq + ["--fp32", "generate", folder, "--prompt", text, "-n", "6", "-t", "0", "--repeat-penalty", "1.0", "--json"],
+                             capture_output=True, text=True)
+    assert json.loads(as_json.stdout.strip().splitlines()[-1])["outputs"] == [want]
+    # without a tokenizer.json the text cannot be taken
+    os.remove(os.path.join(folder, "tokenizer.json"))
+    bad = subprocess.run(tq + ["generate", folder, "--prompt", text], capture_output=True, text=True)
+    assert bad.returncode != 0 and "tokenizer.json" in bad.stderr

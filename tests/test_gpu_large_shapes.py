@@ -209,7 +209,7 @@ def test_prompts_of_two_thousand_tokens_and_graphed_decoding_at_7b_sizes():
     n_first = sum(len(w) for w in wants)
 
     def run(dtype, spoil=False):
-        eng = Engine(build(raw, dtype, tensors), max_tokens=len(lens) * 2240)
+        eng = Engine(build(raw, dtype, tensors), max_tokens=len(lens) * 2240)        # (the tensors of the seed at hand)
         slots = [eng.open() for _ in prompts]
         got = [eng.step([(s, p, w) for s, p, w in zip(slots, prompts, wants)])]
         if spoil:          # sequence 0's page 10 (positions 640..703) becomes sequence 2's, in every layer
@@ -244,14 +244,26 @@ def test_prompts_of_two_thousand_tokens_and_graphed_decoding_at_7b_sizes():
     want = plain_rows(tensors, dict(raw), seq, rows)
     got = torch.cat([f32[:len(wants[0])]] + [f32[n_first + len(lens) * i][None] for i in range(8)])
     torch.testing.assert_close(got, want, atol=2e-5 * max(1.0, want.abs().max().item()), rtol=2e-5)
-    # a foreign page is noticed, in the sequence it belongs to and nowhere else
-    spoiled, _ = run("bfloat16", spoil=True)
-    rms, _ = row_errors(spoiled, bf16_plain_kernel)
+    # a foreign page is noticed, in the sequence it belongs to and nowhere else; on three sets of weights, so that the
+    # distance between a clean run (under 0.02 of the spread) and a spoiled one (over 0.03) is known to hold
     decoded_0 = [n_first + len(lens) * i for i in range(8)]
-    others = [r for r in range(spoiled.shape[0]) if r not in decoded_0]
-    assert rms[decoded_0].min().item() > 0.03, rms[decoded_0]
-    assert rms[others].max().item() < 0.02, rms[others].max()
-    print("rms of the spoiled sequence's rows", rms[decoded_0], "largest of the others", rms[others].max())
+    for seed in (6, 16, 26):
+        if seed != 6:
+            tensors = sharpened(tensors_for(raw, seed))
+            POLICY.update(decode_mfma=False, prefill_mfma=False)
+            try:
+                bf16_plain_kernel, _ = run("bfloat16")
+            finally:
+                POLICY.update(old)
+            clean, _ = run("bfloat16")
+            rms, worst = row_errors(clean, bf16_plain_kernel)
+            assert rms.max().item() < 0.02 and worst.max().item() < 0.1, (seed, rms.max().item(), worst.max().item())
+        spoiled, _ = run("bfloat16", spoil=True)
+        rms, _ = row_errors(spoiled, bf16_plain_kernel)
+        others = [r for r in range(spoiled.shape[0]) if r not in decoded_0]
+        assert rms[decoded_0].min().item() > 0.03, (seed, rms[decoded_0])
+        assert rms[others].max().item() < 0.02, (seed, rms[others].max())
+        print("seed", seed, "rms of the spoiled sequence's rows", rms[decoded_0], "largest of the others", rms[others].max())
 
 
 def test_a_step_of_more_than_three_thousand_tokens_takes_the_wide_tiles():

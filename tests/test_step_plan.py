@@ -138,3 +138,51 @@ def test_runs_of_pages_lie_an_odd_number_of_pages_apart():
     c.reserve([(a, 32 * PAGE), (b, 32 * PAGE)])
     assert sorted(c.pages(0, a) + c.pages(0, b)) == list(range(64))
     c.check()
+
+
+def test_the_library_refuses_negative_counts_and_changes_nothing():
+    """What no caller of the engine can send but a C caller might: negative numbers of wanted places or of new
+    positions.  Each is a status and a message (no exception escapes the library), and nothing was changed."""
+    c = native.NativeCache(3, [(8, 0)])
+    a, b = c.acquire(), c.acquire()
+    i32 = lambda *v: np.asarray(v, dtype=np.int32)
+    with pytest.raises(native.EngineLibraryError, match="wants -1 places"):
+        native.plan_step(c, i32(a), i32(0), i32(1), i32(5), i32(-1), i32(), 1)
+    with pytest.raises(native.EngineLibraryError, match="-3 new positions"):
+        c.reserve([(a, 2), (b, -3)])
+    assert c.pages(0, a) is None and c.counts(0) == (8, 8)
+    c.reserve([(a, 70), (b, 1)])
+    with pytest.raises(native.EngineLibraryError, match="-1000000000 new positions"):
+        c.commit([(a, 70), (b, -10 ** 9)])
+    assert c.length(a) == 0 and c.length(b) == 0                   # commit is all or nothing: a was not committed either
+    with pytest.raises(AssertionError, match="slot 2 is not held"):
+        c.commit([(a, 70), (2, 1)])
+    assert c.length(a) == 0
+    with pytest.raises(AssertionError, match="were not reserved"):
+        c.commit([(a, 200)])
+    c.commit([(a, 70), (b, 1)])
+    assert (c.length(a), c.length(b)) == (70, 1)
+    # a reservation that is given back: the pages beyond what the lengths need are free again
+    c.reserve([(a, 100), (b, 64)])
+    assert c.counts(0)[0] == 8 - 3 - 2
+    c.trim([a, b])
+    assert c.counts(0)[0] == 8 - 2 - 1 and len(c.pages(0, a)) == 2 and len(c.pages(0, b)) == 1
+    c.check()
+
+
+def test_pages_that_were_passed_over_come_back_into_use_on_an_engine_that_is_never_idle():
+    """Requests that overlap for ever: some sequence is always live, so the pool is never wholly free.  The pages that
+    were passed over to space the runs must not pile up at the end of the free list for good: after many rounds a new
+    prompt still gets a run of neighbouring pages."""
+    c = native.NativeCache(4, [(6 * 40, 0)])
+    live = [c.acquire()]
+    c.reserve([(live[0], 32 * PAGE)]), c.commit([(live[0], 32 * PAGE)])
+    for round_ in range(200):
+        s = c.acquire()
+        c.reserve([(s, 32 * PAGE)]), c.commit([(s, 32 * PAGE)])
+        pages = c.pages(0, s)
+        assert pages == list(range(pages[0], pages[0] + 32)), (round_, pages)          # a run of neighbours every time
+        live.append(s)
+        c.release(live.pop(0))                                                      # the older one ends: never idle
+        c.check()
+    assert c.counts(0)[0] == 6 * 40 - 32

@@ -18,8 +18,8 @@ import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["host.cpp", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip",
-           "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip", "random_init.hip", "utility.hip"]
-HEADERS = ["common.h", "tq_kernels.h"]
+           "attention_decode.hip", "attention_prefill.hip", "skinny_fused.hip", "mid_product.hip", "random_init.hip", "utility.hip", "probe.hip"]
+HEADERS = ["common.h", "tq_kernels.h", "tq_no_alloc.h"]
 # the engine: host code only (config, weights, parts, model, cache, step, loop), built with the host compiler into a
 # library of its own that reaches the GPU through the HIP runtime, hipBLASLt and the kernel library above
 HOST_SOURCES = ["host_engine.cpp"] + ["engine/" + n for n in (

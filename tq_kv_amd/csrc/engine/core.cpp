@@ -102,43 +102,87 @@ void device_synchronize() {
 static size_t round_up(size_t n, size_t to) { return (n + to - 1) / to * to; }
 
 void Workspace::reserve(size_t bytes) {
-    chunks_.clear();
-    chunks_.emplace_back();
-    chunks_.back().mem.allocate(round_up(std::max<size_t>(bytes, 256), 256));
-    step_ = 0;
+    Arena& a = arenas_[current_];
+    a.chunks.clear();
+    a.chunks.emplace_back();
+    a.chunks.back().mem.allocate(round_up(std::max<size_t>(bytes, 256), 256));
+    a.at = a.held = 0;
+}
+
+void Workspace::reserve_like(const Workspace& measured, size_t more_for_the_step) {
+    for (int i = 0; i < N_ARENAS; ++i) {
+        const size_t need = measured.arenas_[i].high + (i == STEP ? more_for_the_step : 0);
+        Arena& a = arenas_[i];
+        a.chunks.clear();
+        a.at = a.held = 0;
+        if (need == 0) continue;
+        a.chunks.emplace_back();
+        a.chunks.back().mem.allocate(round_up(need, 256));
+    }
 }
 
 size_t Workspace::capacity() const {
     size_t n = 0;
-    for (const Chunk& c : chunks_) n += c.mem.bytes();
+    for (const Arena& a : arenas_)
+        for (const Chunk& c : a.chunks) n += c.mem.bytes();
+    return n;
+}
+
+size_t Workspace::high_water() const {
+    size_t n = 0;
+    for (const Arena& a : arenas_) n += a.high;
     return n;
 }
 
 void Workspace::reset(hipStream_t stream) {
-    if (chunks_.size() > 1 && !fixed_) {
-        // what the last step needed, in one piece: first let that step finish
-        const size_t want = capacity() + capacity() / 4;
-        stream_synchronize(stream);
-        reserve(want);
+    bool waited = false;
+    for (Arena& a : arenas_) {
+        if (a.chunks.size() > 1 && !fixed_) {
+            // what the arena needed at most, in one piece: first let the last step finish
+            if (!waited) stream_synchronize(stream);
+            waited = true;
+            const size_t want = a.high + a.high / 8;
+            a.chunks.clear();
+            a.chunks.emplace_back();
+            a.chunks.back().mem.allocate(round_up(std::max<size_t>(want, 256), 256));
+        }
+        for (Chunk& c : a.chunks) c.used = 0;
+        a.at = a.held = a.high = 0;
     }
-    for (Chunk& c : chunks_) c.used = 0;
-    step_ = 0;
+    current_ = STEP;
 }
 
-void* Workspace::alloc(size_t bytes) {
+void Workspace::rewind(int arena) {
+    Arena& a = arenas_[arena];
+    for (Chunk& c : a.chunks) c.used = 0;
+    a.at = a.held = 0;
+}
+
+int Workspace::arena_of(const void* p) const {
+    for (int i = 0; i < N_ARENAS; ++i)
+        for (const Chunk& c : arenas_[i].chunks)
+            if (p >= c.mem.data() && p < (const char*)c.mem.data() + c.mem.bytes()) return i;
+    return -1;
+}
+
+void* Workspace::alloc_in(int arena, size_t bytes) {
+    Arena& a = arenas_[arena];
     bytes = round_up(std::max<size_t>(bytes, 1), 256);
-    if (chunks_.empty() || chunks_.back().used + bytes > chunks_.back().mem.bytes()) {
-        if (fixed_ && !chunks_.empty())
+    while (a.at < a.chunks.size() && a.chunks[a.at].used + bytes > a.chunks[a.at].mem.bytes()) ++a.at;
+    if (a.at >= a.chunks.size()) {
+        if (fixed_)
             raise(TQE_ERR_DEVICE, "a captured step's workspace of %zu bytes is too small (%zu more asked for)", capacity(), bytes);
-        const size_t grow = std::max(bytes, std::max<size_t>(capacity(), (size_t)8 << 20));
-        chunks_.emplace_back();
-        chunks_.back().mem.allocate(grow);
+        size_t have = 0;
+        for (const Chunk& c : a.chunks) have += c.mem.bytes();
+        a.chunks.emplace_back();
+        a.chunks.back().mem.allocate(std::max(bytes, std::max<size_t>(have / 2, (size_t)4 << 20)));
+        a.at = a.chunks.size() - 1;
     }
-    Chunk& c = chunks_.back();
+    Chunk& c = a.chunks[a.at];
     void* p = (char*)c.mem.data() + c.used;
     c.used += bytes;
-    step_ += bytes;
-    high_ = std::max(high_, step_);
+    a.held += bytes;
+    a.high = std::max(a.high, a.held);
     return p;
 }
 

@@ -110,27 +110,39 @@ private:
 };
 
 // The scratch memory of one step: handed out front to back, all of it given back when the
-// next step starts.  A growing workspace adds a chunk when it runs out and, at the next
-// reset, makes one chunk of everything (after the stream has drained); a fixed one (what a
-// captured graph's kernels point into) refuses instead.
+// next step starts.  A growing workspace adds a chunk to an arena that runs out and, at the
+// next reset, makes one chunk of what that arena needed (after the stream has drained); a fixed
+// one (what a captured graph's kernels point into) refuses instead.
 class Workspace {
 public:
+    // Three arenas, each a bump allocator: what lives for the whole step (STEP), and two that the
+    // layers of a model use in turn, so that the temporaries of a layer go into the memory that the
+    // layer before the last one has left: a step needs the memory of two layers, not of all, and
+    // its kernels meet the same addresses layer after layer.
+    enum { STEP = 0, N_ARENAS = 3 };
     explicit Workspace(bool fixed = false) : fixed_(fixed) {}
-    void reserve(size_t bytes);                  // one chunk of at least so many bytes (drops what it has)
-    void reset(hipStream_t stream);
-    void* alloc(size_t bytes);
+    void reserve(size_t bytes);                  // the current arena: one chunk of at least so many bytes (drops what it has)
+    void reserve_like(const Workspace& measured, size_t more_for_the_step);     // every arena: what `measured` needed since its reset
+    void reset(hipStream_t stream);              // a new step: every arena is empty, the current one is STEP
+    void* alloc(size_t bytes) { return alloc_in(current_, bytes); }
+    void* alloc_for_step(size_t bytes) { return alloc_in(STEP, bytes); }
     Tensor tensor(int dtype, std::initializer_list<int64_t> dims) {
         Tensor t(nullptr, dtype, dims);
         t.data = alloc(t.bytes());
         return t;
     }
-    size_t high_water() const { return high_; }
+    void use(int arena) { current_ = arena; }
+    void rewind(int arena);                      // what the arena holds is no longer needed
+    int arena_of(const void* p) const;           // the arena whose memory p points into, or -1
+    size_t high_water() const;                   // the most that was held at once since the last reset
     size_t capacity() const;
 private:
     struct Chunk { Buffer mem; size_t used = 0; };
-    std::vector<Chunk> chunks_;
+    struct Arena { std::vector<Chunk> chunks; size_t at = 0, held = 0, high = 0; };
+    void* alloc_in(int arena, size_t bytes);
+    Arena arenas_[N_ARENAS];
+    int current_ = STEP;
     bool fixed_;
-    size_t step_ = 0, high_ = 0;
 };
 
 // Pinned host buffers for small uploads, used in turn; a buffer is written again only after

@@ -125,7 +125,6 @@ const float* Engine::graphed_step(StepContext& probe, int n_seqs, const int32_t*
         probe.upload();
         if (device_tokens) copy_on_device((void*)probe.dev.tokens, device_tokens, (size_t)n_seqs * sizeof(int32_t), stream);
         const float* logits = (const float*)model->forward(probe, *cache, logits_out).data;
-        const size_t need = ws_.high_water();
         device_synchronize();
         if ((int)graphs_.size() >= MAX_GRAPHS) {
             release_graph(graphs_.front());
@@ -136,7 +135,7 @@ const float* Engine::graphed_step(StepContext& probe, int n_seqs, const int32_t*
         try {
             g.shape = shape;
             g.flat.allocate(probe.flat_count * sizeof(int32_t));
-            g.ws.reserve(need + logits_bytes + (size_t)(1 << 16));         // the eager run's logits may have gone to the caller's memory
+            g.ws.reserve_like(ws_, logits_bytes + (size_t)(1 << 16));      // the eager run's logits may have gone to the caller's memory
             g.ctx.stream = capture_stream_;
             g.ctx.staging = &staging_;
             g.ctx.act_dtype = model->dtype;

@@ -110,6 +110,13 @@ OwnedPtr Model::held(const std::string& name) const {
     return nullptr;
 }
 
+// whether anything the stream holds lies in this arena of the workspace
+static bool lives_in(const Workspace& ws, const Stream& s, int arena) {
+    for (const void* p : {s.h.data, s.pending.t.data, s.pending.s.sums.data, s.xw_buffer.data, s.ss_buffer.data})
+        if (p && ws.arena_of(p) == arena) return true;
+    return false;
+}
+
 Tensor Model::forward(StepContext& c, const CacheStore& cache, float* out) {
     if (!loaded) raise(TQE_ERR_STATE, "the model has no weights yet");
     Span span("model");                     // the reference's span, src/models/turbo_generic.rs:1932
@@ -142,8 +149,16 @@ Tensor Model::forward(StepContext& c, const CacheStore& cache, float* out) {
         stream.invalidate();            // what the gather prepared for the first norm is of the stream before this
     }
     Stream* cur = &stream;
-    for (size_t i = 0; i < s.order.size(); ++i)
+    for (size_t i = 0; i < s.order.size(); ++i) {
+        // The layers take their temporaries from two arenas in turn.  What a layer leaves for the next one (an update
+        // of the stream that is still pending) is read by that next layer, so the arena of the layer before the last
+        // holds nothing that is still needed: unless a block handed on what it was given, which is looked for.
+        const int arena = 1 + (int)(i & 1);
+        if (!lives_in(*c.ws, *cur, arena)) c.ws->rewind(arena);
+        c.ws->use(arena);
         cur = blocks_[(size_t)s.order[i].layer]->forward(c, cur, cache.entry((int)i), firsts[i + 1], i + 1 == s.order.size());
+    }
+    c.ws->use(Workspace::STEP);
     if (c.n_want == 0) return Tensor(nullptr, F32, {0, s.vocab_size});
     Span out_span("output");                // src/models/turbo_generic.rs:1933
     Tensor logits = head_logits(c, *cur, out);

@@ -87,7 +87,7 @@ Tiles StepContext::upload_tiles(std::vector<int32_t>& seq, std::vector<int32_t>&
     t.n = (int)n;
     if (n == 0) return t;
     if (capturing) raise(TQE_ERR_STATE, "a part asked for query tiles while its step was being captured as a graph (it is not graph_safe)");
-    int32_t* dev_mem = (int32_t*)ws->alloc(host.size() * sizeof(int32_t));
+    int32_t* dev_mem = (int32_t*)ws->alloc_for_step(host.size() * sizeof(int32_t));     // later layers read them too
     staging->upload(dev_mem, host.data(), host.size() * sizeof(int32_t), stream);
     t.seq = dev_mem;
     t.tok0 = dev_mem + n;

@@ -23,6 +23,7 @@
 // the history and u.
 #include "common.h"
 #include "tq_kernels.h"
+#include "tq_no_alloc.h"
 
 #define SAMP_THREADS 1024
 

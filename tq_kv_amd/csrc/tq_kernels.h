@@ -22,6 +22,13 @@ int tqk_skinny_max_rows(void);          /* most rows the skinny products (tqk_fu
 int tqk_mid_max_rows(void);             /* most rows tqk_mid_store and tqk_mid_gated take */
 int tqk_attention_max_head_dim(void);   /* the largest head size any attention kernel here takes (tqk_attention's) */
 
+/* Two probes of the GPU at hand, for a bench to set its figures against (the caller times the launches): a plain streaming read of
+ * `bytes` bytes (a multiple of 16, 16-byte aligned) by all compute units, and `turns` times four 32x32x16 bfloat16 matrix-core
+ * products per wave on operands that stay in registers (*flops_out, on the host: the operations of the launch).  sink: 4 bytes of
+ * device memory. */
+int tqk_probe_read(const void* src, long long bytes, void* sink, void* stream);
+int tqk_probe_mfma(long long turns, void* sink, double* flops_out, void* stream);
+
 /* dst row r = src row rows[r], rows of row_bytes bytes each (at most 65535 rows) */
 int tqk_gather_rows(const void* src, const int32_t* rows, int n_rows, long long row_bytes, void* dst, void* stream);
 /* x[r, :] += bias in place; x [n_rows, n], bias [n] */
@@ -170,19 +177,7 @@ int tqk_swiglu(const void* gate_up, void* out, int act_dtype, int n_tokens, int 
 int tqk_argmax_scratch_floats(int n_rows, int vocab);
 int tqk_argmax(const float* logits, int n_rows, int vocab, int32_t* out, float* scratch, void* stream);
 
-/* tqk_argmax for callers that cannot allocate device memory (code under HIP graph capture, tight
- * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
- * chunks' results go to an array inside the library's image on the current GPU (128 KiB per GPU,
- * held until the process ends) in place of a caller's scratch; n_rows * ceil(vocab / 4096) must
- * not exceed tqk_argmax_static_max_pairs() (16384), more is refused with an error.  It calls no
- * hipMalloc, hipFree or allocating library routine.  Every call on a GPU shares that GPU's array:
- * calls that overlap in time on one GPU (different streams or threads) race; calls on one stream
- * are ordered.  The GPU whose stream is given must be the current one.  The array's address is
- * looked up at the first call on each GPU; tqk_argmax_static_prepare() does that lookup for the
- * current GPU ahead of time (call it before a graph capture that will hold tqk_argmax_static). */
-int tqk_argmax_static_max_pairs(void);
-int tqk_argmax_static_prepare(void);
-int tqk_argmax_static(const float* logits, int n_rows, int vocab, int32_t* out, void* stream);
+/* tqk_argmax_static, the variant that allocates nothing: csrc/tq_no_alloc.h */
 
 /* In place: for every token in the history of the row's request, once per occurrence,
  * l > 0 ? l / penalty : l * penalty.  hist, times [n_req, hist_cap], hist_len [n_req]: the

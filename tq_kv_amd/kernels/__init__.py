@@ -107,6 +107,39 @@ def random_normal(out, key, std, plus_one=False):
     return out
 
 
+def probe_read(buf, repeats=5):
+    """GB/s of a plain streaming read of `buf` (a contiguous tensor of a multiple of 16 bytes) by all compute units: the
+    best of `repeats` timed launches after one that does not count."""
+    n = buf.numel() * buf.element_size()
+    sink = torch.zeros(1, dtype=torch.int32, device=buf.device)
+    best = 0.0
+    for i in range(repeats + 1):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        _check(library().tqk_probe_read(_dev(buf, "buf"), ctypes.c_longlong(n), _dev(sink, "sink"), _stream()), "probe_read")
+        b.record()
+        b.synchronize()
+        if i:
+            best = max(best, n / (a.elapsed_time(b) * 1e-3) / 1e9)
+    return best
+
+
+def probe_mfma(turns=200000, repeats=3):
+    """PFLOP/s of a loop of 32x32x16 bfloat16 matrix-core products on registers, all compute units busy."""
+    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
+    flops = ctypes.c_double(0.0)
+    best = 0.0
+    for i in range(repeats + 1):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        _check(library().tqk_probe_mfma(ctypes.c_longlong(turns if i else 1000), _dev(sink, "sink"), ctypes.byref(flops), _stream()), "probe_mfma")
+        b.record()
+        b.synchronize()
+        if i:
+            best = max(best, flops.value / (a.elapsed_time(b) * 1e-3) / 1e15)
+    return best
+
+
 def gather_rows(src, rows, out):
     """out[r] = src[rows[r]]: rows of any dtype and width gathered by int32 index (at most 65535 of them)."""
     n = rows.shape[0]
