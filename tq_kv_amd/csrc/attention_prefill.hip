@@ -317,9 +317,12 @@ void attention_prefill_kernel(const PrefillArgs p) {
 
     // Two buffers: while a page is worked on, the next one is on its way into registers, and goes
     // into the other buffer afterwards; one barrier per page.
+    // The numbers of the pages are read 64 at a time, a lane each, and handed round inside the wave: a
+    // page's loads then do not wait for the load of its number, which would cost a trip to memory per page.
     const int32_t* pages = p.page_table + (size_t)seq * p.table_width;
+    int my_pages = pages[min(first_page + w.lane, w.last_page)];
     u32x4_t kr[D / 32], vr[D / 32];
-    int page_now = pages[first_page];
+    int page_now = __shfl(my_pages, 0, TQK_WAVE);
     fetch_page<D>(w, page_now, kr, vr);
     stage_page<D>(w, kr, vr, kb + (first_page & 1) * L::K_BYTES, vb + (first_page & 1) * L::V_BYTES);
     for (int pg = first_page; pg <= w.last_page; ++pg) {
@@ -327,7 +330,9 @@ void attention_prefill_kernel(const PrefillArgs p) {
         __syncthreads();                      // the page is whole; all are done with the other buffer
         int page_next = -1;
         if (pg < w.last_page) {
-            page_next = pages[pg + 1];
+            const int ahead = (pg + 1 - first_page) & (TQK_WAVE - 1);
+            if (ahead == 0) my_pages = pages[min(pg + 1 + w.lane, w.last_page)];
+            page_next = __shfl(my_pages, ahead, TQK_WAVE);
             fetch_page<D>(w, page_next, kr, vr);
         }
         page_step<D>(w, pg, page_now, kb + cur * L::K_BYTES, vb + cur * L::V_BYTES);

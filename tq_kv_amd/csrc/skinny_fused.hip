@@ -393,7 +393,9 @@ static int pick_tiles(int N, int K) {
 }
 
 // Waves per block, which split K between them: about a thousand waves on the chip keep HBM
-// busy; no more than there are chunks of K to share out; a power of two.
+// busy; no more than there are chunks of K to share out; a power of two.  (Two and four thousand
+// waves, so that a wave has two rounds of loads instead of four, were measured no faster on the
+// q/k/v and o products of the 7B sizes and slower on the down product.)
 static int pick_waves(int blocks, int K, int tiles) {
     const int chunks = K / (4 * 32) > 0 ? K / (4 * 32) : 1;
     const int max_waves = tiles >= 2 ? 8 : 16;
