@@ -1059,3 +1059,14 @@ def test_attention_prefill_over_thousands_of_keys(nh, nkv, d, spans, tile, windo
             other = attention_reference(qs[0][-1:].float(), ks[0], vs[0], torch.tensor([b - 1]), 0 if window else 1000, scale)
             assert (other - out[off + n - 1:off + n].float().cpu()).abs().max() > 0.1
         off += n
+
+
+def test_the_probes_read_and_multiply():
+    """What the bench sets its figures against: a streaming read and a loop of matrix-core products.  Their figures are
+    the GPU's; here only that they run, read every shape of grid they are asked for, and refuse what they cannot do."""
+    buf = torch.ones(1 << 24, dtype=torch.float32, device=DEV)            # 64 MB
+    assert K.probe_read(buf, repeats=2) > 200.0                              # GB/s: any GPU this runs on does that
+    assert K.probe_read(buf[:4 * 1000 + 4], repeats=1, shapes=((3, 64), (7, 128))) > 0.0     # regions that do not divide evenly
+    assert K.probe_mfma(turns=2000, repeats=1) > 0.01                       # PFLOP/s
+    with pytest.raises(K.KernelError, match="blocks of 96 threads"):
+        K.probe_read(buf, repeats=1, shapes=((8, 96),))

@@ -150,7 +150,7 @@ void mid_product_kernel(const MidArgs p) {
         for (int u = 0; u < 4; ++u) {
             const size_t at = (size_t)min(c / 32 + u, K / 32 - 1) * 512;
 #pragma unroll
-            for (int t = 0; t < TN; ++t) a[t][u] = *reinterpret_cast<const bf16x8_t*>(wtile[t] + at);
+            for (int t = 0; t < TN; ++t) a[t][u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wtile[t] + at));      // read once
         }
     };
     // x comes from LDS four row groups at a time (two where registers are short), the next ones on
@@ -182,7 +182,7 @@ void mid_product_kernel(const MidArgs p) {
                 if (grp == NG - 1) {
                     const size_t at = (size_t)min(refill_c / 32 + u, K / 32 - 1) * 512;
 #pragma unroll
-                    for (int t = 0; t < TN; ++t) a[t][u] = *reinterpret_cast<const bf16x8_t*>(wtile[t] + at);
+                    for (int t = 0; t < TN; ++t) a[t][u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(wtile[t] + at));      // read once
                 }
                 __builtin_amdgcn_sched_barrier(0);       // or the reads of many steps are issued at once and held
             }

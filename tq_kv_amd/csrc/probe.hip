@@ -10,18 +10,21 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
-// every thread reads 16-byte pieces a whole grid apart, four under way at a time; the sum keeps the loads alive
+// every block reads a region of its own front to back, four pieces of 16 bytes per thread under way; the loads say
+// that nothing is read twice; the sum keeps them alive
 __global__ __launch_bounds__(256)
 void probe_read_kernel(const u32x4_t* __restrict__ src, long long n16, uint32_t* __restrict__ sink) {
-    const long long stride = (long long)gridDim.x * blockDim.x;
-    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long per = (n16 + gridDim.x - 1) / gridDim.x;
+    const long long begin = per * blockIdx.x, end = begin + per < n16 ? begin + per : n16;
     u32x4_t acc = {0u, 0u, 0u, 0u};
-    for (; i + 3 * stride < n16; i += 4 * stride) {
-        const u32x4_t a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + stride);
-        const u32x4_t c = __builtin_nontemporal_load(src + i + 2 * stride), d = __builtin_nontemporal_load(src + i + 3 * stride);
+    const long long step = blockDim.x;
+    long long i = begin + threadIdx.x;
+    for (; i + 3 * step < end; i += 4 * step) {
+        const u32x4_t a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + step);
+        const u32x4_t c = __builtin_nontemporal_load(src + i + 2 * step), d = __builtin_nontemporal_load(src + i + 3 * step);
         acc ^= a ^ b ^ c ^ d;
     }
-    for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+    for (; i < end; i += step) acc ^= __builtin_nontemporal_load(src + i);
     const uint32_t v = acc.x ^ acc.y ^ acc.z ^ acc.w;
     if (v == 0x9E3779B9u) sink[0] = v;              // (never, in practice: the store is only there so that the loads are)
 }
@@ -45,13 +48,15 @@ void probe_mfma_kernel(long long turns, float* __restrict__ sink) {
 
 }  // namespace
 
-/* Reads `bytes` bytes (a multiple of 16, 16-byte aligned) once, by 16 blocks of 256 threads per compute unit.  sink: 4 bytes of
- * device memory (nothing meaningful is written).  The caller times the launch: bytes / time is what a kernel that only reads can reach. */
-extern "C" int tqk_probe_read(const void* src, long long bytes, void* sink, void* stream) {
+/* Reads `bytes` bytes (a multiple of 16, 16-byte aligned) once, by `blocks` blocks of `threads` threads (64, 128 or 256; blocks 0:
+ * two blocks of 256 per compute unit), each block a region of its own.  sink: 4 bytes of device memory (nothing meaningful is
+ * written).  The caller times the launch and tries several shapes: bytes / time of the best is what a kernel that only reads reaches. */
+extern "C" int tqk_probe_read(const void* src, long long bytes, int blocks, int threads, void* sink, void* stream) {
     TQK_REQUIRE(src && sink && bytes > 0 && bytes % 16 == 0 && (((uintptr_t)src) & 15) == 0, "tqk_probe_read: needs a 16-byte aligned buffer of a multiple of 16 bytes");
+    TQK_REQUIRE(blocks >= 0 && blocks <= (1 << 20) && (threads == 64 || threads == 128 || threads == 256), "tqk_probe_read: %d blocks of %d threads", blocks, threads);
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    probe_read_kernel<<<cus * 16, 256, 0, (hipStream_t)stream>>>((const u32x4_t*)src, bytes / 16, (uint32_t*)sink);
+    probe_read_kernel<<<blocks ? blocks : cus * 2, threads, 0, (hipStream_t)stream>>>((const u32x4_t*)src, bytes / 16, (uint32_t*)sink);
     return tqk_check_launch("tqk_probe_read");
 }
 

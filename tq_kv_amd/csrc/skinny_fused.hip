@@ -59,6 +59,11 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
 __device__ __forceinline__ bf16x8_t load8f(const bf16_t* p) {
     return *reinterpret_cast<const bf16x8_t*>(p);
 }
+// the weights: read once and never again, so the load says so (a plain streaming read of a gigabyte runs at
+// 7.0 TB/s with this hint and at 6.2 without it on an MI355X)
+__device__ __forceinline__ bf16x8_t load8w(const bf16_t* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(p));
+}
 
 enum { EPI_STORE = 0, EPI_GATED = 1, EPI_RESIDUAL = 2, EPI_QKV = 3 };
 
@@ -199,7 +204,7 @@ void skinny_fused_kernel(const FusedArgs p) {
         for (int u = 0; u < SF_UNROLL; ++u) {
             const int k0 = min(wave * chunk + u * 32, K - 32);
 #pragma unroll
-            for (int t = 0; t < TILES; ++t) a[t][u] = load8f(wrow[t] + (size_t)k0 * kmul);
+            for (int t = 0; t < TILES; ++t) a[t][u] = load8w(wrow[t] + (size_t)k0 * kmul);
             bx[u] = load8f(xrow + k0);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -234,7 +239,7 @@ void skinny_fused_kernel(const FusedArgs p) {
 #pragma unroll
         for (int u = 0; u < SF_UNROLL; ++u) {
 #pragma unroll
-            for (int t = 0; t < TILES; ++t) a[t][u] = load8f(wrow[t] + (size_t)(k0 + u * 32) * kmul);
+            for (int t = 0; t < TILES; ++t) a[t][u] = load8w(wrow[t] + (size_t)(k0 + u * 32) * kmul);
             bx[u] = load8f(xrow + k0 + u * 32);
         }
         __builtin_amdgcn_sched_barrier(0);          // every load of the chunk is on its way before the first product waits
@@ -245,7 +250,7 @@ void skinny_fused_kernel(const FusedArgs p) {
         const bf16x8_t bxs = load8f(xrow + k0);
 #pragma unroll
         for (int t = 0; t < TILES; ++t)
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load8f(wrow[t] + (size_t)k0 * kmul), bxs, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load8w(wrow[t] + (size_t)k0 * kmul), bxs, acc[t], 0, 0, 0);
     }
 
     if (NORM) {

@@ -23,10 +23,11 @@ int tqk_mid_max_rows(void);             /* most rows tqk_mid_store and tqk_mid_g
 int tqk_attention_max_head_dim(void);   /* the largest head size any attention kernel here takes (tqk_attention's) */
 
 /* Two probes of the GPU at hand, for a bench to set its figures against (the caller times the launches): a plain streaming read of
- * `bytes` bytes (a multiple of 16, 16-byte aligned) by all compute units, and `turns` times four 32x32x16 bfloat16 matrix-core
+ * `bytes` bytes (a multiple of 16, 16-byte aligned) by `blocks` blocks of `threads` threads (blocks 0: two of 256 per compute unit;
+ * the caller tries several shapes and keeps the best), and `turns` times four 32x32x16 bfloat16 matrix-core
  * products per wave on operands that stay in registers (*flops_out, on the host: the operations of the launch).  sink: 4 bytes of
  * device memory. */
-int tqk_probe_read(const void* src, long long bytes, void* sink, void* stream);
+int tqk_probe_read(const void* src, long long bytes, int blocks, int threads, void* sink, void* stream);
 int tqk_probe_mfma(long long turns, void* sink, double* flops_out, void* stream);
 
 /* dst row r = src row rows[r], rows of row_bytes bytes each (at most 65535 rows) */

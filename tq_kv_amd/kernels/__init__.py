@@ -107,20 +107,22 @@ def random_normal(out, key, std, plus_one=False):
     return out
 
 
-def probe_read(buf, repeats=5):
-    """GB/s of a plain streaming read of `buf` (a contiguous tensor of a multiple of 16 bytes) by all compute units: the
-    best of `repeats` timed launches after one that does not count."""
+def probe_read(buf, repeats=5, shapes=((0, 256), (1024, 256), (2048, 64), (4096, 64), (4096, 256))):
+    """GB/s of a plain streaming read of `buf` (a contiguous tensor of a multiple of 16 bytes): the best timed launch of
+    `repeats` for each of a few grid shapes (blocks, threads per block; 0 blocks: two per compute unit), after one launch
+    each that does not count.  How many waves stream at once moves the figure by a fifth, so the best shape is the probe."""
     n = buf.numel() * buf.element_size()
     sink = torch.zeros(1, dtype=torch.int32, device=buf.device)
     best = 0.0
-    for i in range(repeats + 1):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        _check(library().tqk_probe_read(_dev(buf, "buf"), ctypes.c_longlong(n), _dev(sink, "sink"), _stream()), "probe_read")
-        b.record()
-        b.synchronize()
-        if i:
-            best = max(best, n / (a.elapsed_time(b) * 1e-3) / 1e9)
+    for blocks, threads in shapes:
+        for i in range(repeats + 1):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            _check(library().tqk_probe_read(_dev(buf, "buf"), ctypes.c_longlong(n), int(blocks), int(threads), _dev(sink, "sink"), _stream()), "probe_read")
+            b.record()
+            b.synchronize()
+            if i:
+                best = max(best, n / (a.elapsed_time(b) * 1e-3) / 1e9)
     return best
 
 
