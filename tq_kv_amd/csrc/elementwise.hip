@@ -555,7 +555,9 @@ static int rope_store(const void* qkv, const PartSums ps, int act_dtype, const v
         ((((uintptr_t)qkv) | ((uintptr_t)ps.sums) | ((uintptr_t)bias) | ((uintptr_t)cos_table) | ((uintptr_t)sin_table) |
           ((uintptr_t)keys) | ((uintptr_t)q_out)) & 15) == 0) {
         const int slots = (n_heads + 2 * n_kv_heads) * (head_dim / 8);
-        const bool values_apart = write_kv && n_tokens >= STORE_VALUES_MIN_TOKENS;
+        // (lanes along the tokens pay where neighbouring tokens share a page: prompts, not steps of one token per sequence,
+        // where 128 sequences took 20 us that way and take 8 the plain way)
+        const bool values_apart = write_kv && n_tokens >= STORE_VALUES_MIN_TOKENS && n_tokens >= 8 * n_seqs;
         const int layers = (slots + 255) / 256;
         dim3 vgrid(n_tokens, layers + (values_apart ? 1 : 0));
         rope_store_halves_bf16_kernel<<<vgrid, 256, 0, s>>>(
