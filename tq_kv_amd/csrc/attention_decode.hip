@@ -1,6 +1,6 @@
 // Attention for decoding: one new token per sequence attends over its sequence's pages
 // of the cache.  bfloat16 in, MFMA, float32 softmax.  Bound by the bytes of keys and
-// values, so the work is cut for memory: a block of 4 waves per (sequence, kv head,
+// values, so the work is cut for memory: a block of 4 waves (2 in large grids) per (sequence, kv head,
 // partition of the pages); the partitions take the live pages in turn (partition p the pages
 // first + p, first + p + parts, ...: however long the sequence is, they get the same share)
 // and so do the four waves inside a partition; all
@@ -37,9 +37,9 @@ union pack8 {
     uint4 q;
 };
 
-#define AD_WAVES 4
+#define AD_WAVES 4            // the most; blocks of 2 where the grid alone is more than the memory can serve at once
 
-template <int D, bool NT>
+template <int D, bool NT, int W>
 __global__ __launch_bounds__(AD_WAVES * TQK_WAVE)
 void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ keys,
                              const bf16_t* __restrict__ values, const int32_t* __restrict__ tok_pos,
@@ -50,7 +50,7 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     constexpr int KB = D / 32;          // k-blocks of the score product
     constexpr int DB = D / 16;          // 16-element blocks of the output
     constexpr int ROW = DB * 4 + 2;     // floats a lane hands over: its out^T values, m, l
-    __shared__ float xch[(AD_WAVES - 1) * TQK_WAVE * ROW];
+    __shared__ float xch[(W - 1) * TQK_WAVE * ROW];
     const int wave = threadIdx.x / TQK_WAVE, lane = threadIdx.x % TQK_WAVE;
     const int col = lane % 16, g = lane / 16;
     const int part = blockIdx.x;
@@ -88,7 +88,7 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 
         const int32_t* pages = page_table + (size_t)seq * table_width;
         const size_t page_stride = (size_t)n_kv_heads * TQK_PAGE * D;
-        for (int pg = start_page; pg <= last_page; pg += AD_WAVES * n_parts) {
+        for (int pg = start_page; pg <= last_page; pg += W * n_parts) {
             const int page = pages[pg];
             if (page < 0) continue;                     // the host never lets this happen
             const bf16_t* kp = keys + (size_t)page * page_stride + (size_t)kvh * TQK_PAGE * D;
@@ -193,7 +193,7 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     __syncthreads();
     const size_t row = ((size_t)seq * n_heads + head) * n_parts + part;
     if (wave == 0) {
-        for (int w = 1; w < AD_WAVES; ++w) {
+        for (int w = 1; w < W; ++w) {
             const float* theirs = xch + ((size_t)(w - 1) * TQK_WAVE + lane) * ROW;
             const float m2 = theirs[DB * 4], l2 = theirs[DB * 4 + 1];
             if (m2 == -INFINITY) continue;
@@ -277,9 +277,13 @@ extern "C" int tqk_attention_decode(const void* q, const void* keys, const void*
     // caches hold (64 sequences of 2100 positions at the 7B sizes: 56.2 against 57.5 us) and costs where it reads little
     // (8 sequences: 14.4 against 13.6 us), so it goes by the most that the step's tables can name.
     const bool nt = (double)n_seqs * table_width * n_kv_heads * TQK_PAGE * head_dim * 4.0 > 128e6;
-#define LAUNCH(DD) (nt ? attention_decode_kernel<DD, true> : attention_decode_kernel<DD, false>)<<<grid, AD_WAVES * TQK_WAVE, 0, s>>>( \
+    // Four waves a block; two where there are 512 blocks or more without partitions: then the memory has more
+    // pages asked of it at once than it serves well (128 sequences x 4 kv heads of 2100 positions: 106 against 114 us).
+    const bool two = n_parts == 1 && (long long)n_seqs * n_kv_heads * q_blocks >= 512;
+#define LAUNCH_W(DD, NT, W) attention_decode_kernel<DD, NT, W><<<grid, W * TQK_WAVE, 0, s>>>( \
         (const bf16_t*)q, (const bf16_t*)keys, (const bf16_t*)values, tok_pos, page_table, table_width, window, scale, \
         n_parts, n_heads, n_kv_heads, q_blocks, (float*)part_out, (float*)part_ml, (bf16_t*)out)
+#define LAUNCH(DD) { if (two) { if (nt) LAUNCH_W(DD, true, 2); else LAUNCH_W(DD, false, 2); } else { if (nt) LAUNCH_W(DD, true, 4); else LAUNCH_W(DD, false, 4); } }
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;
@@ -287,6 +291,7 @@ extern "C" int tqk_attention_decode(const void* q, const void* keys, const void*
         case 128: LAUNCH(128); break;
         case 256: LAUNCH(256); break;
     }
+#undef LAUNCH_W
 #undef LAUNCH
     if (tqk_check_launch("tqk_attention_decode")) return -1;
     if (n_parts == 1) return 0;
