@@ -628,7 +628,8 @@ tqe_batch_t* tqe_batch_new(int n_requests, int max_new, const int32_t* stop_ids,
         return nullptr;
     }
     b->max_new = max_new;
-    b->stop.assign(stop_ids, stop_ids + n_stop_ids);
+    for (int i = 0; i < n_stop_ids; ++i)
+        if (stop_ids[i] >= 0) b->stop.push_back(stop_ids[i]);       // no token has a negative id: such an entry stops nothing
     std::sort(b->stop.begin(), b->stop.end());
     b->emitted.assign(n_requests, 0);
     b->ended.assign(n_requests, 0);

@@ -388,6 +388,12 @@ void skinny_fused_kernel(const FusedArgs p) {
     }
 }
 
+// (17 to 32 rows through this kernel, two groups of 16 rows per wave against the same weights, were built and taken
+// out again: every wave then reads twice as much of x beside its weights, and the products took 57.6 us (o + down),
+// 56.5 us (gate + up) and 16.3 us (q/k/v) at the 7B sizes against 34.7, 48.7 and 12.0 with up to 16 rows; the kernels
+// that stage x in LDS once per block, mid_product.hip, are the better way for those steps in spite of their eight
+// launches a layer.)
+
 // Tiles per block for the back ends "store" and "residual", from the product's shape alone
 // (never from M: a row's sums then have one order in every batch).  Two tiles halve the
 // reads of x, but also the number of blocks, and a block keeps one compute unit busy:
