@@ -156,6 +156,7 @@ int tqe_page_size(void) { return TQE_PAGE; }
 int tqe_set_kernel_library(const char* path) {
     return guarded([&] { need(path, "tqe_set_kernel_library"); set_kernel_library(path); });
 }
+void tqe_set_kernel_builder(tqe_kernel_builder_t builder) { set_kernel_builder(builder); }
 const char* tqe_kernel_library(void) {
     return guarded_text([] { return kernel_library_path(); });
 }

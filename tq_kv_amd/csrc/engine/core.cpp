@@ -220,6 +220,13 @@ static std::mutex g_kernel_mutex;
 static std::string g_kernel_path;
 static void* g_kernel_handle = nullptr;
 
+static const char* (*g_kernel_builder)(void) = nullptr;
+
+void set_kernel_builder(const char* (*builder)(void)) {
+    std::lock_guard<std::mutex> lock(g_kernel_mutex);
+    g_kernel_builder = builder;
+}
+
 void set_kernel_library(const std::string& path) {
     std::lock_guard<std::mutex> lock(g_kernel_mutex);
     if (g_kernel_handle && path != g_kernel_path) { dlclose(g_kernel_handle); g_kernel_handle = nullptr; }
@@ -255,6 +262,11 @@ void* kernel_symbol(const char* name) {
     std::lock_guard<std::mutex> lock(g_kernel_mutex);
     if (!g_kernel_handle) {
         if (g_kernel_path.empty()) g_kernel_path = find_kernel_library();
+        if (g_kernel_path.empty() && g_kernel_builder) {
+            // the program that loaded this library knows how to build the kernels (the Python package compiles them)
+            const char* built = g_kernel_builder();
+            if (built && *built) g_kernel_path = built;
+        }
         if (g_kernel_path.empty())
             throw Error(TQE_ERR_DEVICE, "the HIP kernel library is not built: no libtqkernels_*.so beside the engine library "
                                         "(build it with tq_kv_amd/csrc/build.py, or name it in TQ_KERNEL_LIBRARY)");

@@ -165,6 +165,7 @@ private:
 // The kernel library is a shared object of its own (built by hipcc); it is opened at the first
 // use and its entry points are looked up by name.
 void set_kernel_library(const std::string& path);
+void set_kernel_builder(const char* (*builder)(void));       // asked for the library's path when none is found
 std::string kernel_library_path();
 void* kernel_symbol(const char* name);             // raises if the library or the symbol is missing
 [[noreturn]] void raise_kernel_error(const char* what);

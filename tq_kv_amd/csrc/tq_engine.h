@@ -154,8 +154,12 @@ int tqe_batch_ended(const tqe_batch_t* batch, int row);
 enum { TQE_F32 = 0, TQE_BF16 = 1, TQE_I32 = 2 };
 
 /* The HIP kernels live in a shared library of their own (libtqkernels_*.so beside this one, or what
- * TQ_KERNEL_LIBRARY names); it is opened at first use.  tqe_set_kernel_library names it outright. */
+ * TQ_KERNEL_LIBRARY names); it is opened at first use.  tqe_set_kernel_library names it outright.
+ * tqe_set_kernel_builder: a function of the caller's that is asked for the library's path when none is
+ * found (the Python package compiles the kernels there); it returns null or "" if it cannot. */
 int tqe_set_kernel_library(const char* path);
+typedef const char* (*tqe_kernel_builder_t)(void);
+void tqe_set_kernel_builder(tqe_kernel_builder_t builder);
 const char* tqe_kernel_library(void);
 /* Switches of the product and attention routines, for tests that compare one routine with another:
  * skinny, library, fused, prune_last, packed, mid, keep_rows, decode_mfma, prefill_mfma (all 1 to

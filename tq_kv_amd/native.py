@@ -133,6 +133,25 @@ class tqe_loop_callbacks(ctypes.Structure):
                 ("read", LOOP_READ)]
 
 
+_KERNEL_BUILDER_TYPE = ctypes.CFUNCTYPE(ctypes.c_void_p)
+_KERNEL_PATH = None
+
+
+def _build_kernels():
+    """What the engine library calls when it needs the kernel library and finds none: compile it (progress lines on
+    standard error) and say where it is."""
+    global _KERNEL_PATH
+    try:
+        _KERNEL_PATH = CString(_build.ensure_built())
+        return _KERNEL_PATH.address
+    except BaseException as e:          # nothing may escape into the library; the caller sees it once the library has returned
+        _pending_exception.append(e)
+        return None
+
+
+_KERNEL_BUILDER = _KERNEL_BUILDER_TYPE(_build_kernels)
+
+
 def library():
     global _LIB
     if _LIB is None:
@@ -204,6 +223,9 @@ def library():
         lib.tqe_trace_push.argtypes = [S]
         lib.tqe_trace_pop.restype = None
         lib.tqe_trace_pop.argtypes = []
+        lib.tqe_set_kernel_builder.restype = None
+        lib.tqe_set_kernel_builder.argtypes = [_KERNEL_BUILDER_TYPE]
+        lib.tqe_set_kernel_builder(_KERNEL_BUILDER)
         _LIB = lib
     return _LIB
 
