@@ -416,7 +416,9 @@ private:
         // partitions take the live pages in turn, four waves each: no more than a quarter of the pages there can be
         // (more partitions than one block per compute unit, so that no wave has a second page to bring in, measured
         // slower: 14.6 against 13.8 us for 8 sequences of 2100 positions at the 7B sizes; 64 sequences in 2 and 4
-        // partitions 60.6 and 65.9 against 56.4 us, 128 sequences 118 and 133 against 114)
+        // partitions 60.6 and 65.9 against 56.4 us, 128 sequences 118 and 133 against 114).  Nor fewer, larger blocks
+        // that need no merge: one block of eight waves per (sequence, kv head) took 37 us for the 8 sequences, since a
+        // compute unit alone pulls about 30 GB/s whatever its waves ask for.
         const int n_parts = std::max(1, std::min((width + 3) / 4, (target_blocks + groups - 1) / groups));
         Tensor part_out, part_ml;
         if (n_parts > 1) {
