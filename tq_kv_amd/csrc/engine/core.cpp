@@ -93,6 +93,16 @@ void stream_synchronize(hipStream_t stream) {
     hip_check(hipStreamSynchronize(stream), "waiting for the device");
 }
 
+int compute_units() {
+    if (g_null_device) return 0;
+    static int n = -1;
+    if (n < 0) {
+        int dev = 0, v = 0;
+        n = (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess) ? v : 0;
+    }
+    return n;
+}
+
 void device_synchronize() {
     if (g_null_device) return;
     hip_check(hipDeviceSynchronize(), "waiting for the device");

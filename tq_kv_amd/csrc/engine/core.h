@@ -85,6 +85,7 @@ void copy_on_device(void* dst, const void* src, size_t bytes, hipStream_t stream
 void zero_device(void* dst, size_t bytes, hipStream_t stream);                               // not inside a captured graph
 void stream_synchronize(hipStream_t stream);
 void device_synchronize();
+int compute_units();                  // of the current device (0 on the null device)
 void hip_check(int status, const char* what);
 
 class Buffer {

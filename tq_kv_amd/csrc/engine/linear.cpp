@@ -210,8 +210,25 @@ Tensor gated_silu_linear(StepContext& c, const Tensor& x, const Weight& w) {
     return act;
 }
 
+// The few-row kernel that adds to the stream keeps one block per tile of 16 features, a block stays on one compute
+// unit, and a compute unit alone pulls about a 256th of what the memory gives when all of them pull.  Where the tiles
+// fall badly on the units (the 320 tiles of a 5120-wide product on 256 units: a quarter of the units work twice as long
+// as the others) the kernel that cuts K into pieces over all units is faster, in spite of the norm kernel that then
+// has to add the pieces up.  Estimated from the shape alone, so a product takes one way whatever the batch.
+static bool pieces_pay(const Weight& w) {
+    if (!policy().mid || !w.packed || w.dtype != BF16 || w.k % 32 != 0) return false;
+    const int units = compute_units();
+    if (units <= 0 || K::mid_splits.raw((int)w.n, (int)w.k, 0) <= 1) return false;
+    const int blocks = K::fused_residual_parts.raw((int)w.n, (int)w.k);
+    const double rounds = (double)((blocks + units - 1) / units);
+    const double covered = (double)blocks / (rounds * units);
+    const double bytes = 2.0 * (double)w.n * (double)w.k, rate = 6.5e6;          // bytes a microsecond with every unit pulling
+    const double fused_us = bytes / (covered * rate), pieces_us = bytes / (0.85 * rate) + 6.0;
+    return pieces_us + 2.0 < fused_us;
+}
+
 void add_product(StepContext& c, Stream& stream, const Tensor& x, const Weight& w) {
-    if (x.shape[0] > skinny_max_rows()) {
+    if (x.shape[0] > skinny_max_rows() || pieces_pay(w)) {
         const bool leave = stream.next_norm && stream.next_norm->takes_partial_sums();
         Product p = k_mid_store(c, x, w, BF16, leave, nullptr);
         stream.pending = p.is_sums ? Pending::of(p.sums) : Pending::of(p.t);
