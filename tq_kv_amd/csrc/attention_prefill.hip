@@ -206,7 +206,12 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 16; i += 2) mx = fmaxf(mx, fmaxf(s[i], s[i + 1]));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, TQK_WAVE));         // the column's other 16 keys
+        {
+            // the column's other 16 keys, held by the lane 32 further on: the two halves of the wave change places in
+            // the registers themselves (v_permlane32_swap), no trip through LDS
+            const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+            mx = fmaxf(__uint_as_float(both[0]), __uint_as_float(both[1]));
+        }
         const float top = mx * w.c2;                           // c2 > 0
         if (__any(top > w.m + PF_LAZY)) {
             // raise the running maximum (on a query's first keys m is -inf and alpha 0)
