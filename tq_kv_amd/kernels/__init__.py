@@ -12,6 +12,7 @@ import torch
 from ..csrc import build as _build
 
 _LIB = None
+KERNEL_ABI = 12         # tqk_abi_version of the kernel library these wrappers are written against
 
 F32, BF16 = 0, 1
 STYLE_NONE, STYLE_HALVES, STYLE_PAIRS = 0, 1, 2
@@ -34,6 +35,9 @@ def library():
         lib.tqk_sample_scratch_bytes.restype = ctypes.c_size_t
         lib.tqk_gemm_scratch_bytes.restype = ctypes.c_size_t
         from .. import native
+        if int(lib.tqk_abi_version()) != KERNEL_ABI:
+            raise KernelError("the kernel library %s has interface version %d, these wrappers are written against %d: build it from these sources"
+                              % (path, lib.tqk_abi_version(), KERNEL_ABI))
         if int(lib.tqk_page_size()) != native.page_size():
             raise KernelError("the kernel library's cache pages hold %d positions, the engine library's %d: build both from the same sources"
                               % (lib.tqk_page_size(), native.page_size()))
