@@ -1,7 +1,8 @@
 """The engine library under AddressSanitizer and UndefinedBehaviorSanitizer: built with them into a
 temporary folder, loaded in a child process in place of the ordinary build, and driven by the tests
 that need no GPU: configuration, weights and their errors (models in host memory), the cache, the
-step's arrays, and the generation loop over stand-in engines and samplers."""
+step's arrays, the generation loop over stand-in engines and samplers, and whole steps and generation of models on
+the null device (every line of the engine that is not a kernel)."""
 import os
 import shutil
 import subprocess
@@ -36,7 +37,7 @@ def test_host_library_is_clean_under_address_and_ub_sanitizers(tmp_path):
     os.environ.setdefault("CXX", cxx)
     build.compile_host(lib, extra_flags=["-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer"])
     tests = [os.path.join(ROOT, "tests", n) for n in ("test_cache.py", "test_step_plan.py", "test_generate_loop.py", "test_config.py",
-                                                      "test_weights.py")]
+                                                      "test_weights.py", "test_dry_run.py")]
     env = dict(os.environ, LD_PRELOAD=" ".join(runtimes), ASAN_OPTIONS="detect_leaks=0:abort_on_error=1",
                TQ_KERNEL_LIBRARY=build.find_library(), TQ_ENGINE_LIBRARY=lib)
     child = subprocess.run([sys.executable, "-c", CHILD.format(root=ROOT, lib=lib, tests=tests)], capture_output=True, text=True, env=env,
