@@ -652,7 +652,7 @@ def test_products_of_17_to_128_rows_refuse_what_they_do_not_take():
 
 @pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (3, 1, 96), (40, 2, 64), (4, 1, 256)])
 @pytest.mark.parametrize("window", [0, 70])
-@pytest.mark.parametrize("target_blocks", [1, 24, 100000])
+@pytest.mark.parametrize("target_blocks", [1, 24, 100000, "a partition a page"])
 def test_attention_decode(nh, nkv, d, window, target_blocks):
     # three sequences of lengths 300, 64 and 1, pages scrambled, everything unread is NaN
     lens = [300, 64, 1]
@@ -678,8 +678,11 @@ def test_attention_decode(nh, nkv, d, window, target_blocks):
     pos = torch.tensor([n - 1 for n in lens])
     out = torch.empty(3, nh * d, dtype=torch.bfloat16, device=DEV)
     scale = 1 / math.sqrt(d)
-    K.attention_decode(q.to(DEV), keys, values, pos.to(torch.int32).to(DEV), ints(tables), window, scale, out,
-                       target_blocks=target_blocks)
+    if isinstance(target_blocks, str):         # as many partitions as the table is wide: blocks of one wave, one page each
+        K.attention_decode(q.to(DEV), keys, values, pos.to(torch.int32).to(DEV), ints(tables), window, scale, out, n_parts=len(tables[0]))
+    else:
+        K.attention_decode(q.to(DEV), keys, values, pos.to(torch.int32).to(DEV), ints(tables), window, scale, out,
+                           target_blocks=target_blocks)
     for i in range(3):
         want = attention_reference(q[i:i + 1].float(), ks[i], vs[i], pos[i:i + 1], window, scale)
         torch.testing.assert_close(out[i:i + 1].float().cpu(), want, atol=2e-2, rtol=2e-2)
@@ -993,6 +996,10 @@ def test_attention_decode_over_thousands_of_keys(nh, nkv, d, n_keys, window):
     for i in range(2):
         want = attention_reference(q[i:i + 1].float(), ks[i], vs[i], pos[i:i + 1], window, scale)
         torch.testing.assert_close(out[i:i + 1].float().cpu(), want, atol=2e-2, rtol=2e-2)
+    # a partition per page of the table (most of them empty behind a window, or beyond the short sequence's end)
+    thin = torch.full_like(out, float("nan"))
+    K.attention_decode(q.to(DEV), keys, values, pos.to(torch.int32).to(DEV), table, window, scale, thin, n_parts=table.shape[1])
+    torch.testing.assert_close(thin.float(), out.float(), atol=2e-2, rtol=2e-2)
     # the planted keys matter: without the window (or with it) the sharp query's answer is another
     other = attention_reference(q[:1].float(), ks[0], vs[0], pos[:1], 0 if window else 1000, scale)
     assert (other - out[:1].float().cpu()).abs().max() > 0.1

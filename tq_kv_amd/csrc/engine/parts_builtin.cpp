@@ -419,7 +419,10 @@ private:
         // partitions 60.6 and 65.9 against 56.4 us, 128 sequences 118 and 133 against 114).  Nor fewer, larger blocks
         // that need no merge: one block of eight waves per (sequence, kv head) took 37 us for the 8 sequences, since a
         // compute unit alone pulls about 30 GB/s whatever its waves ask for.
-        const int n_parts = std::max(1, std::min((width + 3) / 4, (target_blocks + groups - 1) / groups));
+        int n_parts = std::max(1, std::min((width + 3) / 4, (target_blocks + groups - 1) / groups));
+        // few sequences: a partition per page of the table, which the kernel gives a block of one wave each (faster up to
+        // four sequences of 2100 positions at the 7B sizes, slower from eight on)
+        if (width > 1 && (long long)groups * width <= 640) n_parts = width;
         Tensor part_out, part_ml;
         if (n_parts > 1) {
             part_out = c.alloc(F32, {n, n_heads_, n_parts, head_dim_});

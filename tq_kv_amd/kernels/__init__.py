@@ -350,9 +350,10 @@ def attention_decode_supported(head_dim):
     return bool(library().tqk_attention_decode_supported(int(head_dim)))
 
 
-def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, target_blocks=256):
+def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, target_blocks=256, n_parts=None):
     """Attention of one new token per sequence (q [B, heads, d] bfloat16, row b belongs to
-    sequence b at position tok_pos[b]) over the paged cache; out [B, heads*d]."""
+    sequence b at position tok_pos[b]) over the paged cache; out [B, heads*d].  n_parts: into how many partitions
+    a sequence's pages are dealt (as many as the table is wide: a block of one wave per page)."""
     n, n_heads, head_dim = q.shape
     n_pages, n_kv_heads = keys.shape[0], keys.shape[1]
     n_seqs, width = page_table.shape
@@ -361,7 +362,8 @@ def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, t
     q_blocks = (n_heads // n_kv_heads + 15) // 16
     groups = max(1, n * n_kv_heads * q_blocks)
     # partitions take the live pages in turn, four waves each: no more than a quarter of the pages there can be
-    n_parts = max(1, min((width + 3) // 4, (target_blocks + groups - 1) // groups))
+    if n_parts is None:
+        n_parts = max(1, min((width + 3) // 4, (target_blocks + groups - 1) // groups))
     part_out = part_ml = None
     if n_parts > 1:
         part_out = torch.empty((n, n_heads, n_parts, head_dim), dtype=torch.float32, device=q.device)
