@@ -353,6 +353,27 @@ static MidPlan mid_plan(int N, int K, bool gated) {
             if (waves == MID_MAX_WAVES || covered > best + 0.02) { best = covered; plan.waves = waves; plan.blocks = blocks; plan.splits = splits; }
         }
     }
+    if (gated && plan.splits > 1) {
+        // A gated product in pieces needs a kernel of its own to add them up and apply the gate (4 to 5 us); where the
+        // blocks of the whole K already cover half the units, that costs more than the pieces gain.  Estimated with a
+        // unit pulling 34 GB/s and the memory giving 6.5 TB/s (a width of 1536 and 8960 gate rows, 55 MB: 15.4 us whole
+        // against 13.9 + 4.6 in three pieces).
+        const double bytes = 2.0 * (double)N * (double)K;
+        auto time_us = [&](int blocks) { return 4.0 + bytes / (1e6 * (blocks * 0.034 < 6.5 ? blocks * 0.034 : 6.5)); };
+        double best_whole = 1e30;
+        int whole_waves = 0;
+        for (int waves = MID_MAX_WAVES; waves >= MID_MIN_WAVES; --waves) {
+            const int blocks = (items + waves - 1) / waves;
+            if (blocks > MID_UNITS) continue;
+            const double t = time_us(blocks);
+            if (t < best_whole - 0.1) { best_whole = t; whole_waves = waves; }
+        }
+        if (whole_waves && best_whole < time_us(plan.blocks * plan.splits) + 4.6) {
+            plan.waves = whole_waves;
+            plan.blocks = (items + whole_waves - 1) / whole_waves;
+            plan.splits = 1;
+        }
+    }
     const int per = (chunks + plan.splits - 1) / plan.splits;
     plan.splits = (chunks + per - 1) / per;             // no empty piece
     plan.k_per_split = per * MID_CHUNK;
