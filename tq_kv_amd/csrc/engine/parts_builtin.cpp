@@ -419,7 +419,9 @@ private:
         // partitions 60.6 and 65.9 against 56.4 us, 128 sequences 118 and 133 against 114).  Nor fewer, larger blocks
         // that need no merge: one block of eight waves per (sequence, kv head) took 37 us for the 8 sequences, since a
         // compute unit alone pulls about 30 GB/s whatever its waves ask for.
-        int n_parts = std::max(1, std::min((width + 3) / 4, (target_blocks + groups - 1) / groups));
+        // (no more blocks than compute units: with 288 blocks 32 units get two, and 12 sequences took 19.5 us against
+        // 16.1 with 240 blocks, 24 sequences 32.2 against 27.0, 48 sequences 48.9 + merge against 40.8 without)
+        int n_parts = std::max(1, std::min((width + 3) / 4, target_blocks / groups));
         // few sequences: a partition per page of the table, which the kernel gives a block of one wave each (faster up to
         // four sequences of 2100 positions at the 7B sizes, slower from eight on)
         if (width > 1 && (long long)groups * width <= 640) n_parts = width;

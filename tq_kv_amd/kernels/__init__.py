@@ -363,7 +363,7 @@ def attention_decode(q, keys, values, tok_pos, page_table, window, scale, out, t
     groups = max(1, n * n_kv_heads * q_blocks)
     # partitions take the live pages in turn, four waves each: no more than a quarter of the pages there can be
     if n_parts is None:
-        n_parts = max(1, min((width + 3) // 4, (target_blocks + groups - 1) // groups))
+        n_parts = max(1, min((width + 3) // 4, target_blocks // groups))
     part_out = part_ml = None
     if n_parts > 1:
         part_out = torch.empty((n, n_heads, n_parts, head_dim), dtype=torch.float32, device=q.device)
