@@ -13,6 +13,14 @@
 // memory into registers while this one is computed on and is written to the other buffer
 // afterwards, so a page costs one barrier.
 //
+// A prompt of a few thousand tokens gives a block or two per compute unit, the last tile's block walks
+// the most pages, and a wave alone on its SIMD takes nearly as long for a page as two waves take for
+// two.  Such steps run with two sets of waves per block (SPLIT = 2): both sets hold the same columns,
+// the first set takes the first 32 keys of every page and the second set the other 32, and the sets'
+// running maxima, sums and outputs are put together through LDS at the end.  The block then walks its
+// pages nearly twice as fast, one block fills a compute unit, and the blocks that come later go to the
+// units that finish first: the causal triangle evens itself out.
+//
 // Matrix-core mapping, v_mfma_f32_32x32x16_bf16 (D[32x32] += A[32x16] B[16x32]; a lane
 // holds of A row l%32 and the 8 k starting at 8*(l/32), of B the same k of column l%32, of
 // D column l%32 and the rows 8*(i/4) + 4*(l/32) + i%4, i = 0..15):
@@ -95,6 +103,7 @@ struct PrefillArgs {
     int n_heads, n_kv_heads, n_tiles;
     int tq_shift;            // log2 of the queries per tile
     int heads_per_block, head_chunks;
+    int col_waves;           // waves that hold the block's columns; with SPLIT = 2 the block has twice as many
     int snake_width;
 };
 
@@ -104,6 +113,7 @@ struct Wave {
     static constexpr int KS = D / 16;           // k steps of the score product
     static constexpr int DT = D / 32;           // tiles of 32 elements of the output
     int tid, n_threads, wave, n_waves, lane, c32, h;
+    int set;                                     // SPLIT = 2: which 32 keys of every page this wave takes
     int kvh;
     int my_pos, my_lo;                           // this lane's query and the first key it sees
     bool wave_live;
@@ -127,9 +137,13 @@ __device__ __forceinline__ void fetch_page(const Wave<D>& w, int page, u32x4_t (
     const size_t base = (size_t)(page < 0 ? 0 : page) * w.page_stride + (size_t)w.kvh * TQK_PAGE * D;
     const u32x4_t* kg = reinterpret_cast<const u32x4_t*>(w.keys + base);
     const u32x4_t* vg = reinterpret_cast<const u32x4_t*>(w.values + base);
+    const int wave_first = __builtin_amdgcn_readfirstlane(w.tid);
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) {
-        const int i = min(w.tid + c * w.n_threads, 8 * D - 1);      // (beyond the page: its last piece again, not stored)
+        // a wave whose pieces all lie beyond the page asks for nothing: a load of nothing takes the wave's turn at the
+        // compute unit's memory port as long as a load of a kilobyte (a block of eight waves: every other load)
+        if (wave_first + c * w.n_threads >= 8 * D) continue;
+        const int i = min(w.tid + c * w.n_threads, 8 * D - 1);      // (lanes beyond the page: its last piece again, not stored)
         kr[c] = kg[i];
         vr[c] = vg[i];
     }
@@ -150,7 +164,7 @@ __device__ __forceinline__ void stage_page(const Wave<D>& w, const u32x4_t (&kr)
 }
 
 // The work on one page, held in kc, vc.
-template <int D>
+template <int D, int SPLIT>
 __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_byte* __restrict__ kc, lds_byte* __restrict__ vc) {
     using L = Layout<D>;
     constexpr int KS = Wave<D>::KS, DT = Wave<D>::DT;
@@ -175,6 +189,7 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
     for (int t = 0; t < 2; ++t) {
         // a tile of 32 keys at a time
         const int k0 = key0 + 32 * t;
+        if (SPLIT == 2 && t != w.set) continue;
         if (k0 > w.wave_last || k0 + 31 < w.wave_lo) continue;
         // all operands of the tile's score product first, so that their reads are under way together
         bf16x8_t ka[KS];
@@ -243,15 +258,21 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
     }
 }
 
-template <int D>
+// What the second set of waves hands to the first at the end, a tile of 32 output elements at a time: 16 values a
+// lane, and with the first tile the running maximum and sum.  [value][column wave][lane]: the lanes' words lie side by side.
+#define PF_SPLIT_COL_WAVES 4
+#define PF_HANDOVER_BYTES (18 * PF_SPLIT_COL_WAVES * TQK_WAVE * 4)
+
+template <int D, int SPLIT>
 __global__ __launch_bounds__(PF_MAX_WAVES * TQK_WAVE)
 void attention_prefill_kernel(const PrefillArgs p) {
     using L = Layout<D>;
     constexpr int KS = Wave<D>::KS, DT = Wave<D>::DT;
-    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * L::K_BYTES];
-    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * L::V_BYTES];
-    lds_byte* const kb = (lds_byte*)k_lds;
-    lds_byte* const vb = (lds_byte*)v_lds;
+    constexpr int PAGES_BYTES = 2 * L::K_BYTES + 2 * L::V_BYTES;
+    constexpr int LDS_BYTES = SPLIT == 2 && PAGES_BYTES < PF_HANDOVER_BYTES ? PF_HANDOVER_BYTES : PAGES_BYTES;
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[LDS_BYTES];
+    lds_byte* const kb = (lds_byte*)lds;
+    lds_byte* const vb = kb + 2 * L::K_BYTES;
 
     Wave<D> w;
     w.tid = threadIdx.x;
@@ -261,6 +282,9 @@ void attention_prefill_kernel(const PrefillArgs p) {
     w.n_waves = blockDim.x / TQK_WAVE;
     w.c32 = w.lane & 31;
     w.h = w.lane >> 5;
+    // the wave's place among those that hold columns
+    const int cw = SPLIT == 2 ? w.wave % p.col_waves : w.wave;
+    w.set = SPLIT == 2 ? w.wave / p.col_waves : 0;
 
     // Blocks in the order of their work (the host lists the tiles longest first), kv heads and
     // head chunks fastest.  With snake_width > 0 every other run of snake_width blocks is taken
@@ -285,16 +309,16 @@ void attention_prefill_kernel(const PrefillArgs p) {
     const int tq = 1 << p.tq_shift;
 
     // this lane's column: a query of a head
-    const int col = w.wave * 32 + w.c32;
+    const int col = cw * 32 + w.c32;
     const int head_local = col >> p.tq_shift, qi = col & (tq - 1);
     const bool live = head_local < heads_here && qi < count;
     const int head = head0 + (live ? head_local : 0);
     w.my_pos = live ? pos0 + qi : -1;
     w.my_lo = p.window > 0 ? max(0, w.my_pos - p.window + 1) : 0;
     // the wave's range of queries (the same for all its heads)
-    const int wq_first = (w.wave * 32) & (tq - 1);
+    const int wq_first = (cw * 32) & (tq - 1);
     const int wq_last = min(tq >= 32 ? wq_first + 31 : tq - 1, count - 1);
-    w.wave_live = (w.wave * 32 >> p.tq_shift) < heads_here && wq_first < count;
+    w.wave_live = (cw * 32 >> p.tq_shift) < heads_here && wq_first < count;
     w.wave_first = pos0 + wq_first;
     w.wave_last = pos0 + wq_last;
     w.wave_lo = p.window > 0 ? max(0, w.wave_first - p.window + 1) : 0;            // first key any of its queries sees
@@ -340,13 +364,44 @@ void attention_prefill_kernel(const PrefillArgs p) {
             page_next = __shfl(my_pages, ahead, TQK_WAVE);
             fetch_page<D>(w, page_next, kr, vr);
         }
-        page_step<D>(w, pg, page_now, kb + cur * L::K_BYTES, vb + cur * L::V_BYTES);
+        page_step<D, SPLIT>(w, pg, page_now, kb + cur * L::K_BYTES, vb + cur * L::V_BYTES);
         if (pg < w.last_page) stage_page<D>(w, kr, vr, kb + (cur ^ 1) * L::K_BYTES, vb + (cur ^ 1) * L::V_BYTES);
         page_now = page_next;
     }
+    if constexpr (SPLIT == 2) {
+        // The second set's columns saw the other keys: out = (o0 2^(m0 - m) + o1 2^(m1 - m)) / (l0 2^(m0 - m) + l1 2^(m1 - m)),
+        // m the larger of the two maxima (a set that saw no key has m = -inf and counts for nothing).
+        __attribute__((address_space(3))) float* hand = (__attribute__((address_space(3))) float*)lds + cw * TQK_WAVE + w.lane;
+        constexpr int STEP = PF_SPLIT_COL_WAVES * TQK_WAVE;
+        float mine = 1.f, theirs = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            __syncthreads();                  // all are done with the pages (or with the tile handed over before)
+            if (w.set == 1) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) hand[i * STEP] = w.o[dt][i];
+                if (dt == 0) {
+                    hand[16 * STEP] = w.m;
+                    hand[17 * STEP] = w.l;
+                }
+            }
+            __syncthreads();
+            if (w.set == 0) {
+                if (dt == 0) {
+                    const float m1 = hand[16 * STEP], l1 = hand[17 * STEP];
+                    const float m = fmaxf(w.m, m1);
+                    mine = w.m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w.m - m);
+                    theirs = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - m);
+                    w.l = w.l * mine + l1 * theirs;
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) w.o[dt][i] = w.o[dt][i] * mine + hand[i * STEP] * theirs;
+            }
+        }
+    }
     float l = w.l;
     l += __shfl_xor(l, 32, TQK_WAVE);
-    if (live) {
+    if (live && w.set == 0) {
         // out^T[element 32 dt + 8 (i/4) + 4 h + i%4][this column]
         bf16_t* orow = p.out + ((size_t)(tok0 + qi) * p.n_heads + head) * D;
         const float inv = 1.f / l;
@@ -365,6 +420,10 @@ void attention_prefill_kernel(const PrefillArgs p) {
 
 }  // namespace
 
+// Up to this many blocks per compute unit a step runs with two sets of waves per block.  Measured with 7 heads a
+// group and head size 128, causal prompts alone: 1024 tokens (one block a unit) 30.8 -> 28.5 us, 2048 tokens (two)
+// 61.9 -> 60.9, 4096 tokens (four) 178 -> 191.
+#define PF_SPLIT_BLOCKS_PER_CU 2
 extern "C" int tqk_attention_prefill_supported(int head_dim) {
     return head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128;
 }
@@ -436,18 +495,22 @@ extern "C" int tqk_attention_prefill(const void* q, const void* keys, const void
     a.tq_shift = tile_queries == 16 ? 4 : (tile_queries == 32 ? 5 : (tile_queries == 64 ? 6 : 7));
     prefill_heads(n_heads / n_kv_heads, tile_queries, &a.heads_per_block, &a.head_chunks);
     // at least four waves: the page's journey through registers is dealt out to 256 threads or more
-    const int waves = max(4, (a.heads_per_block * tile_queries + 31) / 32);
+    a.col_waves = max(4, (a.heads_per_block * tile_queries + 31) / 32);
     const long long total = (long long)n_tiles * n_kv_heads * a.head_chunks;
     TQK_REQUIRE(total <= 0x7fffffffLL, "tqk_attention_prefill: %d tiles are more than the grid takes", n_tiles);
     const int n_cus = prefill_compute_units();
     TQK_REQUIRE(n_cus > 0, "tqk_attention_prefill: cannot read the number of compute units");
+    // two sets of waves per block where the columns leave room for them and the blocks are few (see the top)
+    const bool split = a.col_waves == PF_SPLIT_COL_WAVES && total <= (long long)PF_SPLIT_BLOCKS_PER_CU * n_cus;
+    const int waves = split ? 2 * a.col_waves : a.col_waves;
     // Blocks that are all resident at once (a compute unit holds 8 such waves) are not shared out
     // as they finish: then the runs of one block per compute unit alternate their direction.
     const int per_cu = waves <= 4 ? 2 : 1;
     a.snake_width = (total > n_cus && total <= (long long)per_cu * n_cus) ? n_cus : 0;
     hipStream_t s = (hipStream_t)stream;
     dim3 grid((unsigned)total);
-#define LAUNCH(DD) attention_prefill_kernel<DD><<<grid, waves * TQK_WAVE, 0, s>>>(a)
+#define LAUNCH(DD) do { if (split) attention_prefill_kernel<DD, 2><<<grid, waves * TQK_WAVE, 0, s>>>(a); \
+                        else attention_prefill_kernel<DD, 1><<<grid, waves * TQK_WAVE, 0, s>>>(a); } while (0)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;
