@@ -115,6 +115,9 @@ void mid_product_kernel(const MidArgs p) {
 
     // Loads past the end of K stay inside the row (and are valid memory); x is zeroed there as it
     // goes into LDS, so they add nothing.  Nothing is under a condition: the waits can be counted.
+    // (Measured: with the loads of a wave whose pieces all lie past the chunk left out under a
+    // condition, the compiler waits for all loads at every use, and a step of 64 rows at the 7B
+    // sizes takes 16.6 ms instead of 4.1.)
     auto load_x = [&](int c, u32x4_t (&xr)[XS]) {
         if constexpr (WIDE) {
             if (!stages) return;
