@@ -702,7 +702,9 @@ def test_attention_decode_refuses_other_head_sizes():
                            torch.empty(1, 48, dtype=torch.bfloat16, device=DEV))
 
 
-@pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (3, 1, 96), (40, 2, 64), (12, 2, 128)])
+# (every head size both ways: blocks of four waves of columns, which run as two sets of waves that share each page's
+# keys between them, and blocks of more waves of columns, which do not; head size 32 the second way with 10 heads on 2)
+@pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (10, 2, 32), (3, 1, 96), (40, 2, 64), (12, 2, 128)])
 @pytest.mark.parametrize("window", [0, 70, 12])
 @pytest.mark.parametrize("tile", [16, 32, 64, 128])
 def test_attention_prefill(nh, nkv, d, window, tile):
