@@ -42,6 +42,7 @@
 // until then p may be up to 2^8, which float32 sums and bfloat16 products carry as well.
 #include "common.h"
 #include "tq_kernels.h"
+#include <type_traits>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
@@ -123,6 +124,10 @@ struct Wave {
     const bf16_t* keys;
     const bf16_t* values;
     size_t page_stride;
+    // Where this lane's operands lie in a page's buffer (byte offsets): the keys' pieces of step ks of a tile's first
+    // row, and the values' pieces of step st of tile t, of the first 32 elements.  Worked out once and held as they
+    // are: a read's address is then one of these registers plus a constant that is part of the instruction.
+    int k_off[KS], v_off[2][2];
     bf16x8_t bq[KS];                             // the queries: B operand of the score product
     float m, l;
     floatx16_t o[DT];
@@ -184,7 +189,6 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
         __syncthreads();
     }
     if (!w.wave_live || page_now < 0) return;
-    const int krow = tile_key(c32);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         // a tile of 32 keys at a time
@@ -194,7 +198,7 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
         // all operands of the tile's score product first, so that their reads are under way together
         bf16x8_t ka[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) ka[ks] = *(lds_bf16x8*)(kc + L::k_at(32 * t + krow, 2 * ks + h));
+        for (int ks = 0; ks < KS; ++ks) ka[ks] = *(lds_bf16x8*)(kc + 32 * t * L::KROW + w.k_off[ks]);
         __builtin_amdgcn_sched_barrier(0);
         floatx16_t s;
 #pragma unroll
@@ -206,7 +210,7 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
 #pragma unroll
         for (int st = 0; st < 2; ++st)
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) va[st][dt] = *(lds_bf16x8*)(vc + L::v_at(32 * dt + c32, 4 * t + 2 * st + h));
+            for (int dt = 0; dt < DT; ++dt) va[st][dt] = *(lds_bf16x8*)(vc + 32 * dt * 128 + w.v_off[t][st]);
         __builtin_amdgcn_sched_barrier(0);
         // the mask is needed only on tiles that cross a query's causal or window edge
         const bool need_mask = k0 + 31 > w.wave_first || k0 < w.wave_lo_last;
@@ -284,7 +288,7 @@ void attention_prefill_kernel(const PrefillArgs p) {
     w.h = w.lane >> 5;
     // the wave's place among those that hold columns
     const int cw = SPLIT == 2 ? w.wave % p.col_waves : w.wave;
-    w.set = SPLIT == 2 ? w.wave / p.col_waves : 0;
+    w.set = SPLIT == 2 ? __builtin_amdgcn_readfirstlane(w.wave / p.col_waves) : 0;
 
     // Blocks in the order of their work (the host lists the tiles longest first), kv heads and
     // head chunks fastest.  With snake_width > 0 every other run of snake_width blocks is taken
@@ -318,9 +322,11 @@ void attention_prefill_kernel(const PrefillArgs p) {
     // the wave's range of queries (the same for all its heads)
     const int wq_first = (cw * 32) & (tq - 1);
     const int wq_last = min(tq >= 32 ? wq_first + 31 : tq - 1, count - 1);
-    w.wave_live = (cw * 32 >> p.tq_shift) < heads_here && wq_first < count;
-    w.wave_first = pos0 + wq_first;
-    w.wave_last = pos0 + wq_last;
+    // (the same in all lanes of the wave, and said so: what is decided from them is then decided once per wave, by
+    // scalar compares and branches)
+    w.wave_live = __builtin_amdgcn_readfirstlane((cw * 32 >> p.tq_shift) < heads_here && wq_first < count);
+    w.wave_first = __builtin_amdgcn_readfirstlane(pos0 + wq_first);
+    w.wave_last = __builtin_amdgcn_readfirstlane(pos0 + wq_last);
     w.wave_lo = p.window > 0 ? max(0, w.wave_first - p.window + 1) : 0;            // first key any of its queries sees
     w.wave_lo_last = p.window > 0 ? max(0, w.wave_last - p.window + 1) : 0;        // first key all of them see
     w.c2 = p.scale * 1.44269504088896340736f;
@@ -337,6 +343,23 @@ void attention_prefill_kernel(const PrefillArgs p) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) w.bq[ks] = live ? *reinterpret_cast<const bf16x8_t*>(qrow + ks * 16) : zero8;
     }
+    {
+        // (the swizzles of k_at and v_at look only at bits of the row's number that the tile's and the element tile's
+        // first rows, multiples of 32, leave alone)
+        const int krow = tile_key(w.c32);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            w.k_off[ks] = L::k_at(krow, 2 * ks + w.h);
+            asm volatile("" : "+v"(w.k_off[ks]));
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                w.v_off[t][st] = L::v_at(w.c32, 4 * t + 2 * st + w.h);
+                asm volatile("" : "+v"(w.v_off[t][st]));
+            }
+    }
     w.m = -INFINITY;
     w.l = 0.f;
 #pragma unroll
@@ -351,22 +374,31 @@ void attention_prefill_kernel(const PrefillArgs p) {
     const int32_t* pages = p.page_table + (size_t)seq * p.table_width;
     int my_pages = pages[min(first_page + w.lane, w.last_page)];
     u32x4_t kr[D / 32], vr[D / 32];
-    int page_now = __shfl(my_pages, 0, TQK_WAVE);
+    int page_now = __builtin_amdgcn_readfirstlane(__shfl(my_pages, 0, TQK_WAVE));
     fetch_page<D>(w, page_now, kr, vr);
-    stage_page<D>(w, kr, vr, kb + (first_page & 1) * L::K_BYTES, vb + (first_page & 1) * L::V_BYTES);
-    for (int pg = first_page; pg <= w.last_page; ++pg) {
-        const int cur = pg & 1;
+    stage_page<D>(w, kr, vr, kb, vb);
+    // The loop is written out for its two buffers (the first page lies in the first one): which buffer a
+    // read or write goes to is then part of the instruction, not an addition in front of each of them.
+    int pg = first_page;
+    auto one_page = [&](auto which) {
+        constexpr int cur = decltype(which)::value;
         __syncthreads();                      // the page is whole; all are done with the other buffer
         int page_next = -1;
         if (pg < w.last_page) {
             const int ahead = (pg + 1 - first_page) & (TQK_WAVE - 1);
             if (ahead == 0) my_pages = pages[min(pg + 1 + w.lane, w.last_page)];
-            page_next = __shfl(my_pages, ahead, TQK_WAVE);
+            page_next = __builtin_amdgcn_readfirstlane(__shfl(my_pages, ahead, TQK_WAVE));
             fetch_page<D>(w, page_next, kr, vr);
         }
         page_step<D, SPLIT>(w, pg, page_now, kb + cur * L::K_BYTES, vb + cur * L::V_BYTES);
         if (pg < w.last_page) stage_page<D>(w, kr, vr, kb + (cur ^ 1) * L::K_BYTES, vb + (cur ^ 1) * L::V_BYTES);
         page_now = page_next;
+        ++pg;
+    };
+    while (pg <= w.last_page) {
+        one_page(std::integral_constant<int, 0>());
+        if (pg > w.last_page) break;
+        one_page(std::integral_constant<int, 1>());
     }
     if constexpr (SPLIT == 2) {
         // The second set's columns saw the other keys: out = (o0 2^(m0 - m) + o1 2^(m1 - m)) / (l0 2^(m0 - m) + l1 2^(m1 - m)),
