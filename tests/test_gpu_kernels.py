@@ -28,7 +28,7 @@ def ints(values):
 
 
 def test_library_is_built_and_loaded():
-    assert K.library().tqk_abi_version() == K.KERNEL_ABI == 12
+    assert K.library().tqk_abi_version() == K.KERNEL_ABI == 13
     assert K.library_path().endswith(".so")
     with pytest.raises(K.KernelError, match="GPU only"):
         K.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
@@ -65,6 +65,14 @@ def test_pack_weight_on_the_gpu_equals_the_plain_reordering():
         got = K.pack_weight(w, parts)
         want = K.pack_weight(w.cpu(), parts)              # torch's reshape and permute on the host
         assert tuple(got.data.shape) == tuple(want.data.shape) and torch.equal(got.data.cpu(), want.data)
+
+
+def test_unpack_weight_gives_the_rows_back():
+    # parts whose rows are no multiple of 16 (the packed copy pads them), k of less and of more than a block's 512
+    # columns and no multiple of them, and the width of a vocabulary
+    for n, k, parts in ((40, 96, 1), (38, 96, 2), (224, 1056, 2), (3584, 512, 1), (19, 64, 1), (50000, 160, 1)):
+        w = rand(n, k, seed=n + 1, dtype=torch.bfloat16)
+        assert torch.equal(K.unpack_weight(K.pack_weight(w, parts)), w), (n, k, parts)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -44,7 +44,7 @@ def _add_model(p):
                    help="Tensors in the folder that the model does not use are a warning, not an error")
     p.add_argument("--packed-weights-only", action="store_true",
                    help="Keep only the copy of the bfloat16 weights that the decoding kernels read (half the weight memory; "
-                        "prompts of more than 128 tokens then run several times slower)")
+                        "a prompt's products get the rows back from it for their own length: a seventh more time for 2048 tokens)")
     p.add_argument("--max-cache-tokens", type=int, default=0,
                    help="Positions the cache holds for all live requests together (0: what the prompts need)")
 

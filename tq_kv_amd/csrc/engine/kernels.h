@@ -57,6 +57,7 @@ TQ_KERNEL(sample, cf32, int, int, float, int, float, cf32, int32_t*, void*, void
 TQ_KERNEL(gather_rows, cptr, ci32, int, long long, void*, void*);
 TQ_KERNEL(add_bias, void*, int, cptr, int, int, int, void*);
 TQ_KERNEL(pack_weight, cptr, void*, int, int, int, void*);
+TQ_KERNEL(unpack_weight, cptr, void*, int, int, int, void*);
 TQ_KERNEL(convert, cptr, int, void*, int, long long, void*);
 
 #undef TQ_KERNEL

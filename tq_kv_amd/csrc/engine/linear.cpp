@@ -167,8 +167,17 @@ Product linear(StepContext& c, const Tensor& x, const Weight& w, const Tensor* b
             return p;
         }
         if (mid_ok(x, w)) return k_mid_store(c, x, w, out_dtype, leave_sums, out);
+        if (!w.rows && m > mid_max_rows() && policy().library && !null_device()) {
+            // the rows were given up and this is a prompt: the rows come back for the length of this product (the weight
+            // read and written once more, against reading it once per 128 rows of x)
+            Tensor rows = c.alloc(BF16, {w.n, w.k});
+            K::unpack_weight(w.packed->t.data, rows.data, (int)w.n, (int)w.k, w.parts, c.stream);
+            p.t = out ? *out : c.alloc(out_dtype, {m, w.n});
+            library_gemm(x, rows, p.t, c.stream);
+            return p;
+        }
         if (!w.rows) {
-            // the rows were given up: every number of rows through the own kernels, in pieces that each stream the weight once
+            // every number of rows through the own kernels, in pieces that each stream the weight once
             p.t = out ? *out : c.alloc(out_dtype, {m, w.n});
             const int64_t step = mid_max_rows();
             for (int64_t r = 0; r < m; r += step) {
@@ -196,7 +205,7 @@ Tensor gated_silu_linear(StepContext& c, const Tensor& x, const Weight& w) {
     Tensor act = c.alloc(x.dtype, {m, inter});
     if (skinny_ok(x, w)) { k_fused_gated(c, x, nullptr, w, act); return act; }
     if (mid_ok(x, w)) { k_mid_gated(c, x, w, act); return act; }
-    if (!w.rows) {
+    if (!w.rows && !(m > mid_max_rows() && policy().library && !null_device())) {
         const int64_t step = mid_max_rows();
         for (int64_t r = 0; r < m; r += step) {
             Tensor xs = x.slice(r, std::min(m, r + step)), os = act.slice(r, std::min(m, r + step));

@@ -23,7 +23,8 @@ namespace tq {
 // kernel); nothing else reads these.  "packed": parts keep the second, packed copy of their
 // weights for the few-row kernels (twice the weight memory, about an eighth less time per
 // decoding step).  "keep_rows": off gives the rows up once a weight is packed (set it before
-// loading): products of more rows than the own kernels take then go through them in pieces.
+// loading): a product of more rows than the own kernels take then gets the rows back from the
+// packed copy for its own length (or, with the library off, goes through the own kernels in pieces).
 struct Policy {
     int skinny = 1, library = 1, fused = 1, prune_last = 1, packed = 1, mid = 1, keep_rows = 1;
     int decode_mfma = 1, prefill_mfma = 1;

@@ -22,4 +22,4 @@ int tqk_check_launch(const char* what) {
 }
 
 extern "C" const char* tqk_last_error(void) { return g_last_error; }
-extern "C" int tqk_abi_version(void) { return 12; }
+extern "C" int tqk_abi_version(void) { return 13; }

@@ -20,7 +20,7 @@ extern "C" {
 #endif
 
 #define TQE_PAGE 64             /* positions per cache page (the kernel library is asked for its own and must agree) */
-#define TQE_KERNEL_ABI 12       /* the version of the kernel library's interface (tqk_abi_version) this engine is written against */
+#define TQE_KERNEL_ABI 13       /* the version of the kernel library's interface (tqk_abi_version) this engine is written against */
 #define TQE_MAX_GROUPS 16       /* groups of cached runs a cache may have */
 
 enum {

@@ -39,6 +39,8 @@ int tqk_convert(const void* src, int src_dtype, void* dst, int dst_dtype, long l
 /* A bfloat16 weight [n, k] (k a multiple of 32; `parts` stacked weights of n / parts rows) in the order the lanes of the
  * few-row kernels take it: out [parts * ceil(n / parts / 16)][k / 32][64][8], see tqk_fused_store. */
 int tqk_pack_weight(const void* w, void* out, int n, int k, int parts, void* stream);
+/* and back: rows [n, k] from the packed copy (for products of many rows, which the library takes from rows) */
+int tqk_unpack_weight(const void* packed, void* rows, int n, int k, int parts, void* stream);
 
 /* out[t, :] = scale * float(table[ids[t], :]); ids outside [0, vocab) give zeros.  copy_bf16
  * (optional): the same values as bfloat16 [tokens, hidden], times copy_weight [hidden]

@@ -48,6 +48,28 @@ void pack_weight_kernel(const uint16_t* __restrict__ w, uint16_t* __restrict__ o
     }
 }
 
+// The other way round, for products of many rows that go to the library: 16 rows x 512 columns a block (16 k steps
+// of a tile: 16 KB that lie together in the packed copy), turned through LDS so that both the reads and the writes
+// are runs of a kilobyte.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+#define UNPACK_KSTEPS 16
+__global__ __launch_bounds__(256)
+void unpack_weight_kernel(const u32x4_t* __restrict__ packed, u32x4_t* __restrict__ rows, int per, int k, int tiles) {
+    __shared__ u32x4_t turn[16][UNPACK_KSTEPS * 4 + 1];           // [row][piece of 8 columns]; the odd pitch keeps the rows' banks apart
+    const int ksteps = k / 32, ks0 = blockIdx.x * UNPACK_KSTEPS, n_ks = min(UNPACK_KSTEPS, ksteps - ks0);
+    const long long pt = blockIdx.y;                               // part * tiles + tile
+    for (int i = threadIdx.x; i < n_ks * 64; i += blockDim.x) {
+        const int lane = i % 64;
+        turn[lane % 16][(i / 64) * 4 + lane / 16] = packed[(pt * ksteps + ks0) * 64 + i];
+    }
+    __syncthreads();
+    const int tile = (int)(pt % tiles), part = (int)(pt / tiles), pieces = n_ks * 4;
+    for (int i = threadIdx.x; i < 16 * pieces; i += blockDim.x) {
+        const int r = i / pieces, c = i % pieces, row = tile * 16 + r;
+        if (row < per) rows[(((long long)part * per + row) * k + ks0 * 32) / 8 + c] = turn[r][c];
+    }
+}
+
 int blocks_for(long long n) {
     const long long want = (n + 255) / 256;
     return (int)(want < 1 ? 1 : want > 65535 ? 65535 : want);
@@ -103,6 +125,18 @@ extern "C" int tqk_convert(const void* src, int src_dtype, void* dst, int dst_dt
     else if (src_dtype == TQK_BF16 && dst_dtype == TQK_BF16) convert_kernel<bf16_t, bf16_t><<<b, 256, 0, s>>>((const bf16_t*)src, (bf16_t*)dst, n);
     else return tqk_fail("tqk_convert: unknown dtype codes %d, %d", src_dtype, dst_dtype);
     return tqk_check_launch("tqk_convert");
+}
+
+extern "C" int tqk_unpack_weight(const void* packed, void* rows, int n, int k, int parts, void* stream) {
+    TQK_REQUIRE(packed && rows, "tqk_unpack_weight: null pointer");
+    TQK_REQUIRE(n > 0 && k > 0 && parts > 0 && k % 32 == 0 && n % parts == 0,
+                "tqk_unpack_weight: needs bfloat16 [n, k] with k a multiple of 32 and n of %d parts, got [%d, %d]", parts, n, k);
+    TQK_REQUIRE((((uintptr_t)packed | (uintptr_t)rows) & 15) == 0, "tqk_unpack_weight: both copies must be 16-byte aligned");
+    const int per = n / parts, tiles = (per + 15) / 16;
+    TQK_REQUIRE((long long)parts * tiles <= 65535, "tqk_unpack_weight: %d rows are more than the grid takes", n);
+    dim3 grid((k / 32 + UNPACK_KSTEPS - 1) / UNPACK_KSTEPS, parts * tiles);
+    unpack_weight_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const u32x4_t*)packed, (u32x4_t*)rows, per, k, tiles);
+    return tqk_check_launch("tqk_unpack_weight");
 }
 
 extern "C" int tqk_pack_weight(const void* w, void* out, int n, int k, int parts, void* stream) {

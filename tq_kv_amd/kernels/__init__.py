@@ -12,7 +12,7 @@ import torch
 from ..csrc import build as _build
 
 _LIB = None
-KERNEL_ABI = 12         # tqk_abi_version of the kernel library these wrappers are written against
+KERNEL_ABI = 13         # tqk_abi_version of the kernel library these wrappers are written against
 
 F32, BF16 = 0, 1
 STYLE_NONE, STYLE_HALVES, STYLE_PAIRS = 0, 1, 2
@@ -452,6 +452,14 @@ def pack_weight(weight, parts=1):
     # [part, tile, row, k step, k group, 8] -> [part, tile, k step, k group, row, 8]
     data = w.reshape(parts, tiles, 16, k // 32, 4, 8).permute(0, 1, 3, 4, 2, 5).contiguous()
     return PackedWeight(data.reshape(parts * tiles, k // 32, 64, 8), n, k, parts)
+
+
+def unpack_weight(packed):
+    """The rows [n, k] of a PackedWeight on the GPU (what pack_weight was given)."""
+    n, k = packed.shape
+    rows = torch.empty((n, k), dtype=torch.bfloat16, device=packed.data.device)
+    _check(library().tqk_unpack_weight(_dev(packed.data, "data"), _dev(rows, "rows"), n, k, packed.parts, _stream()), "unpack_weight")
+    return rows
 
 
 def _weight(weight, name, n, k, parts=1):

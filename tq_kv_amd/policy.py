@@ -7,7 +7,8 @@ another; nothing else reads these.  They live in the engine library (tqe_policy_
   packed                 parts keep a second copy of their bfloat16 weights in the few-row kernels'
                          order (twice the weight memory, about an eighth less time per decoding step)
   keep_rows              off: the rows are given up once a weight is packed (set it before loading):
-                         half the weight memory again; prompts then run through the own kernels in pieces
+                         half the weight memory again; a product of more than 128 rows (a prompt) gets the
+                         rows back from the packed copy for its own length
   decode_mfma, prefill_mfma   the two matrix-core attention kernels (off: the plain kernel)
 """
 from . import native
