@@ -13,13 +13,15 @@
 // memory into registers while this one is computed on and is written to the other buffer
 // afterwards, so a page costs one barrier.
 //
-// A prompt of a few thousand tokens gives a block or two per compute unit, the last tile's block walks
-// the most pages, and a wave alone on its SIMD takes nearly as long for a page as two waves take for
-// two.  Such steps run with two sets of waves per block (SPLIT = 2): both sets hold the same columns,
-// the first set takes the first 32 keys of every page and the second set the other 32, and the sets'
-// running maxima, sums and outputs are put together through LDS at the end.  The block then walks its
-// pages nearly twice as fast, one block fills a compute unit, and the blocks that come later go to the
-// units that finish first: the causal triangle evens itself out.
+// A prompt of a thousand or two tokens gives a block or two per compute unit, the last tile's block
+// walks the most pages, and once the short blocks are gone its waves are alone on their SIMDs, where
+// a page takes a wave nearly as long as it takes each of two waves that share a SIMD.  Such steps run
+// with two sets of waves per block (SPLIT = 2): both sets hold the same columns, the first set takes
+// the first 32 keys of every page and the second set the other 32, and the sets' running maxima, sums
+// and outputs are put together through LDS at the end.  A page then costs a wave one tile instead of
+// two (1024 tokens: 30.8 -> 28.5 us, 2048 tokens: 61.9 -> 60.9 with 7 heads a group of size 128);
+// with more blocks than two per unit the later meeting of eight waves at the barrier costs more than
+// that gains, and the step runs with one set.
 //
 // Matrix-core mapping, v_mfma_f32_32x32x16_bf16 (D[32x32] += A[32x16] B[16x32]; a lane
 // holds of A row l%32 and the 8 k starting at 8*(l/32), of B the same k of column l%32, of
