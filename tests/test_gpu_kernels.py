@@ -1021,6 +1021,7 @@ def test_attention_decode_over_thousands_of_keys(nh, nkv, d, n_keys, window):
 @pytest.mark.parametrize("nh,nkv,d,spans,tile", [
     (28, 4, 128, [(0, 2048)], 16),                    # the benchmarked prompt: two heads a wave, all blocks resident
     (28, 4, 128, [(0, 2048)], 64),
+    (28, 4, 128, [(0, 4096)], 16),                    # more blocks than two a compute unit: one set of four waves a block
     (28, 4, 128, [(0, 3200)], 32),                    # a head a wave, blocks of seven waves shared out as they finish
     (28, 4, 128, [(0, 3200)], 128),
     (28, 4, 128, [(1100, 2100), (0, 70)], 32),        # a piece of a prompt behind 1100 cached positions
