@@ -257,10 +257,15 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
         w.l += psum;
         // out^T += V^T P^T: step st takes the lane's registers 8 st .. 8 st + 7 and the 16 bytes of
         // values that hold the same keys
+        // (at a higher priority than the vector work of the SIMD's other wave: its operands are all there, and the
+        // sooner the chain is under way the sooner the matrix cores work beside that wave's softmax; 8192 tokens in
+        // tiles of 64: 528 -> 514 us)
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int st = 0; st < 2; ++st)
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) w.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[st][dt], pb[st], w.o[dt], 0, 0, 0);
+        __builtin_amdgcn_s_setprio(0);
     }
 }
 
