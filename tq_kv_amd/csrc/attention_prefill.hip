@@ -224,6 +224,13 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
                 if (j < w.my_lo || j > w.my_pos) s[i] = -INFINITY;
             }
         }
+        // The scores against the running maximum as it stands, in powers of two: t = s c - m (0 for m while the column
+        // has no key yet).  Nearly always they are the exponents already; the largest of them says whether the maximum
+        // has to be raised first.  (The maximum is taken of these, not of the raw scores: a product of the matrix
+        // cores would have to be made canonical value by value before a maximum may look at it.)
+        const float m_was = w.m == -INFINITY ? 0.f : w.m;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = fmaf(s[i], w.c2, -m_was);
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 16; i += 2) mx = fmaxf(mx, fmaxf(s[i], s[i + 1]));
@@ -233,24 +240,26 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
             const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
             mx = fmaxf(__uint_as_float(both[0]), __uint_as_float(both[1]));
         }
-        const float top = mx * w.c2;                           // c2 > 0
-        if (__any(top > w.m + PF_LAZY)) {
-            // raise the running maximum (on a query's first keys m is -inf and alpha 0)
-            const float m_new = top > w.m + PF_LAZY ? top : w.m;
-            const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(w.m - m_new);
-            w.m = m_new;
+        // a score that passes the maximum by more than 2^PF_LAZY raises it, and so does a column's first key
+        const bool raise = w.m == -INFINITY ? mx > -INFINITY : mx > PF_LAZY;
+        if (__any(raise)) {
+            const float up = raise ? mx : 0.f;                 // by how much
+            const float alpha = w.m == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(-up);       // (nothing summed yet: out and l are 0)
+            if (raise) w.m = m_was + up;
             w.l *= alpha;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) w.o[dt][i] *= alpha;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[i] -= up;
         }
-        const float m_use = w.m == -INFINITY ? 0.f : w.m;      // a column without a key so far: every p is 2^(-inf) = 0
+        // (a column without a key so far: every t is -inf and every p is 2^(-inf) = 0)
         bf16x8_t pb[2];
         float psum = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float pr = __builtin_amdgcn_exp2f(fmaf(s[i], w.c2, -m_use));
+            const float pr = __builtin_amdgcn_exp2f(s[i]);
             psum += pr;
             pb[i >> 3][i & 7] = (__bf16)pr;
         }
