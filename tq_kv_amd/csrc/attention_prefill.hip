@@ -131,7 +131,9 @@ struct Wave {
     // are: a read's address is then one of these registers plus a constant that is part of the instruction.
     int k_off[KS], v_off[2][2];
     bf16x8_t bq[KS];                             // the queries: B operand of the score product
-    float m, l;
+    // The running maximum m that the exponents are set against (0 while the column has no key yet), the running sum l,
+    // and how far a score must pass m to raise it: PF_LAZY, and -inf while there is no key yet (any score then does).
+    float m, l, pass;
     floatx16_t o[DT];
 };
 
@@ -224,13 +226,12 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
                 if (j < w.my_lo || j > w.my_pos) s[i] = -INFINITY;
             }
         }
-        // The scores against the running maximum as it stands, in powers of two: t = s c - m (0 for m while the column
-        // has no key yet).  Nearly always they are the exponents already; the largest of them says whether the maximum
-        // has to be raised first.  (The maximum is taken of these, not of the raw scores: a product of the matrix
-        // cores would have to be made canonical value by value before a maximum may look at it.)
-        const float m_was = w.m == -INFINITY ? 0.f : w.m;
+        // The scores against the running maximum as it stands, in powers of two: t = s c - m.  Nearly always they are
+        // the exponents already; the largest of them says whether the maximum has to be raised first.  (The maximum
+        // is taken of these, not of the raw scores: a product of the matrix cores would have to be made canonical
+        // value by value before a maximum may look at it.)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = fmaf(s[i], w.c2, -m_was);
+        for (int i = 0; i < 16; ++i) s[i] = fmaf(s[i], w.c2, -w.m);
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 16; i += 2) mx = fmaxf(mx, fmaxf(s[i], s[i + 1]));
@@ -240,12 +241,14 @@ __device__ __forceinline__ void page_step(Wave<D>& w, int pg, int page_now, lds_
             const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
             mx = fmaxf(__uint_as_float(both[0]), __uint_as_float(both[1]));
         }
-        // a score that passes the maximum by more than 2^PF_LAZY raises it, and so does a column's first key
-        const bool raise = w.m == -INFINITY ? mx > -INFINITY : mx > PF_LAZY;
+        const bool raise = mx > w.pass;
         if (__any(raise)) {
             const float up = raise ? mx : 0.f;                 // by how much
-            const float alpha = w.m == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(-up);       // (nothing summed yet: out and l are 0)
-            if (raise) w.m = m_was + up;
+            // (a column's first key may lie below 0, the maximum's stand-in until then: out and l are 0 there, and alpha
+            // must only stay finite)
+            const float alpha = __builtin_amdgcn_exp2f(-fmaxf(up, 0.f));
+            w.m += up;
+            if (raise) w.pass = PF_LAZY;
             w.l *= alpha;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
@@ -376,7 +379,8 @@ void attention_prefill_kernel(const PrefillArgs p) {
                 asm volatile("" : "+v"(w.v_off[t][st]));
             }
     }
-    w.m = -INFINITY;
+    w.m = 0.f;
+    w.pass = -INFINITY;
     w.l = 0.f;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -429,7 +433,7 @@ void attention_prefill_kernel(const PrefillArgs p) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) hand[i * STEP] = w.o[dt][i];
                 if (dt == 0) {
-                    hand[16 * STEP] = w.m;
+                    hand[16 * STEP] = w.pass == -INFINITY ? -INFINITY : w.m;
                     hand[17 * STEP] = w.l;
                 }
             }
@@ -437,8 +441,9 @@ void attention_prefill_kernel(const PrefillArgs p) {
             if (w.set == 0) {
                 if (dt == 0) {
                     const float m1 = hand[16 * STEP], l1 = hand[17 * STEP];
-                    const float m = fmaxf(w.m, m1);
-                    mine = w.m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w.m - m);
+                    const float m0 = w.pass == -INFINITY ? -INFINITY : w.m;
+                    const float m = fmaxf(m0, m1);
+                    mine = m0 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m0 - m);
                     theirs = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - m);
                     w.l = w.l * mine + l1 * theirs;
                 }
