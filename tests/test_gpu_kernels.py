@@ -1018,6 +1018,34 @@ def test_attention_decode_over_thousands_of_keys(nh, nkv, d, n_keys, window):
     torch.testing.assert_close(out.float(), out2.float(), atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("tile", [16, 64])
+def test_attention_prefill_with_scores_far_below_zero(tile):
+    # Every score of the first keys lies hundreds of powers of two below 0 (q = c, k = -c in every element), so the
+    # running maximum starts far below the 0 it stands at before a column's first key, and later keys lie far above
+    # (k = +c from position 100 on): what is summed up to then has to vanish without a trace, not turn into 0 * inf.
+    nh, nkv, d, n = 4, 2, 128, 200
+    c = 4.0
+    q = torch.full((n, nh, d), c).to(torch.bfloat16)
+    k = torch.full((nkv, n, d), -c)
+    k[:, 100:] = c
+    k[:, 150] = -c
+    v = rand(nkv, n, d, seed=5).cpu().to(torch.bfloat16).float()
+    table = [0, 1, 2, 3]
+    kk, vv = paged(k, v, table, 4, torch.bfloat16)
+    keys, values = kk.to(DEV), vv.to(DEV)
+    pos = torch.arange(n)
+    tile_tok0 = list(range(0, n, tile))
+    out = torch.empty(n, nh * d, dtype=torch.bfloat16, device=DEV)
+    scale = 1 / math.sqrt(d)
+    K.attention_prefill(q.to(DEV), keys, values, pos.to(torch.int32).to(DEV), ints([table]), ints([0] * len(tile_tok0)), ints(tile_tok0),
+                        ints([min(tile, n - t) for t in tile_tok0]), ints([0]), ints([n]), 0, scale, out, tile_queries=tile)
+    want = attention_reference(q.float(), k, v, pos, 0, scale)
+    assert torch.isfinite(out.float()).all()
+    torch.testing.assert_close(out.float().cpu(), want, atol=2e-2, rtol=2e-2)
+    # (before position 100 a query's output is the mean of the values it sees, afterwards that of the keys from 100 on)
+    torch.testing.assert_close(want[50, :d], v[0, :51].mean(0), atol=1e-3, rtol=1e-3)
+
+
 @pytest.mark.parametrize("nh,nkv,d,spans,tile", [
     (28, 4, 128, [(0, 2048)], 16),                    # the benchmarked prompt: two heads a wave, all blocks resident
     (28, 4, 128, [(0, 2048)], 64),
