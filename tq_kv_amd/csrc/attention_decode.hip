@@ -69,7 +69,7 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     const int kvh = blockIdx.y / q_blocks, qb = blockIdx.y % q_blocks;
     const int seq = blockIdx.z;
     const int n_rep = n_heads / n_kv_heads;
-    const int pos = tok_pos[seq];
+    const int pos = __builtin_amdgcn_readfirstlane(tok_pos[seq]);
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
     // exponentials to base 2 (one instruction each): the scores carry log2(e), and so do the running
     // maxima m here, in part_ml and in the merge kernel
@@ -101,7 +101,7 @@ void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
         const int32_t* pages = page_table + (size_t)seq * table_width;
         const size_t page_stride = (size_t)n_kv_heads * TQK_PAGE * D;
         for (int pg = start_page; pg <= last_page; pg += W * n_parts) {
-            const int page = pages[pg];
+            const int page = __builtin_amdgcn_readfirstlane(pages[pg]);        // the same in all lanes: the page's address is then a scalar
             if (page < 0) continue;                     // the host never lets this happen
             const bf16_t* kp = keys + (size_t)page * page_stride + (size_t)kvh * TQK_PAGE * D;
             const bf16_t* vp = values + (size_t)page * page_stride + (size_t)kvh * TQK_PAGE * D;
