@@ -710,8 +710,7 @@ def test_attention_decode_refuses_other_head_sizes():
                            torch.empty(1, 48, dtype=torch.bfloat16, device=DEV))
 
 
-# (every head size both ways: blocks of four waves of columns, which run as two sets of waves that share each page's
-# keys between them, and blocks of more waves of columns, which do not; head size 32 the second way with 10 heads on 2)
+# (short sequences: one set of waves a block; head size 32 in blocks of more than four waves with 10 heads on 2)
 @pytest.mark.parametrize("nh,nkv,d", [(28, 4, 128), (6, 2, 64), (5, 5, 32), (10, 2, 32), (3, 1, 96), (40, 2, 64), (12, 2, 128)])
 @pytest.mark.parametrize("window", [0, 70, 12])
 @pytest.mark.parametrize("tile", [16, 32, 64, 128])
@@ -1057,6 +1056,8 @@ def test_attention_prefill_with_scores_far_below_zero(tile):
     (40, 2, 64, [(0, 1500), (300, 900)], 32),         # groups of 20 heads: three blocks a group
     (3, 1, 96, [(0, 2500)], 64),
     (5, 5, 32, [(0, 2100)], 128),
+    (6, 2, 64, [(0, 1500)], 16),                      # few blocks of four waves of columns and long sequences: two sets of
+    (3, 1, 96, [(0, 1200)], 32),                      # waves a block share each page's keys (as the first and the last line)
 ])
 @pytest.mark.parametrize("window", [0, 1000])
 def test_attention_prefill_over_thousands_of_keys(nh, nkv, d, spans, tile, window):

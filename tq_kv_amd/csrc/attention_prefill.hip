@@ -474,9 +474,10 @@ void attention_prefill_kernel(const PrefillArgs p) {
 }  // namespace
 
 // Up to this many blocks per compute unit a step runs with two sets of waves per block.  Measured with 7 heads a
-// group and head size 128, causal prompts alone: 1024 tokens (one block a unit) 30.8 -> 28.5 us, 2048 tokens (two)
-// 61.9 -> 60.9, 4096 tokens (four) 178 -> 191.
+// group and head size 128, causal prompts alone, one set against two: 1024 tokens (one block a unit) 29.7 -> 27.0 us,
+// 1536 tokens 43.4 -> 37.3, 2048 tokens (two blocks a unit) 56.4 -> 54.6, 4096 tokens (four) 178 -> 191.
 #define PF_SPLIT_BLOCKS_PER_CU 2
+#define PF_SPLIT_MIN_TOKENS 512         // new tokens a sequence, on average
 extern "C" int tqk_attention_prefill_supported(int head_dim) {
     return head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128;
 }
@@ -554,7 +555,10 @@ extern "C" int tqk_attention_prefill(const void* q, const void* keys, const void
     const int n_cus = prefill_compute_units();
     TQK_REQUIRE(n_cus > 0, "tqk_attention_prefill: cannot read the number of compute units");
     // two sets of waves per block where the columns leave room for them and the blocks are few (see the top)
-    const bool split = a.col_waves == PF_SPLIT_COL_WAVES && total <= (long long)PF_SPLIT_BLOCKS_PER_CU * n_cus;
+    // (and the sequences are long enough for the walk to outweigh the handing over at the end: 256 tokens 11.7 -> 12.8 us
+    // with two sets, 512 tokens 17.7 -> 17.4, 1536 tokens 43.4 -> 37.3)
+    const bool split = a.col_waves == PF_SPLIT_COL_WAVES && total <= (long long)PF_SPLIT_BLOCKS_PER_CU * n_cus &&
+                       n_tokens >= PF_SPLIT_MIN_TOKENS * n_seqs;
     const int waves = split ? 2 * a.col_waves : a.col_waves;
     // Blocks that are all resident at once (a compute unit holds 8 such waves) are not shared out
     // as they finish: then the runs of one block per compute unit alternate their direction.
