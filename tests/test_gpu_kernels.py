@@ -1059,7 +1059,7 @@ def test_attention_prefill_with_scores_far_below_zero(tile):
     (6, 2, 64, [(0, 1500)], 16),                      # few blocks of four waves of columns and long sequences: two sets of
     (3, 1, 96, [(0, 1200)], 32),                      # waves a block share each page's keys (as the first and the last line)
 ])
-@pytest.mark.parametrize("window", [0, 1000])
+@pytest.mark.parametrize("window", [0, 1000, 20])        # 20: most queries see keys of one half of a page only (one set of waves sees none)
 def test_attention_prefill_over_thousands_of_keys(nh, nkv, d, spans, tile, window):
     scale = 1 / math.sqrt(d)
     need = [(b + 63) // 64 for _, b in spans]
